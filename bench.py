@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the Swin3D-S stage-1 window-attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of the fused attention forward (s3d_attn_fwd) over the whole
+headline workload: the 10x8x3 m synthetic room cut to <= 200k voxels, C=48, 6 heads,
+window 5, quant 4, cRSE=XYZ_RGB_NORM, fp16 I/O with fp32 accumulation.  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line.
+
+The CPU oracle (oracle/) is used here only for the `cpu_baseline` leg.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
+
+
+def algorithmic_bytes(n, c, elem_bytes, nd, w, table_len):
+    """q,k,v in + out (4*C*s), n_coords fp32 (4*nd), n2n (4) per voxel; w_sizes + w2n per window;
+    the three tables once."""
+    return n * (4 * c * elem_bytes + 4 * nd + 4) + 8 * w + 3 * table_len * elem_bytes
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (windows are independent; see DESIGN.md for how "
+              "the path would shard); --gpus must be 1", file=sys.stderr)
+        return 2
+
+    import torch
+    import swin3d_amd
+    from swin3d_amd import _lib, build, crse, synth
+
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build(force=True)
+    lib = _lib.lib()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---- workload: BASELINE.json configs[1] -------------------------------------------------
+    heads, dim, ws, quant, cRSE = 6, 8, 5, 4, "XYZ_RGB_NORM"
+    channels = heads * dim
+    scene = synth.make_room((10.0, 8.0, 3.0), 30, 200_000, seed=0)
+    n = scene.coords.shape[0]
+    sizes = crse.crse_table_sizes(ws, quant, heads, dim, cRSE)
+    table_len = int(sum(sizes))
+    nd = len(sizes)
+    q, k, v, tables = synth.layer_inputs(n, channels, heads, table_len, seed=0, recipe="layer",
+                                         dtype=np.float16)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    coords_d = t(scene.coords)
+    # window index on the GPU (timed separately below)
+    index = swin3d_amd.build_window_index(coords_d, 1, ws, 0)
+    order = index.n2n.long()
+    n_xyz = index.local_xyz().float() + t(scene.frac)[order]
+    n_coords = torch.cat([n_xyz, t(synth.signals(scene, cRSE))[order]], 1)
+    n_crse = crse.scale_crse_coords(n_coords, quant, cRSE)
+    q_d, k_d, v_d = t(q), t(k), t(v)
+    tq_d, tk_d, tv_d = (t(x) for x in tables)
+    sizes_d = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q_d)
+    num_w, num_m = index.num_windows, index.num_pairs
+    stream = torch.cuda.current_stream(dev)
+
+    def step():
+        status = lib.s3d_attn_fwd(q_d.data_ptr(), k_d.data_ptr(), v_d.data_ptr(), tq_d.data_ptr(),
+                                  tk_d.data_ptr(), tv_d.data_ptr(), sizes_d.data_ptr(), nd, table_len,
+                                  index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
+                                  n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
+                                  _lib.S3D_DTYPE_F16, stream.cuda_stream)
+        if status != 0:
+            _lib.check(status, "s3d_attn_fwd")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # per-launch kernel time from events on the launch stream (torch's current stream)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record(stream)
+        step()
+        ends[i].record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / args.steps
+    launch_ms = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+    kernel_ms = float(launch_ms.mean())
+
+    bytes_alg = algorithmic_bytes(n, channels, 2, nd, num_w, table_len)
+    achieved = bytes_alg / (kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "window-attn fwd voxel-pairs/s",
+        "value": num_m / (wall_ms * 1e-3),
+        "unit": "voxel-pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "Swin3D-S stage-1 window attention fwd, synthetic 10x8x3 m room, fp16, "
+                        "C=48 H=6 D=8 window=5 quant=4 cRSE=XYZ_RGB_NORM (BASELINE configs[1])",
+            "voxels": n, "windows": num_w, "pairs": num_m,
+            "mean_window_voxels": n / max(num_w, 1), "max_window_voxels": index.max_window_voxels,
+        },
+        "voxels_per_s": n / (wall_ms * 1e-3),
+        "kernel_ms": {"mean": kernel_ms, "median": float(np.median(launch_ms)),
+                      "p10": float(np.percentile(launch_ms, 10)), "p90": float(np.percentile(launch_ms, 90))},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes": bytes_alg},
+    }
+
+    if not args.no_extras:
+        result["extras"] = extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev)
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m)
+
+    print(json.dumps(result))
+    return 0
+
+
+def _time_gpu(torch, fn, reps=20, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(reps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / reps
+
+
+def extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev):
+    """Side figures for the supporting kernels (same scene): window index and both KNN directions."""
+    n = scene.coords.shape[0]
+    out = {}
+    ms = _time_gpu(torch, lambda: swin3d_amd.build_window_index(coords_d, 1, ws, 0), reps=10)
+    out["window_index"] = {"ms": ms, "voxels_per_s": n / (ms * 1e-3),
+                           "algorithmic_bytes": 24 * n, "note": "includes one host sync per call"}
+    coarse, _ = synth.grid_downsample(scene, 2)
+    centres = np.ascontiguousarray((coarse.coords[:, 1:].astype(np.float32) + np.float32(1.0))[:50_000])
+    fine_d = torch.from_numpy(scene.xyz).to(dev)
+    cen_d = torch.from_numpy(centres).to(dev)
+    fo = torch.tensor([n], dtype=torch.int32, device=dev)
+    co = torch.tensor([centres.shape[0]], dtype=torch.int32, device=dev)
+    for name, (k, s, q, so, qo) in {"knn_down_k16": (16, fine_d, cen_d, fo, co),
+                                    "knn_up_k3": (3, cen_d, fine_d, co, fo)}.items():
+        ms = _time_gpu(torch, lambda: swin3d_amd.knn_query(k, s, q, so, qo), reps=10)
+        ns, nq = s.shape[0], q.shape[0]
+        alg = 12 * ns + 12 * nq + 8 * k * nq
+        out[name] = {"ms": ms, "queries_per_s": nq / (ms * 1e-3), "sources": ns, "queries": nq,
+                     "algorithmic_bytes": alg, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    return out
+
+
+def cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m):
+    """The reference math on the host cores: the C oracle's fp32 variant (a port, not the
+    reference binary) over the whole headline workload, all OpenMP threads."""
+    import oracle
+    threads = min(oracle.max_threads(), os.cpu_count() or 1)
+    f = lambda a: a.astype(np.float32)
+    args = (f(q), f(k), f(v), f(tables[0]), f(tables[1]), f(tables[2]), np.asarray(sizes, np.int32),
+            index.w_sizes.cpu().numpy(), index.w2n.cpu().numpy(), index.n2n.cpu().numpy(),
+            n_crse.cpu().numpy())
+    t0 = time.perf_counter()
+    oracle.attn_fwd(*args, acc="f32", num_threads=threads)
+    dt = time.perf_counter() - t0
+    return {"value": num_m / dt, "unit": "voxel-pairs/s", "cores": threads, "kind": "port",
+            "sample": f"whole headline workload once ({num_m} pairs), fp32 accumulate, "
+                      f"OpenMP over windows, {dt:.2f} s", "seconds": dt}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

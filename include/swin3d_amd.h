@@ -1,0 +1,149 @@
+/*
+ * swin3d_amd -- C ABI of the MI355X (gfx950) sparse window-attention forward,
+ * window index builder and KNN helper.
+ *
+ * Plain pointers and sizes only: every pointer named "device" is a HIP device
+ * address, `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * All entry points enqueue work on `stream` and return without synchronising
+ * unless stated otherwise.  The library keeps no device state; every output and
+ * every workspace is allocated by the caller.
+ *
+ * Return value: 0 on success, a negative S3D_ERR_* code for a rejected argument,
+ * a positive value = the hipError_t of a failed runtime call.  A human readable
+ * description of the last failure on the calling thread is returned by
+ * s3d_last_error_string().
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to
+ * the microsoft/Swin3D tree).
+ */
+#ifndef SWIN3D_AMD_H
+#define SWIN3D_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define S3D_OK 0
+#define S3D_ERR_NULL_POINTER (-1)
+#define S3D_ERR_BAD_SHAPE (-2)
+#define S3D_ERR_BAD_DTYPE (-3)
+#define S3D_ERR_UNSUPPORTED (-4)
+#define S3D_ERR_WORKSPACE (-5)
+
+/* element type of q/k/v, the tables and the attention output */
+#define S3D_DTYPE_F32 0
+#define S3D_DTYPE_F16 1
+
+/* largest K of s3d_knn (K_MAX of Swin3D/src/knn/knn_cuda_kernel.cu:4) */
+#define S3D_KNN_KMAX 64
+/* squared distance stored in unfilled KNN slots: float(0x7fffffff)
+ * (MAX_DIST of Swin3D/src/knn/knn_cuda_kernel.cu:5); their index is -1 */
+#define S3D_KNN_PAD_DIST2 2147483648.0f
+
+/* Library version, major*10000 + minor*100 + patch. */
+int s3d_version(void);
+
+/* Description of the last error raised on the calling thread ("" if none). */
+const char *s3d_last_error_string(void);
+
+/*
+ * Windowed self-attention forward with contextual relative signal encoding.
+ *
+ * Replaces the pair of pybind entry points
+ *   cal_max_coffs           Swin3D/src/attn/self_attn_aio_fwd.cu:255-455
+ *   self_attn_cuda_forward  Swin3D/src/attn/self_attn_aio_fwd.cu:457-688
+ * (declared in Swin3D/src/attn/self_attn_aio_fwd.h:11-26, exported at
+ * Swin3D/src/attn/attn_api.cpp:20,23) and the division
+ * Swin3D/sparse_dl/attn/attn_coff.py:184, for pos_mode SEPARATE (3) and
+ * indice_mode INDIRECT (2), in ONE pass and without the O(M) pair arrays
+ * m2w_indices / w2m_offsets.
+ *
+ *   q, k, v        device [N,H,D] of `dtype`, original voxel order (q pre-scaled)
+ *   table_q/k/v    device [table_len] of `dtype`, layout [axis][row][h][c]
+ *   table_sizes    device int32 [nd], table_sizes[n] = rows_n * H * D
+ *                  (the reference's `table_offsets` tensor, fwd.cu:258,285)
+ *   table_len      elements per table = sum_n table_sizes[n]
+ *   w_sizes, w2n   device int32 [W]: voxels per window, exclusive prefix sum
+ *   n2n            device int32 [N]: window-sorted position -> original row
+ *   n_coords       device fp32 [N,nd], window-sorted order, scaled by the quant sizes
+ *   out            device [N,H,D] of `dtype`: softmax-normalised attention output
+ *   out_max        device fp32 [N,H] or NULL: max logit per (voxel, head)
+ *                  (the tensor cal_max_coffs returns)
+ *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
+ *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
+ *   D in {8,16,32}, nd in {3,6,9}, H >= 1.
+ *
+ * Row index of axis n for the pair (query i, key j), all in fp32:
+ *   rel = (n_coords[i][n] - n_coords[j][n]) + float(rows_n / 2)
+ *   row = min(int(min(max(rel, 0), rows_n)), rows_n - 1)
+ * (Swin3D/src/attn/attn_utils.cuh:444-450; the reference indexes one row past
+ * the axis table when the clamped value equals rows_n, this library folds that
+ * case onto the last row).
+ */
+int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_q,
+                 const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
+                 int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
+                 const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
+                 int32_t H, int32_t D, int64_t W, int32_t dtype, void *stream);
+
+/*
+ * Window sort + segment offsets.
+ *
+ * Replaces BasicLayer.get_map_pair / get_window_mapping
+ * (Swin3D/modules/swin3d_layers.py:713-787, MinkowskiEngine pooling + kernel_map +
+ * torch.sort) and the w2n / w_sizes part of sparse_self_attention (:96-103).
+ *
+ *   coords     device int32 [N,4] rows (batch, x, y, z); x,y,z multiples of `stride`
+ *   stride     tensor stride of the voxel grid (>= 1)
+ *   window     window size in voxels per side (1..10)
+ *   shift      window shift in voxels (0 or window/2; get_shifted_sp, :824-838)
+ *   n2n        device int32 [N]  out: window-sorted position -> original row
+ *   w_w_id     device int32 [N]  out: local id lx*window^2 + ly*window + lz per sorted position
+ *   w_sizes    device int32 [N]  out: first W entries = voxels per window
+ *   w2n        device int32 [N]  out: first W entries = exclusive prefix sum of w_sizes
+ *   counts     device int64 [4]  out: {W, M = sum w_sizes^2, max w_size, error flag}
+ *                                 error flag != 0: a coordinate was outside the supported
+ *                                 range (batch 0..4095, window coordinates -8192..8191)
+ *   workspace  device scratch of at least s3d_window_index_workspace_bytes(N) bytes
+ *
+ * Window order: ascending (batch, wx, wy, wz) with floor division of the shifted
+ * coordinate by window*stride; inside a window ascending local id; equal keys by
+ * ascending original row.
+ */
+size_t s3d_window_index_workspace_bytes(int64_t N);
+int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t window,
+                     int32_t shift, int32_t *n2n, int32_t *w_w_id, int32_t *w_sizes, int32_t *w2n,
+                     int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * K nearest sources of every query inside the same batch segment.
+ *
+ * Replaces knn_cuda (Swin3D/src/knn/knn_cuda_kernel.cu:207-244, declared in
+ * Swin3D/src/knn/knn_cuda_kernel.h:5-12, exported at Swin3D/src/knn/knn_api.cpp:5).
+ *
+ *   src_xyz      device fp32 [Ns,3]      query_xyz  device fp32 [Nq,3]
+ *   src_offset   device int32 [B] cumulative END offsets of the batch segments of src
+ *   query_offset device int32 [B] same for the queries
+ *   ret_idx      device int32 [Nq,K] out: global source rows
+ *   ret_dist2    device fp32 [Nq,K] out: SQUARED distances ((dx*dx + dy*dy) + dz*dz with
+ *                every operation rounded to fp32, d = src - query)
+ *   cell_size    edge of the bucketing grid in the units of xyz; <= 0 picks it from the data
+ *   workspace    device scratch of at least s3d_knn_workspace_bytes(Ns, Nq, B) bytes
+ *
+ * Result per query: the K smallest sources under the order (distance, source row),
+ * emitted in that order (ties go to the lower row).  Segments with fewer than K
+ * sources are padded with row -1 and S3D_KNN_PAD_DIST2.  1 <= K <= S3D_KNN_KMAX.
+ */
+size_t s3d_knn_workspace_bytes(int64_t Ns, int64_t Nq, int32_t B);
+int s3d_knn(int32_t K, const float *src_xyz, int64_t Ns, const float *query_xyz, int64_t Nq,
+            const int32_t *src_offset, const int32_t *query_offset, int32_t B, int32_t *ret_idx,
+            float *ret_dist2, float cell_size, void *workspace, size_t workspace_bytes,
+            void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SWIN3D_AMD_H */

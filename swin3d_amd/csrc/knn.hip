@@ -1,0 +1,467 @@
+// Grid-bucketed exact K nearest neighbours inside batch segments (gfx950).
+//
+// Replaces the brute-force kernel of Swin3D/src/knn/knn_cuda_kernel.cu:139-204
+// (one thread streaming every source of the batch through a 64-slot heap).
+// Sources are bucketed into a uniform grid (one counting sort), every query
+// thread walks cubic shells of cells around its own cell and keeps the K best
+// candidates in registers, ordered by (squared distance, source row).  A shell
+// walk stops once the K-th best distance is provably smaller than the distance
+// to anything outside the visited cube, so the result is exact and independent
+// of the visiting order: ties go to the lower source row.
+//
+// Distance arithmetic: d = src - query per axis, ((dx*dx) + (dy*dy)) + (dz*dz),
+// every operation individually rounded to fp32 (no fused multiply-add).
+#include "s3d_common.h"
+
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+namespace s3d {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxBatch = 4096;
+
+struct KnnPlan {
+    // bounding box of all sources as order-preserving integer images of the floats
+    int lo[3], hi[3];
+    float origin[3];
+    float cell, inv_cell, slack;
+    int dim[3];
+    int cells_per_batch;
+    int src_end;  // sources at or beyond this row belong to no batch segment
+};
+
+struct Layout {
+    size_t plan, counts, starts, src_cell, sorted, temp, temp_bytes, total;
+    int64_t cells_cap;
+};
+
+int64_t cells_cap_for(int64_t Ns)
+{
+    int64_t cap = 4 * Ns;
+    if (cap < 4096) cap = 4096;
+    if (cap > (1LL << 24)) cap = 1LL << 24;
+    return cap;
+}
+
+size_t scan_temp_bytes(int64_t n)
+{
+    size_t bytes = 0;
+    int32_t *p = nullptr;
+    (void)rocprim::exclusive_scan(nullptr, bytes, p, p, 0, static_cast<size_t>(n),
+                                  rocprim::plus<int32_t>(), hipStream_t(0));
+    return bytes;
+}
+
+Layout make_layout(int64_t Ns)
+{
+    Layout L{};
+    L.cells_cap = cells_cap_for(Ns);
+    const size_t ns = static_cast<size_t>(Ns > 0 ? Ns : 1);
+    const size_t cells = static_cast<size_t>(L.cells_cap) + 1;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 256);
+        return at;
+    };
+    L.plan = take(sizeof(KnnPlan));
+    L.counts = take(cells * sizeof(int32_t));
+    L.starts = take(cells * sizeof(int32_t));
+    L.src_cell = take(ns * sizeof(int32_t));
+    L.sorted = take(ns * sizeof(float4));
+    L.temp_bytes = scan_temp_bytes(static_cast<int64_t>(cells));
+    L.temp = take(L.temp_bytes);
+    L.total = off;
+    return L;
+}
+
+// order-preserving map float -> int (so integer atomicMin/Max work on floats)
+__device__ __forceinline__ int float_to_ordered(float f)
+{
+    const int i = __float_as_int(f);
+    return i >= 0 ? i : i ^ 0x7fffffff;
+}
+__device__ __forceinline__ float ordered_to_float(int i)
+{
+    return __int_as_float(i >= 0 ? i : i ^ 0x7fffffff);
+}
+
+__global__ __launch_bounds__(kThreads) void knn_init_kernel(KnnPlan *plan, int32_t *counts,
+                                                            int64_t cells)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i < cells) counts[i] = 0;
+    if (i < 3) {
+        plan->lo[i] = 0x7fffffff;
+        plan->hi[i] = static_cast<int>(0x80000000u);
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restrict__ src,
+                                                            int64_t Ns, KnnPlan *plan)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    int lo[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
+    int hi[3] = {static_cast<int>(0x80000000u), static_cast<int>(0x80000000u),
+                 static_cast<int>(0x80000000u)};
+    if (i < Ns) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) lo[a] = hi[a] = float_to_ordered(src[i * 3 + a]);
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        for (int off = 32; off > 0; off >>= 1) {
+            lo[a] = min(lo[a], __shfl_down(lo[a], off));
+            hi[a] = max(hi[a], __shfl_down(hi[a], off));
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            atomicMin(&plan->lo[a], lo[a]);
+            atomicMax(&plan->hi[a], hi[a]);
+        }
+    }
+}
+
+// One thread: turn the bounding box into grid parameters that fit `cells_cap`.
+__global__ void knn_plan_kernel(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B,
+                                int64_t Ns, float cell_hint, int64_t cells_cap)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int src_end = src_offset[B - 1];
+    if (src_end > Ns) src_end = static_cast<int>(Ns);
+    if (src_end < 0) src_end = 0;
+    plan->src_end = src_end;
+    if (src_end == 0) {  // no candidate anywhere: the query kernel pads every slot
+        for (int a = 0; a < 3; ++a) {
+            plan->origin[a] = 0.0f;
+            plan->dim[a] = 1;
+        }
+        plan->cell = plan->inv_cell = 1.0f;
+        plan->slack = 0.0f;
+        plan->cells_per_batch = 1;
+        return;
+    }
+    float ext[3], max_abs = 0.0f;
+    for (int a = 0; a < 3; ++a) {
+        const float lo = ordered_to_float(plan->lo[a]);
+        const float hi = ordered_to_float(plan->hi[a]);
+        plan->origin[a] = lo;
+        ext[a] = fmaxf(hi - lo, 0.0f);
+        max_abs = fmaxf(max_abs, fmaxf(fabsf(lo), fabsf(hi)));
+    }
+    float cell = cell_hint;
+    if (!(cell > 0.0f)) {
+        // no hint: aim at about one source per cell if the sources filled the box
+        const float floor_ext = fmaxf(fmaxf(ext[0], ext[1]), ext[2]) * 1e-3f + 1e-12f;
+        const float vol = fmaxf(ext[0], floor_ext) * fmaxf(ext[1], floor_ext) * fmaxf(ext[2], floor_ext);
+        cell = cbrtf(vol / static_cast<float>(src_end > 0 ? src_end : 1));
+    }
+    if (!(cell > 1e-20f)) cell = 1.0f;
+    const int64_t per_batch_cap = cells_cap / B;  // B <= kMaxBatch <= cells_cap
+    int dim[3];
+    for (int iter = 0; iter < 200; ++iter) {
+        double total = 1.0;
+        for (int a = 0; a < 3; ++a) {
+            const float cells_f = floorf(ext[a] / cell) + 1.0f;
+            dim[a] = cells_f < 2.0e9f ? static_cast<int>(cells_f) : 2000000000;
+            total *= static_cast<double>(dim[a]);
+        }
+        if (total <= static_cast<double>(per_batch_cap)) break;
+        cell *= 1.25f;
+    }
+    {
+        double total = static_cast<double>(dim[0]) * dim[1] * dim[2];
+        if (total > static_cast<double>(per_batch_cap)) {  // degenerate input: single cell
+            dim[0] = dim[1] = dim[2] = 1;
+            cell = fmaxf(fmaxf(ext[0], ext[1]), ext[2]) * 2.0f + 1.0f;
+        }
+    }
+    plan->cell = cell;
+    plan->inv_cell = 1.0f / cell;
+    // sources within `slack` of a cell face may sit in either neighbour cell
+    plan->slack = 1e-3f * cell + 8e-6f * max_abs;
+    for (int a = 0; a < 3; ++a) plan->dim[a] = dim[a];
+    plan->cells_per_batch = dim[0] * dim[1] * dim[2];
+}
+
+__device__ __forceinline__ int cell_coord(float p, float origin, float inv_cell)
+{
+    const float t = floorf((p - origin) * inv_cell);
+    // keep the conversion defined for far-away queries
+    return static_cast<int>(fminf(fmaxf(t, -1.0e9f), 1.0e9f));
+}
+
+__device__ __forceinline__ int find_batch(const int32_t *__restrict__ offset, int B, int64_t g)
+{
+    int b = 0;
+    for (; b < B; ++b)
+        if (g < offset[b]) break;
+    return b;  // == B: beyond the last segment
+}
+
+__global__ __launch_bounds__(kThreads) void knn_count_kernel(
+    const float *__restrict__ src, int64_t Ns, const int32_t *__restrict__ src_offset, int B,
+    const KnnPlan *__restrict__ plan, int32_t *__restrict__ counts, int32_t *__restrict__ src_cell)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= Ns) return;
+    const int b = find_batch(src_offset, B, i);
+    if (b >= B) {
+        src_cell[i] = -1;
+        return;
+    }
+    int c[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        c[a] = cell_coord(src[i * 3 + a], plan->origin[a], plan->inv_cell);
+        c[a] = min(max(c[a], 0), plan->dim[a] - 1);
+    }
+    const int cell = b * plan->cells_per_batch + (c[2] * plan->dim[1] + c[1]) * plan->dim[0] + c[0];
+    src_cell[i] = cell;
+    atomicAdd(&counts[cell], 1);
+}
+
+__global__ __launch_bounds__(kThreads) void knn_scatter_kernel(
+    const float *__restrict__ src, int64_t Ns, const int32_t *__restrict__ src_cell,
+    const int32_t *__restrict__ starts, int32_t *__restrict__ counts, float4 *__restrict__ sorted)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= Ns) return;
+    const int cell = src_cell[i];
+    if (cell < 0) return;
+    const int slot = atomicSub(&counts[cell], 1) - 1;
+    const int pos = starts[cell] + slot;
+    sorted[pos] = make_float4(src[i * 3], src[i * 3 + 1], src[i * 3 + 2],
+                              __int_as_float(static_cast<int>(i)));
+}
+
+__device__ __forceinline__ bool cand_less(float d, int i, float d2, int i2)
+{
+    return d < d2 || (d == d2 && i < i2);
+}
+
+template <int K>
+struct TopKRegs {
+    float d[K];
+    int id[K];
+    __device__ __forceinline__ void init(int)
+    {
+#pragma unroll
+        for (int t = 0; t < K; ++t) {
+            d[t] = INFINITY;
+            id[t] = 0x7fffffff;
+        }
+    }
+    __device__ __forceinline__ float worst_d(int) const { return d[K - 1]; }
+    __device__ __forceinline__ int worst_i(int) const { return id[K - 1]; }
+    __device__ __forceinline__ void insert(float cd, int ci, int)
+    {
+#pragma unroll
+        for (int t = K - 1; t > 0; --t) {
+            const bool before_prev = cand_less(cd, ci, d[t - 1], id[t - 1]);
+            const bool before_this = cand_less(cd, ci, d[t], id[t]);
+            const float nd = before_prev ? d[t - 1] : (before_this ? cd : d[t]);
+            const int ni = before_prev ? id[t - 1] : (before_this ? ci : id[t]);
+            d[t] = nd;
+            id[t] = ni;
+        }
+        if (cand_less(cd, ci, d[0], id[0])) {
+            d[0] = cd;
+            id[0] = ci;
+        }
+    }
+    __device__ __forceinline__ float get_d(int t) const { return d[t]; }
+    __device__ __forceinline__ int get_i(int t) const { return id[t]; }
+};
+
+// Any K up to S3D_KNN_KMAX: same ordered list, indexed at run time (lives in scratch memory).
+struct TopKAny {
+    float d[S3D_KNN_KMAX];
+    int id[S3D_KNN_KMAX];
+    __device__ __forceinline__ void init(int K)
+    {
+        for (int t = 0; t < K; ++t) {
+            d[t] = INFINITY;
+            id[t] = 0x7fffffff;
+        }
+    }
+    __device__ __forceinline__ float worst_d(int K) const { return d[K - 1]; }
+    __device__ __forceinline__ int worst_i(int K) const { return id[K - 1]; }
+    __device__ __forceinline__ void insert(float cd, int ci, int K)
+    {
+        int t = K - 1;
+        while (t > 0 && cand_less(cd, ci, d[t - 1], id[t - 1])) {
+            d[t] = d[t - 1];
+            id[t] = id[t - 1];
+            --t;
+        }
+        d[t] = cd;
+        id[t] = ci;
+    }
+    __device__ __forceinline__ float get_d(int t) const { return d[t]; }
+    __device__ __forceinline__ int get_i(int t) const { return id[t]; }
+};
+
+template <typename TopK>
+__global__ __launch_bounds__(kThreads) void knn_query_kernel(
+    int K, const float *__restrict__ qry, int64_t Nq, const int32_t *__restrict__ query_offset,
+    int B, const KnnPlan *__restrict__ plan_ptr, const int32_t *__restrict__ starts,
+    const float4 *__restrict__ sorted, int32_t *__restrict__ ret_idx, float *__restrict__ ret_dist2)
+{
+    const int64_t g = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (g >= Nq) return;
+    const KnnPlan plan = *plan_ptr;
+    TopK best;
+    best.init(K);
+    const int b = find_batch(query_offset, B, g);
+    if (b < B && plan.src_end > 0) {
+        const float qx = qry[g * 3], qy = qry[g * 3 + 1], qz = qry[g * 3 + 2];
+        const float qp[3] = {qx, qy, qz};
+        int qc[3], r_first = 0, r_last = 0;
+#pragma unroll
+        for (int a = 0; a < 3; ++a) {
+            qc[a] = cell_coord(qp[a], plan.origin[a], plan.inv_cell);
+            const int below = -qc[a], above = qc[a] - (plan.dim[a] - 1);
+            r_first = max(r_first, max(below, above));          // first shell touching the grid
+            r_last = max(r_last, max(qc[a], -above));           // shell that covers the whole grid
+        }
+        r_last = max(r_last, r_first);
+        const int32_t *cell_base = starts + static_cast<int64_t>(b) * plan.cells_per_batch;
+        for (int r = r_first; r <= r_last; ++r) {
+            const int z0 = max(qc[2] - r, 0), z1 = min(qc[2] + r, plan.dim[2] - 1);
+            const int y0 = max(qc[1] - r, 0), y1 = min(qc[1] + r, plan.dim[1] - 1);
+            for (int z = z0; z <= z1; ++z) {
+                const bool z_face = (z == qc[2] - r) || (z == qc[2] + r);
+                for (int y = y0; y <= y1; ++y) {
+                    const bool face = z_face || (y == qc[1] - r) || (y == qc[1] + r);
+                    const int32_t *row = cell_base + (z * plan.dim[1] + y) * plan.dim[0];
+                    // a face row spans the whole x range of the cube, an interior row only its two ends
+                    const int n_runs = (face || r == 0) ? 1 : 2;
+                    for (int run = 0; run < n_runs; ++run) {
+                        int x0, x1;
+                        if (face || r == 0) {
+                            x0 = qc[0] - r;
+                            x1 = qc[0] + r;
+                        } else {
+                            x0 = x1 = (run == 0) ? qc[0] - r : qc[0] + r;
+                        }
+                        x0 = max(x0, 0);
+                        x1 = min(x1, plan.dim[0] - 1);
+                        if (x0 > x1) continue;
+                        const int s_begin = row[x0], s_end = row[x1 + 1];
+                        for (int s = s_begin; s < s_end; ++s) {
+                            const float4 p = sorted[s];
+                            const float dx = __fsub_rn(p.x, qx), dy = __fsub_rn(p.y, qy),
+                                        dz = __fsub_rn(p.z, qz);
+                            const float d2 = __fadd_rn(
+                                __fadd_rn(__fmul_rn(dx, dx), __fmul_rn(dy, dy)), __fmul_rn(dz, dz));
+                            const int si = __float_as_int(p.w);
+                            if (cand_less(d2, si, best.worst_d(K), best.worst_i(K)))
+                                best.insert(d2, si, K);
+                        }
+                    }
+                }
+            }
+            if (best.worst_i(K) != 0x7fffffff) {
+                // everything outside the visited cube is at least `bound` away from the query
+                float bound = INFINITY;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) {
+                    const float lo_face = plan.origin[a] + static_cast<float>(qc[a] - r) * plan.cell;
+                    const float hi_face = plan.origin[a] + static_cast<float>(qc[a] + r + 1) * plan.cell;
+                    bound = fminf(bound, fminf(qp[a] - lo_face, hi_face - qp[a]));
+                }
+                bound -= plan.slack;
+                if (bound > 0.0f && best.worst_d(K) < bound * bound) break;
+            }
+        }
+    }
+    for (int t = 0; t < K; ++t) {
+        const int si = best.get_i(t);
+        const bool filled = si != 0x7fffffff;
+        ret_idx[g * K + t] = filled ? si : -1;
+        ret_dist2[g * K + t] = filled ? best.get_d(t) : S3D_KNN_PAD_DIST2;
+    }
+}
+
+}  // namespace
+}  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) size_t s3d_knn_workspace_bytes(int64_t Ns, int64_t Nq, int32_t B)
+{
+    (void)Nq;
+    (void)B;
+    return s3d::make_layout(Ns).total;
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const float *src_xyz, int64_t Ns, const float *query_xyz,
+                       int64_t Nq, const int32_t *src_offset, const int32_t *query_offset, int32_t B,
+                       int32_t *ret_idx, float *ret_dist2, float cell_size, void *workspace,
+                       size_t workspace_bytes, void *stream)
+{
+    using namespace s3d;
+    if (K < 1 || K > S3D_KNN_KMAX)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_knn: K=%d outside 1..%d", K, S3D_KNN_KMAX);
+    if (Ns < 0 || Nq < 0 || Ns > 0x7fffffffLL || Nq * K > 0x7fffffffffLL || B < 1 || B > kMaxBatch)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_knn: Ns=%lld Nq=%lld B=%d out of range", (long long)Ns,
+                    (long long)Nq, B);
+    if (Nq == 0) return S3D_OK;
+    if (!query_xyz || !src_offset || !query_offset || !ret_idx || !ret_dist2 || !workspace ||
+        (Ns > 0 && !src_xyz))
+        return fail(S3D_ERR_NULL_POINTER, "s3d_knn: null device pointer");
+    const Layout L = make_layout(Ns);
+    if (workspace_bytes < L.total)
+        return fail(S3D_ERR_WORKSPACE, "s3d_knn: workspace %zu B < required %zu B", workspace_bytes,
+                    L.total);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    char *base = static_cast<char *>(workspace);
+    KnnPlan *plan = reinterpret_cast<KnnPlan *>(base + L.plan);
+    int32_t *counts = reinterpret_cast<int32_t *>(base + L.counts);
+    int32_t *starts = reinterpret_cast<int32_t *>(base + L.starts);
+    int32_t *src_cell = reinterpret_cast<int32_t *>(base + L.src_cell);
+    float4 *sorted = reinterpret_cast<float4 *>(base + L.sorted);
+    void *temp = base + L.temp;
+    size_t temp_bytes = L.temp_bytes;
+    const int64_t cells = L.cells_cap + 1;
+
+    hipLaunchKernelGGL(knn_init_kernel, dim3(static_cast<unsigned>(ceil_div(cells, kThreads))),
+                       dim3(kThreads), 0, s, plan, counts, cells);
+    S3D_HIP_CHECK(hipGetLastError());
+    if (Ns > 0) {
+        const dim3 sgrid(static_cast<unsigned>(ceil_div(Ns, kThreads)));
+        hipLaunchKernelGGL(knn_bbox_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, plan);
+        S3D_HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,
+                           cell_size, L.cells_cap);
+        S3D_HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(knn_count_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_offset, B,
+                           plan, counts, src_cell);
+        S3D_HIP_CHECK(hipGetLastError());
+        S3D_HIP_CHECK(rocprim::exclusive_scan(temp, temp_bytes, counts, starts, 0,
+                                              static_cast<size_t>(cells), rocprim::plus<int32_t>(), s));
+        hipLaunchKernelGGL(knn_scatter_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_cell,
+                           starts, counts, sorted);
+        S3D_HIP_CHECK(hipGetLastError());
+    } else {
+        hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,
+                           cell_size, L.cells_cap);
+        S3D_HIP_CHECK(hipGetLastError());
+    }
+    const dim3 qgrid(static_cast<unsigned>(ceil_div(Nq, kThreads)));
+    if (K == 3)
+        hipLaunchKernelGGL(knn_query_kernel<TopKRegs<3>>, qgrid, dim3(kThreads), 0, s, K, query_xyz,
+                           Nq, query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
+    else if (K == 16)
+        hipLaunchKernelGGL(knn_query_kernel<TopKRegs<16>>, qgrid, dim3(kThreads), 0, s, K, query_xyz,
+                           Nq, query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
+    else
+        hipLaunchKernelGGL(knn_query_kernel<TopKAny>, qgrid, dim3(kThreads), 0, s, K, query_xyz, Nq,
+                           query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}

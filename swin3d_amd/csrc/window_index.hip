@@ -1,0 +1,218 @@
+// Window sort + segment offsets for sparse-voxel window attention (gfx950).
+//
+// Replaces the MinkowskiEngine pooling / kernel_map / torch.sort pipeline of
+// Swin3D/modules/swin3d_layers.py:713-787 and the w2n / w_sizes scans of
+// :96-103.  Every voxel gets one 64-bit key
+//     [ batch:12 | wx+8192:14 | wy+8192:14 | wz+8192:14 | local id:10 ]
+// with w = floor((coord + shift*stride) / (window*stride)) and
+// local id = (lx*window + ly)*window + lz; a stable radix sort of (key, row)
+// yields the window-sorted order, a flag + scan pass yields the segments.
+// Integer work only; HBM traffic is a handful of passes over 12 B per voxel.
+#include "s3d_common.h"
+
+#include <cstring>
+
+#include <rocprim/rocprim.hpp>
+
+namespace s3d {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kLocalBits = 10;
+constexpr int kAxisBits = 14;
+constexpr int kAxisBias = 1 << (kAxisBits - 1);  // 8192
+constexpr int kBatchBits = 12;
+
+struct Layout {
+    size_t keys_in, keys_out, vals_in, flags, ranks, temp, temp_bytes, total;
+};
+
+size_t sort_temp_bytes(int64_t N)
+{
+    size_t bytes = 0;
+    uint64_t *kn = nullptr;
+    int32_t *vn = nullptr;
+    (void)rocprim::radix_sort_pairs(nullptr, bytes, kn, kn, vn, vn, static_cast<size_t>(N), 0, 64,
+                                    hipStream_t(0));
+    return bytes;
+}
+
+size_t scan_temp_bytes(int64_t N)
+{
+    size_t bytes = 0;
+    int32_t *p = nullptr;
+    (void)rocprim::inclusive_scan(nullptr, bytes, p, p, static_cast<size_t>(N),
+                                  rocprim::plus<int32_t>(), hipStream_t(0));
+    return bytes;
+}
+
+Layout make_layout(int64_t N)
+{
+    Layout L{};
+    const size_t n = static_cast<size_t>(N > 0 ? N : 1);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 256);
+        return at;
+    };
+    L.keys_in = take(n * sizeof(uint64_t));
+    L.keys_out = take(n * sizeof(uint64_t));
+    L.vals_in = take(n * sizeof(int32_t));
+    L.flags = take(n * sizeof(int32_t));
+    L.ranks = take(n * sizeof(int32_t));
+    const size_t a = sort_temp_bytes(static_cast<int64_t>(n));
+    const size_t b = scan_temp_bytes(static_cast<int64_t>(n));
+    L.temp_bytes = a > b ? a : b;
+    L.temp = take(L.temp_bytes);
+    L.total = off;
+    return L;
+}
+
+__device__ __forceinline__ int floordiv(int a, int b)
+{
+    int q = a / b;
+    if ((a % b != 0) && ((a < 0) != (b < 0))) --q;
+    return q;
+}
+
+__global__ void init_counts_kernel(int64_t *counts)
+{
+    if (threadIdx.x < 4) counts[threadIdx.x] = 0;
+}
+
+__global__ __launch_bounds__(kThreads) void build_keys_kernel(
+    const int32_t *__restrict__ coords, int64_t N, int stride, int window, int shift,
+    uint64_t *__restrict__ keys, int32_t *__restrict__ vals, int64_t *__restrict__ counts)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= N) return;
+    const int4 c = reinterpret_cast<const int4 *>(coords)[i];
+    const int span = window * stride;
+    const int cc[3] = {c.y + shift * stride, c.z + shift * stride, c.w + shift * stride};
+    int wv[3], lv[3];
+    bool bad = c.x < 0 || c.x >= (1 << kBatchBits);
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        wv[a] = floordiv(cc[a], span);
+        lv[a] = (cc[a] - wv[a] * span) / stride;  // numerator in [0, span)
+        bad = bad || wv[a] < -kAxisBias || wv[a] >= kAxisBias;
+        wv[a] = min(max(wv[a], -kAxisBias), kAxisBias - 1);
+    }
+    if (bad) atomicMax(reinterpret_cast<unsigned long long *>(counts + 3), 1ULL);
+    const uint64_t b = static_cast<uint64_t>(min(max(c.x, 0), (1 << kBatchBits) - 1));
+    const uint64_t local = static_cast<uint64_t>((lv[0] * window + lv[1]) * window + lv[2]);
+    uint64_t key = b;
+    key = (key << kAxisBits) | static_cast<uint64_t>(wv[0] + kAxisBias);
+    key = (key << kAxisBits) | static_cast<uint64_t>(wv[1] + kAxisBias);
+    key = (key << kAxisBits) | static_cast<uint64_t>(wv[2] + kAxisBias);
+    key = (key << kLocalBits) | local;
+    keys[i] = key;
+    vals[i] = static_cast<int32_t>(i);
+}
+
+__global__ __launch_bounds__(kThreads) void flag_kernel(const uint64_t *__restrict__ keys, int64_t N,
+                                                        int32_t *__restrict__ flags,
+                                                        int32_t *__restrict__ w_w_id)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= N) return;
+    const uint64_t key = keys[i];
+    const bool first = (i == 0) || ((keys[i - 1] >> kLocalBits) != (key >> kLocalBits));
+    flags[i] = first ? 1 : 0;
+    w_w_id[i] = static_cast<int32_t>(key & ((1u << kLocalBits) - 1));
+}
+
+__global__ __launch_bounds__(kThreads) void segment_start_kernel(
+    const int32_t *__restrict__ flags, const int32_t *__restrict__ ranks, int64_t N,
+    int32_t *__restrict__ w2n, int64_t *__restrict__ counts)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i >= N) return;
+    if (flags[i]) w2n[ranks[i] - 1] = static_cast<int32_t>(i);
+    if (i == N - 1) counts[0] = ranks[i];
+}
+
+__global__ __launch_bounds__(kThreads) void segment_size_kernel(const int32_t *__restrict__ w2n,
+                                                                int64_t N,
+                                                                int32_t *__restrict__ w_sizes,
+                                                                int64_t *__restrict__ counts)
+{
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int64_t W = counts[0];  // written by the previous kernel on the same stream
+    long long size = 0;
+    if (w < W) {
+        const int32_t begin = w2n[w];
+        const int32_t end = (w + 1 < W) ? w2n[w + 1] : static_cast<int32_t>(N);
+        size = end - begin;
+        w_sizes[w] = static_cast<int32_t>(size);
+    }
+    long long sq = size * size, mx = size;
+    for (int off = 32; off > 0; off >>= 1) {
+        sq += __shfl_down(sq, off);
+        mx = max(mx, __shfl_down(mx, off));
+    }
+    if ((threadIdx.x & 63) == 0 && mx > 0) {
+        atomicAdd(reinterpret_cast<unsigned long long *>(counts + 1), static_cast<unsigned long long>(sq));
+        atomicMax(reinterpret_cast<unsigned long long *>(counts + 2), static_cast<unsigned long long>(mx));
+    }
+}
+
+}  // namespace
+}  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) size_t s3d_window_index_workspace_bytes(int64_t N)
+{
+    return s3d::make_layout(N).total;
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t window,
+                                int32_t shift, int32_t *n2n, int32_t *w_w_id, int32_t *w_sizes,
+                                int32_t *w2n, int64_t *counts, void *workspace,
+                                size_t workspace_bytes, void *stream)
+{
+    using namespace s3d;
+    if (N < 0 || N > 0x7fffffffLL)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index: N=%lld out of range", (long long)N);
+    if (stride < 1 || window < 1 || window > 10 || shift < 0 || shift >= window)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index: stride=%d window=%d shift=%d (need stride>=1, "
+                    "1<=window<=10, 0<=shift<window)", stride, window, shift);
+    if (!counts) return fail(S3D_ERR_NULL_POINTER, "s3d_window_index: counts is null");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(init_counts_kernel, dim3(1), dim3(64), 0, s, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    if (N == 0) return S3D_OK;
+    if (!coords || !n2n || !w_w_id || !w_sizes || !w2n || !workspace)
+        return fail(S3D_ERR_NULL_POINTER, "s3d_window_index: null device pointer");
+    if (reinterpret_cast<uintptr_t>(coords) % 16 != 0)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index: coords must be 16-byte aligned");
+    const Layout L = make_layout(N);
+    if (workspace_bytes < L.total)
+        return fail(S3D_ERR_WORKSPACE, "s3d_window_index: workspace %zu B < required %zu B",
+                    workspace_bytes, L.total);
+    char *base = static_cast<char *>(workspace);
+    uint64_t *keys_in = reinterpret_cast<uint64_t *>(base + L.keys_in);
+    uint64_t *keys_out = reinterpret_cast<uint64_t *>(base + L.keys_out);
+    int32_t *vals_in = reinterpret_cast<int32_t *>(base + L.vals_in);
+    int32_t *flags = reinterpret_cast<int32_t *>(base + L.flags);
+    int32_t *ranks = reinterpret_cast<int32_t *>(base + L.ranks);
+    void *temp = base + L.temp;
+    size_t temp_bytes = L.temp_bytes;
+
+    const dim3 grid(static_cast<unsigned>(ceil_div(N, kThreads)));
+    hipLaunchKernelGGL(build_keys_kernel, grid, dim3(kThreads), 0, s, coords, N, stride, window,
+                       shift, keys_in, vals_in, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    S3D_HIP_CHECK(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_out, vals_in, n2n,
+                                            static_cast<size_t>(N), 0, 64, s));
+    hipLaunchKernelGGL(flag_kernel, grid, dim3(kThreads), 0, s, keys_out, N, flags, w_w_id);
+    S3D_HIP_CHECK(hipGetLastError());
+    temp_bytes = L.temp_bytes;
+    S3D_HIP_CHECK(rocprim::inclusive_scan(temp, temp_bytes, flags, ranks, static_cast<size_t>(N),
+                                          rocprim::plus<int32_t>(), s));
+    hipLaunchKernelGGL(segment_start_kernel, grid, dim3(kThreads), 0, s, flags, ranks, N, w2n, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(segment_size_kernel, grid, dim3(kThreads), 0, s, w2n, N, w_sizes, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}

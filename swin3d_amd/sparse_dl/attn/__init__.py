@@ -1,0 +1,2 @@
+from .attn_coff import (IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims,
+                        window_attention_forward)

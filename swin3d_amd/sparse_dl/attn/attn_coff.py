@@ -1,0 +1,167 @@
+"""All-in-one sparse window self-attention operator on the swin3d_amd HIP library.
+
+Same Python surface as Swin3D/sparse_dl/attn/attn_coff.py (SelfAttnAIOFunction
+:155-232 and the enums :20-40), so WindowAttention (Swin3D/modules/swin3d_layers.py:554-567)
+can call it unchanged.  Differences in mechanism, not in result:
+  * one fused HIP pass (s3d_attn_fwd) instead of cal_max_coffs + self_attn_forward + divide;
+  * slots 0 and 2 of `indices` (the O(pairs) m2w / w2m arrays) are ignored and may be None;
+  * only the combination the model uses is implemented (PosEmb.SEPARATE, TableDims.D0,
+    IndexMode.INDIRECT); the backward pass is not implemented yet.
+"""
+import enum
+
+import torch
+from torch.autograd.function import Function
+
+from ... import _lib
+
+
+class PosEmb(enum.Enum):
+    NONE = 1
+    LINEAR = 2
+    SEPARATE = 3
+
+
+class TableDims(enum.Enum):
+    WHCD = 1
+    DWHC = 2
+    D0 = 3
+
+
+class IndexMode(enum.Enum):
+    DIRECT = 1
+    INDIRECT = 2
+
+
+class PrecisionMode(enum.Enum):
+    HALF_ALL = 1
+    HALF_FORWARD = 2
+    HALF_NONE = 3
+
+
+_DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_F16}
+
+
+def _require_cuda(name, t, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA (HIP) tensor")
+    if device is not None and t.device != device:
+        raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _as_int32(name, t, device):
+    """Index tensors arrive as int64 from torch ops; the kernels read int32."""
+    if not isinstance(t, torch.Tensor):
+        t = torch.as_tensor(t)
+    if t.dtype not in (torch.int32, torch.int64):
+        raise TypeError(f"{name} must be an int32/int64 tensor, got {t.dtype}")
+    if t.device != device:
+        if t.is_cuda:
+            raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+        t = t.to(device)
+    return t.to(torch.int32).contiguous()
+
+
+def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
+                             n_coords, return_stats=False):
+    """softmax-normalised window attention, [N,H,D] in the dtype of q.
+
+    q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5)
+    table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
+    table_sizes    int tensor / list [nd], per-axis element counts rows*H*D
+    w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
+    n2n            [N] window-sorted position -> row of q/k/v
+    n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
+    return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
+    """
+    _require_cuda("query", q)
+    dev = q.device
+    if q.dim() != 3:
+        raise ValueError(f"query must be [N,H,D], got {tuple(q.shape)}")
+    n, h, d = q.shape
+    if q.dtype not in _DTYPE_CODE:
+        raise TypeError(f"unsupported feature dtype {q.dtype} (float16 or float32)")
+    for name, t in (("key", k), ("value", v)):
+        _require_cuda(name, t, dev)
+        if t.shape != q.shape or t.dtype != q.dtype:
+            raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
+    if d not in (8, 16):
+        raise ValueError(f"head_dim must be 8 or 16, got {d}")
+    table_sizes = _as_int32("table_sizes", table_sizes, dev).reshape(-1)
+    nd = table_sizes.numel()
+    if nd not in (3, 6, 9):
+        raise ValueError(f"table_sizes must have 3, 6 or 9 entries, got {nd}")
+    table_len = table_q.numel()
+    for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
+        _require_cuda(name, t, dev)
+        if t.dtype != q.dtype:
+            raise TypeError(f"{name} must have the dtype of the features ({q.dtype}), got {t.dtype}")
+        if t.numel() != table_len:
+            raise ValueError("the three tables must have the same number of elements")
+    if table_len == 0 or table_len % (h * d) != 0:
+        raise ValueError(f"table length {table_len} is not a positive multiple of H*D = {h * d}")
+    w_sizes = _as_int32("w_sizes", w_sizes, dev)
+    w2n = _as_int32("w2n_indices", w2n, dev)
+    n2n = _as_int32("n2n_indices", n2n, dev)
+    if w_sizes.shape != w2n.shape or w_sizes.dim() != 1:
+        raise ValueError("w_sizes and w2n_indices must be 1-D of equal length")
+    if n2n.shape != (n,):
+        raise ValueError(f"n2n_indices must be [{n}], got {tuple(n2n.shape)}")
+    _require_cuda("n_coords", n_coords, dev)
+    if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
+        raise ValueError(f"n_coords must be float32 [{n},{nd}], got {n_coords.dtype} {tuple(n_coords.shape)}")
+
+    out = torch.empty_like(q)
+    omax = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
+    osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        status = _lib.lib().s3d_attn_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), table_q.data_ptr(), table_k.data_ptr(),
+            table_v.data_ptr(), table_sizes.data_ptr(), nd, table_len, w_sizes.data_ptr(),
+            w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
+            omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
+            n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype], stream)
+    _lib.check(status, "s3d_attn_fwd")
+    if return_stats:
+        return out, omax, osum
+    return out
+
+
+def _compute_dtype(precision):
+    """fp32 unless autocast is on and the precision mode allows half (attn_coff.py:172-175)."""
+    if torch.is_autocast_enabled() and precision != PrecisionMode.HALF_NONE:
+        return torch.get_autocast_dtype("cuda")
+    return torch.float32
+
+
+class SelfAttnAIOFunction(Function):
+    """Function of all-in-one self-attention (forward only)."""
+
+    @staticmethod
+    def forward(ctx, raw_query_feats, raw_key_feats, raw_value_feats, query_table, key_table,
+                value_table, table_offsets, indices, pe, table_dim, mode, precision):
+        if table_dim != TableDims.D0:
+            raise NotImplementedError("only TableDims.D0 tables are supported")
+        if pe != PosEmb.SEPARATE or mode != IndexMode.INDIRECT:
+            raise NotImplementedError("only PosEmb.SEPARATE with IndexMode.INDIRECT is implemented")
+        if len(indices) != 6:
+            raise ValueError("indices must be [m2w, w_sizes, w2m, w2n, n2n, n_coords]")
+        c_dtype = _compute_dtype(precision)
+        if c_dtype not in _DTYPE_CODE:
+            raise NotImplementedError(f"compute dtype {c_dtype} is not supported (float16 / float32)")
+        _, w_sizes, _, w2n, n2n, n_coords = indices
+        feats = [t.to(c_dtype).contiguous() for t in (raw_query_feats, raw_key_feats, raw_value_feats)]
+        tables = [t.to(c_dtype).contiguous() for t in (query_table, key_table, value_table)]
+        out = window_attention_forward(*feats, *tables, table_offsets, w_sizes, w2n, n2n,
+                                       n_coords.to(torch.float32).contiguous())
+        ctx.mark_non_differentiable(out)
+        return out
+
+    @staticmethod
+    def backward(ctx, *grad_outputs):
+        raise NotImplementedError("swin3d_amd implements the attention forward only")

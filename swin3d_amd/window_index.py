@@ -1,0 +1,115 @@
+"""Window index of the sparse window attention (host side of s3d_window_index).
+
+Mirrors BasicLayer.get_window_mapping / get_index01 / get_shifted_sp
+(Swin3D/modules/swin3d_layers.py:740-838) and sparse_self_attention (:76-150) without
+MinkowskiEngine: one HIP call sorts the voxels into windows and emits the segment
+offsets.  Window order is ascending (batch, wx, wy, wz); the reference's order is
+whatever MinkowskiEngine's pooling emits and attention does not depend on it.
+"""
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+
+@dataclass
+class WindowIndex:
+    n2n: torch.Tensor       # int32 [N]  window-sorted position -> original row
+    w_w_id: torch.Tensor    # int32 [N]  local id lx*ws^2 + ly*ws + lz per sorted position
+    w_sizes: torch.Tensor   # int32 [W]  voxels per window
+    w2n: torch.Tensor       # int32 [W]  exclusive prefix sum of w_sizes
+    num_windows: int        # W
+    num_pairs: int          # M = sum w_sizes^2
+    max_window_voxels: int
+    window_size: int
+
+    def local_xyz(self):
+        """int32 [N,3] voxel position inside its window, window-sorted order."""
+        ws = self.window_size
+        wid = self.w_w_id
+        return torch.stack([wid // (ws * ws), (wid // ws) % ws, wid % ws], dim=-1)
+
+    def inverse(self):
+        """int64 [N] original row -> window-sorted position."""
+        inv = torch.empty(self.n2n.numel(), dtype=torch.int64, device=self.n2n.device)
+        inv[self.n2n.long()] = torch.arange(self.n2n.numel(), device=self.n2n.device)
+        return inv
+
+
+def build_window_index(coords, stride, window_size, shift=0):
+    """coords int32 [N,4] (batch,x,y,z) CUDA tensor -> WindowIndex.
+
+    `shift` is in voxels (0, or window_size // 2 for the shifted window set).
+    Synchronises once to read the window count back.
+    """
+    if not coords.is_cuda:
+        raise RuntimeError("coords must be a CUDA (HIP) tensor")
+    if coords.dim() != 2 or coords.shape[1] != 4:
+        raise ValueError(f"coords must be [N,4] (batch,x,y,z), got {tuple(coords.shape)}")
+    dev = coords.device
+    coords = coords.to(torch.int32).contiguous()
+    n = coords.shape[0]
+    n2n = torch.empty(n, dtype=torch.int32, device=dev)
+    wwid = torch.empty(n, dtype=torch.int32, device=dev)
+    w_sizes = torch.empty(n, dtype=torch.int32, device=dev)
+    w2n = torch.empty(n, dtype=torch.int32, device=dev)
+    counts = torch.empty(4, dtype=torch.int64, device=dev)
+    lib = _lib.lib()
+    with torch.cuda.device(dev):
+        ws_bytes = lib.s3d_window_index_workspace_bytes(n)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window_size),
+                                      int(shift), n2n.data_ptr(), wwid.data_ptr(),
+                                      w_sizes.data_ptr(), w2n.data_ptr(), counts.data_ptr(),
+                                      workspace.data_ptr(), ws_bytes, stream)
+    _lib.check(status, "s3d_window_index")
+    num_w, num_m, max_w, err = counts.tolist()
+    if err:
+        raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
+                         "-8192..8191)")
+    return WindowIndex(n2n, wwid, w_sizes[:num_w], w2n[:num_w], int(num_w), int(num_m), int(max_w),
+                       int(window_size))
+
+
+def sparse_self_attention(w_w_id, w_sizes, protocol="v1"):
+    """O(pairs) pair index of the windows: x_offset / y_offset [M] (sorted positions of the
+    query / key of every pair, query-major inside a window) and, for protocol "v2", also
+    (m2w_indices [M], w_sizes, w2n_indices [W], w2m_indices [W]).  The fused attention op
+    does not read these arrays; they exist for callers that want the reference's layout."""
+    del w_w_id  # the pair index depends on the window sizes only
+    sizes = w_sizes.long()
+    sq = sizes * sizes
+    w2n = torch.cumsum(sizes, 0) - sizes
+    w2m = torch.cumsum(sq, 0) - sq
+    windows = torch.arange(sizes.numel(), device=sizes.device)
+    m2w = torch.repeat_interleave(windows, sq)
+    within = torch.arange(m2w.numel(), device=sizes.device) - w2m[m2w]
+    n_w = sizes[m2w]
+    x_offset = w2n[m2w] + torch.div(within, n_w, rounding_mode="floor")
+    y_offset = w2n[m2w] + within % n_w
+    if protocol == "v1":
+        return x_offset, y_offset
+    if protocol == "v2":
+        return x_offset, y_offset, m2w, w_sizes, w2n, w2m
+    raise ValueError(f"unknown protocol {protocol!r}")
+
+
+def get_index01(coords, stride, window_size, local_xyz, colors, shift=0, materialize_pairs=False):
+    """Arguments of the attention op for one window set, in the reference's tuple order
+    (x_offset, y_offset, m2w_indices, w_sizes, w2n_indices, n2n_indices, w2m_indices, n_coords).
+
+    local_xyz [N,3] fractional position of the point inside its voxel, colors [N,0|3|6] the
+    other signals, both in original row order.  n_coords = (window-local voxel + fraction,
+    signals) in window-sorted order, fp32.  The four O(pairs) entries are None unless
+    materialize_pairs is set.
+    """
+    index = build_window_index(coords, stride, window_size, shift)
+    order = index.n2n.long()
+    n_xyz = index.local_xyz().to(torch.float32) + local_xyz.to(torch.float32)[order]
+    n_coords = torch.cat([n_xyz, colors.to(torch.float32)[order]], dim=1).contiguous()
+    x_offset = y_offset = m2w = w2m = None
+    if materialize_pairs:
+        x_offset, y_offset, m2w, _, _, w2m = sparse_self_attention(index.w_w_id, index.w_sizes, "v2")
+    return (x_offset, y_offset, m2w, index.w_sizes, index.w2n, index.n2n, w2m, n_coords)

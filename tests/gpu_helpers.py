@@ -1,0 +1,37 @@
+"""Helpers of the GPU parity tests: move a numpy AttnCase to the device and call the op
+through the Python surface (ctypes -> C ABI -> HIP)."""
+import numpy as np
+import torch
+
+import swin3d_amd
+
+
+def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda"):
+    """-> numpy float64 output [N,H,D] of swin3d_amd.window_attention_forward."""
+    dev = torch.device(device)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    res = swin3d_amd.window_attention_forward(
+        t(case.q).to(dtype), t(case.k).to(dtype), t(case.v).to(dtype),
+        t(case.tq).to(dtype), t(case.tk).to(dtype), t(case.tv).to(dtype),
+        t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
+        return_stats=return_stats)
+    torch.cuda.synchronize()
+    if return_stats:
+        return tuple(r.double().cpu().numpy() for r in res)
+    return res.double().cpu().numpy()
+
+
+def assert_attn_close(got, ref, dtype):
+    """fp32: |a-b| <= 1e-5 * max(|b|, 1e-2 * max|ref|)   (1e-5 relative, scale floored at 1 % of
+    the largest reference magnitude); fp16: |a-b| <= 2e-3 absolute."""
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    assert np.isfinite(got).all()
+    err = np.abs(got - ref)
+    if dtype == torch.float32:
+        tol = 1e-5 * np.maximum(np.abs(ref), 1e-2 * np.abs(ref).max())
+    else:
+        tol = np.full_like(ref, 2e-3)
+    worst = np.unravel_index(np.argmax(err - tol), err.shape)
+    assert (err <= tol).all(), (f"max err {err.max():.3e} (tol there {tol[worst]:.3e}) at {worst}: "
+                                f"got {got[worst]:.6f} ref {ref[worst]:.6f}")

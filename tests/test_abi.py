@@ -1,0 +1,51 @@
+"""The C-ABI library loads and exports every symbol include/swin3d_amd.h declares
+(no device calls: runs without a GPU)."""
+import ctypes
+import os
+import re
+
+from conftest import ROOT
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "swin3d_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(s3d_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_symbols()
+    for must in ("s3d_attn_fwd", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+                 "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(hip_lib):
+    for name in _declared_symbols():
+        assert hasattr(hip_lib, name), f"{name} is declared in the header but not exported"
+
+
+def test_python_signatures_cover_the_header(hip_lib):
+    from swin3d_amd import _lib
+    assert sorted(_lib.SIGNATURES) == _declared_symbols()
+
+
+def test_version_and_error_string(hip_lib):
+    assert hip_lib.s3d_version() >= 100
+    assert isinstance(hip_lib.s3d_last_error_string(), bytes)
+
+
+def test_argument_errors_are_reported_without_a_device(hip_lib):
+    from swin3d_amd import _lib
+    # K out of range is rejected before anything touches the GPU
+    status = hip_lib.s3d_knn(0, None, 0, None, 0, None, None, 1, None, None, 0.0, None, 0, None)
+    assert status < 0
+    assert b"K=0" in hip_lib.s3d_last_error_string()
+    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 1, None)
+    assert status < 0 and b"table_len" in hip_lib.s3d_last_error_string()
+    try:
+        _lib.check(status, "s3d_attn_fwd")
+    except ValueError as e:
+        assert "s3d_attn_fwd failed" in str(e)
+    else:
+        raise AssertionError("check() must raise on a negative status")

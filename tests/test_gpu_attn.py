@@ -1,0 +1,176 @@
+"""GPU parity of the window attention forward (HIP through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_attn_case, scene_attn_case, to_half_and_back, n_coords_from_scene
+from swin3d_amd import crse, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(oracle_lib, case, dtype):
+    from gpu_helpers import run_attention, assert_attn_close
+    if dtype == torch.float16:
+        to_half_and_back(case)       # the oracle sees exactly the fp16-rounded inputs
+    ref = oracle_lib.attn_fwd(*case.oracle_args())
+    got = run_attention(case, dtype)
+    assert_attn_close(got, ref, dtype)
+    return got, ref
+
+
+def _sharp16(case):
+    """fp16 variant of the sharp recipe: logits stay peaky, values are scaled so that the fp16
+    rounding of the OUTPUT itself (half an ulp of a number in [4,8) is 2e-3) stays below the
+    2e-3 absolute tolerance."""
+    case.v *= np.float32(0.4)
+    case.tv *= np.float32(0.2)
+    return case
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("cRSE", ["XYZ", "XYZ_RGB", "XYZ_RGB_NORM"])
+@pytest.mark.parametrize("heads,dim,ws", [(6, 8, 5), (6, 16, 7)])
+def test_random_scenes_sharp(oracle_lib, hip_lib, dtype, cRSE, heads, dim, ws):
+    case = make_attn_case(oracle_lib, seed=31, n=1500, ws=ws, quant=4, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(9, 9, 4), batches=2, recipe="sharp")
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_stage1_room_layer_recipe(oracle_lib, hip_lib, dtype):
+    """config 1 (fp32) / a 20k-voxel cut of config 2 (fp16): synthetic room, freshly initialised layer."""
+    cRSE = "XYZ_RGB" if dtype == torch.float32 else "XYZ_RGB_NORM"
+    scene = synth.make_room((6, 5, 3), 8, 20000, seed=0)
+    case = scene_attn_case(oracle_lib, scene, 5, 4, 6, 8, cRSE, recipe="layer")
+    got, ref = _check(oracle_lib, case, dtype)
+    assert got.shape == (scene.coords.shape[0], 6, 8)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_shifted_windows_and_stride(oracle_lib, hip_lib, dtype):
+    case = make_attn_case(oracle_lib, seed=32, n=1200, ws=7, quant=4, heads=12, dim=16, cRSE="XYZ_RGB_NORM",
+                          extent=(10, 10, 5), stride=2, shift=3, recipe="sharp")
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
+    """A fully occupied 14x7x7 block at window 7: two windows of 343 voxels (several key chunks)."""
+    ws, quant, heads, dim = 7, 4, 2, 16
+    g = np.stack(np.meshgrid(np.arange(14), np.arange(7), np.arange(7), indexing="ij"), -1).reshape(-1, 3)
+    coords = np.concatenate([np.zeros((g.shape[0], 1), np.int64), g], 1).astype(np.int32)
+    rng = np.random.default_rng(33)
+    coords = coords[rng.permutation(coords.shape[0])]
+    frac = rng.random((coords.shape[0], 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (coords.shape[0], 6)).astype(np.float32)
+    case = make_attn_case(oracle_lib, seed=33, n=coords.shape[0], ws=ws, quant=quant, heads=heads, dim=dim)
+    case.coords = coords
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
+    assert case.index["w_sizes"].tolist() == [343, 343]
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
+def test_single_voxel_windows_and_one_head(oracle_lib, hip_lib):
+    coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
+    case = make_attn_case(oracle_lib, seed=34, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")
+    frac = np.random.default_rng(3).random((4, 3)).astype(np.float32)
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, np.zeros((4, 0), np.float32),
+                                                    1, 5, 4, "XYZ")
+    assert case.index["w_sizes"].tolist() == [1, 2, 1]
+    _check(oracle_lib, case, torch.float32)
+
+
+def test_upper_edge_rows_are_folded_not_out_of_bounds(oracle_lib, hip_lib):
+    """Opposite unit normals in one window: rel == rows on the last axis table (the reference
+    reads past the table there); the library and the oracle both fold onto the last row."""
+    case = make_attn_case(oracle_lib, seed=35, n=600, ws=5, quant=4, heads=2, dim=8, cRSE="XYZ_RGB_NORM",
+                          extent=(6, 6, 3))
+    rng = np.random.default_rng(35)
+    signs = rng.choice([-1.0, 1.0], size=(case.N, 6)).astype(np.float32)
+    case.n_coords[:, 3:] = signs * 8.0              # +-1 times 2*quant
+    out, _, _, edges = oracle_lib.attn_fwd(*case.oracle_args(), return_stats=True)
+    assert edges > 0
+    _check(oracle_lib, case, torch.float32)
+
+
+def test_stats_outputs(oracle_lib, hip_lib):
+    from gpu_helpers import run_attention
+    case = make_attn_case(oracle_lib, seed=36, n=800, ws=5, quant=4, heads=6, dim=8, extent=(8, 8, 3))
+    ref, rmax, rsum, _ = oracle_lib.attn_fwd(*case.oracle_args(), return_stats=True)
+    got, gmax, gsum = run_attention(case, torch.float32, return_stats=True)
+    np.testing.assert_allclose(gmax, rmax, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(gsum, rsum, rtol=2e-5)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_empty_input(hip_lib):
+    import swin3d_amd
+    dev = torch.device("cuda")
+    q = torch.zeros((0, 6, 8), device=dev)
+    t = torch.zeros(14976, device=dev)
+    sizes = torch.tensor(crse.crse_table_sizes(5, 4, 6, 8, "XYZ_RGB_NORM"), dtype=torch.int32, device=dev)
+    e = torch.zeros(0, dtype=torch.int32, device=dev)
+    out = swin3d_amd.window_attention_forward(q, q, q, t, t, t, sizes, e, e, e,
+                                              torch.zeros((0, 9), device=dev))
+    assert out.shape == (0, 6, 8)
+
+
+def test_autograd_function_surface(oracle_lib, hip_lib):
+    """SelfAttnAIOFunction.apply with the reference's argument list: int64 index tensors, the
+    O(pairs) slots left as None, fp16 under autocast with HALF_FORWARD, fp32 with HALF_NONE."""
+    import swin3d_amd as s3d
+    case = make_attn_case(oracle_lib, seed=37, n=900, ws=5, quant=4, heads=6, dim=8, extent=(8, 8, 3),
+                          recipe="layer")
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    idx = [None, t(case.index["w_sizes"]).long(), None, t(case.index["w2n"]).long(),
+           t(case.index["n2n"]).long(), t(case.n_coords)]
+    args = [t(case.q), t(case.k), t(case.v), t(case.tq), t(case.tk), t(case.tv), t(case.table_sizes), idx,
+            s3d.PosEmb.SEPARATE, s3d.TableDims.D0, s3d.IndexMode.INDIRECT]
+    ref = oracle_lib.attn_fwd(*case.oracle_args())
+    out = s3d.SelfAttnAIOFunction.apply(*args, s3d.PrecisionMode.HALF_NONE)
+    assert out.dtype == torch.float32
+    from gpu_helpers import assert_attn_close
+    assert_attn_close(out.double().cpu().numpy(), ref, torch.float32)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out16 = s3d.SelfAttnAIOFunction.apply(*args, s3d.PrecisionMode.HALF_FORWARD)
+        out32 = s3d.SelfAttnAIOFunction.apply(*args, s3d.PrecisionMode.HALF_NONE)
+    assert out16.dtype == torch.float16 and out32.dtype == torch.float32
+    ref16 = oracle_lib.attn_fwd(*to_half_and_back(case).oracle_args())
+    assert_attn_close(out16.double().cpu().numpy(), ref16, torch.float16)
+
+
+def test_headline_size_properties(oracle_lib, hip_lib):
+    """Config 2 at full size (200k voxels, fp16, 9 axes): size-independent properties on the whole
+    output plus oracle parity on a random sample of windows."""
+    from gpu_helpers import run_attention, assert_attn_close
+    scene = synth.make_room((10, 8, 3), 30, 200_000, seed=0)
+    case = scene_attn_case(oracle_lib, scene, 5, 4, 6, 8, "XYZ_RGB_NORM", recipe="layer")
+    to_half_and_back(case)
+    got = run_attention(case, torch.float16)
+    assert np.isfinite(got).all()
+    # (a) sample of windows against the oracle
+    rng = np.random.default_rng(0)
+    idx = case.index
+    pick = np.sort(rng.choice(idx["W"], size=300, replace=False))
+    pos = np.concatenate([np.arange(idx["w2n"][w], idx["w2n"][w] + idx["w_sizes"][w]) for w in pick])
+    rows = idx["n2n"][pos]
+    sub_sizes = idx["w_sizes"][pick]
+    sub = oracle_lib.attn_fwd(case.q[rows], case.k[rows], case.v[rows], case.tq, case.tk, case.tv,
+                              case.table_sizes, sub_sizes, np.cumsum(sub_sizes) - sub_sizes,
+                              np.arange(rows.shape[0], dtype=np.int32), case.n_coords[pos])
+    assert_attn_close(got[rows], sub, torch.float16)
+    # (b) constant values with a zero value table pass through unchanged (softmax weights sum to 1)
+    case.v[:] = 0.5
+    case.tv[:] = 0
+    const = run_attention(case, torch.float16)
+    assert np.abs(const - 0.5).max() <= 1e-3
+    # (c) the output is a convex combination: inside [min, max] of (v + Tv) bounds
+    assert got.min() >= -5 and got.max() <= 5

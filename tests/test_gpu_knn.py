@@ -1,0 +1,111 @@
+"""GPU parity of the grid-bucketed KNN (bit-exact indices and fp32 squared distances)."""
+import numpy as np
+import pytest
+import torch
+
+from swin3d_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(k, src, qry, so, qo, cell=0.0):
+    import swin3d_amd
+    c = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    idx, d2 = swin3d_amd.knn_query(k, c(src), c(qry), c(so), c(qo), cell_size=cell)
+    torch.cuda.synchronize()
+    return idx.cpu().numpy(), d2.cpu().numpy()
+
+
+def _compare(oracle_lib, k, src, qry, so, qo, cell=0.0):
+    ridx, rd2 = oracle_lib.knn(k, src, qry, so, qo)
+    idx, d2 = _run(k, src, qry, so, qo, cell)
+    np.testing.assert_array_equal(idx, ridx)
+    np.testing.assert_array_equal(d2, rd2)
+
+
+@pytest.mark.parametrize("k", [1, 3, 5, 16, 33, 64])
+@pytest.mark.parametrize("cell", [0.0, 0.7, 5.0, 1000.0])
+def test_random_clouds(oracle_lib, hip_lib, k, cell):
+    rng = np.random.default_rng(k)
+    src = (rng.random((4000, 3)) * [30, 20, 5]).astype(np.float32)
+    qry = (rng.random((1500, 3)) * [34, 24, 9] - 2).astype(np.float32)     # some queries outside the box
+    so, qo = np.array([1500, 4000], np.int32), np.array([700, 1500], np.int32)
+    _compare(oracle_lib, k, src, qry, so, qo, cell)
+
+
+def test_lattice_ties_go_to_lower_row(oracle_lib, hip_lib):
+    g = np.arange(0, 12, dtype=np.float32)
+    src = np.stack(np.meshgrid(g, g, g, indexing="ij"), -1).reshape(-1, 3)
+    rng = np.random.default_rng(5)
+    src = src[rng.permutation(src.shape[0])]
+    qry = np.concatenate([src[:200], src[:200] + np.float32(0.5)])          # on and between lattice points
+    one = lambda n: np.array([n], np.int32)
+    for k in (3, 7, 16):
+        for cell in (0.0, 1.0, 2.5):
+            _compare(oracle_lib, k, src, qry, one(src.shape[0]), one(qry.shape[0]), cell)
+
+
+def test_short_empty_and_unassigned_segments(oracle_lib, hip_lib):
+    rng = np.random.default_rng(6)
+    src = rng.random((50, 3)).astype(np.float32) * 10
+    qry = rng.random((30, 3)).astype(np.float32) * 10
+    so = np.array([2, 2, 40], np.int32)       # 2 sources, none, 38; rows 40..49 belong to no segment
+    qo = np.array([10, 20, 25], np.int32)     # queries 25..29 belong to no segment
+    ridx, rd2 = oracle_lib.knn(4, src, qry, so, qo)
+    idx, d2 = _run(4, src, qry, so, qo)
+    np.testing.assert_array_equal(idx, ridx)
+    np.testing.assert_array_equal(d2, rd2)
+    assert (idx[10:20] == -1).all() and (idx[25:] == -1).all() and (idx[:10, 2:] == -1).all()
+    assert (d2[25:] == np.float32(2147483648.0)).all()
+
+
+def test_identical_points_and_degenerate_extent(oracle_lib, hip_lib):
+    src = np.zeros((100, 3), np.float32)
+    src[:, 0] = np.repeat(np.arange(10, dtype=np.float32), 10)             # a line with 10-fold duplicates
+    qry = np.array([[4.2, 0, 0], [100, 100, 100], [-3, 0, 0]], np.float32)
+    one = lambda n: np.array([n], np.int32)
+    _compare(oracle_lib, 16, src, qry, one(100), one(3))
+    _compare(oracle_lib, 16, np.zeros((40, 3), np.float32), qry, one(40), one(3))   # all sources identical
+
+
+def test_autograd_function_returns_euclidean_distance(oracle_lib, hip_lib):
+    import swin3d_amd
+    rng = np.random.default_rng(7)
+    src = (rng.random((500, 3)) * 10).astype(np.float32)
+    qry = (rng.random((100, 3)) * 10).astype(np.float32)
+    so, qo = torch.tensor([500], dtype=torch.int32).cuda(), torch.tensor([100], dtype=torch.int32).cuda()
+    idx, dist = swin3d_amd.KNN.apply(3, torch.from_numpy(src).cuda(), torch.from_numpy(qry).cuda(), so, qo)
+    ridx, rd2 = oracle_lib.knn(3, src, qry, so.cpu().numpy(), qo.cpu().numpy())
+    assert idx.dtype == torch.int32 and dist.dtype == torch.float32
+    np.testing.assert_array_equal(idx.cpu().numpy(), ridx)
+    np.testing.assert_array_equal(dist.cpu().numpy(), np.sqrt(rd2))
+
+
+def _knn_scene():
+    scene = synth.make_room((10, 8, 3), 30, 200_000, seed=0)
+    coarse, _ = synth.grid_downsample(scene, 2)
+    centres = (coarse.coords[:, 1:].astype(np.float32) + np.float32(1.0))[:50_000]   # (cell + 0.5) * 2
+    return scene.xyz, np.ascontiguousarray(centres)
+
+
+@pytest.mark.parametrize("direction", ["down", "up"])
+def test_headline_sizes(oracle_lib, hip_lib, direction):
+    """Config 4: 200k sources / 50k cell-centre queries, K=16, and the reverse with K=3.
+    Whole output: ordering and self-consistency properties; a random 2000-query sample is
+    compared bit for bit with the brute-force oracle."""
+    fine, centres = _knn_scene()
+    src, qry, k = (fine, centres, 16) if direction == "down" else (centres, fine, 3)
+    one = lambda n: np.array([n], np.int32)
+    idx, d2 = _run(k, src, qry, one(src.shape[0]), one(qry.shape[0]))
+    assert (idx >= 0).all() and (idx < src.shape[0]).all()
+    assert (np.diff(d2, axis=1) >= 0).all()
+    tie = np.diff(d2, axis=1) == 0
+    assert (np.diff(idx, axis=1)[tie] > 0).all()                          # equal distance: ascending row
+    d = src[idx] - qry[:, None, :]
+    recomputed = ((d[..., 0] * d[..., 0]).astype(np.float32) + (d[..., 1] * d[..., 1]).astype(np.float32)).astype(np.float32)
+    recomputed = (recomputed + (d[..., 2] * d[..., 2]).astype(np.float32)).astype(np.float32)
+    np.testing.assert_array_equal(d2, recomputed)
+    pick = np.sort(np.random.default_rng(0).choice(qry.shape[0], 2000, replace=False))
+    ridx, rd2 = oracle_lib.knn(k, src, qry[pick], one(src.shape[0]), one(2000))
+    np.testing.assert_array_equal(idx[pick], ridx)
+    np.testing.assert_array_equal(d2[pick], rd2)

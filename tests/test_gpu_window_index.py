@@ -1,0 +1,93 @@
+"""GPU parity of the window sort / segment offsets (bit-exact against the CPU oracle)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_scene
+from swin3d_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(coords, stride, ws, shift):
+    import swin3d_amd
+    index = swin3d_amd.build_window_index(torch.from_numpy(coords).cuda(), stride, ws, shift)
+    torch.cuda.synchronize()
+    return index
+
+
+def _compare(oracle_lib, coords, stride, ws, shift):
+    ref = oracle_lib.window_index(coords, stride, ws, shift)
+    got = _run(coords, stride, ws, shift)
+    assert got.num_windows == ref["W"] and got.num_pairs == ref["M"]
+    assert got.max_window_voxels == (int(ref["w_sizes"].max()) if ref["W"] else 0)
+    np.testing.assert_array_equal(got.n2n.cpu().numpy(), ref["n2n"])
+    np.testing.assert_array_equal(got.w_w_id.cpu().numpy(), ref["w_w_id"])
+    np.testing.assert_array_equal(got.w_sizes.cpu().numpy(), ref["w_sizes"])
+    np.testing.assert_array_equal(got.w2n.cpu().numpy(), ref["w2n"])
+    return got
+
+
+@pytest.mark.parametrize("ws,stride,shift", [(5, 1, 0), (5, 1, 2), (7, 2, 3), (7, 4, 0), (3, 8, 1), (10, 1, 5)])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_scenes(oracle_lib, hip_lib, ws, stride, shift, seed):
+    rng = np.random.default_rng(seed)
+    coords = random_scene(rng, 5000, extent=(40, 40, 12), batches=3, stride=stride)
+    _compare(oracle_lib, coords, stride, ws, shift)
+
+
+def test_duplicates_keep_row_order(oracle_lib, hip_lib):
+    rng = np.random.default_rng(2)
+    coords = random_scene(rng, 3000, extent=(6, 6, 3), duplicates=True)
+    assert len({tuple(r) for r in coords.tolist()}) < coords.shape[0]
+    _compare(oracle_lib, coords, 1, 5, 0)
+
+
+def test_empty_single_and_one_window(oracle_lib, hip_lib):
+    _compare(oracle_lib, np.zeros((0, 4), np.int32), 1, 5, 0)
+    _compare(oracle_lib, np.array([[3, -7, 8, 9]], np.int32), 1, 5, 2)
+    g = np.stack(np.meshgrid(np.arange(5), np.arange(5), np.arange(5), indexing="ij"), -1).reshape(-1, 3)
+    coords = np.concatenate([np.zeros((125, 1), np.int64), g], 1).astype(np.int32)[::-1].copy()
+    got = _compare(oracle_lib, coords, 1, 5, 0)
+    assert got.num_windows == 1 and got.num_pairs == 125 * 125
+
+
+def test_out_of_range_coordinates_are_reported(hip_lib):
+    import swin3d_amd
+    coords = torch.tensor([[0, 0, 0, 0], [0, 5 * 9000, 0, 0]], dtype=torch.int32).cuda()
+    with pytest.raises(ValueError, match="range"):
+        swin3d_amd.build_window_index(coords, 1, 5, 0)
+    with pytest.raises(ValueError):
+        swin3d_amd.build_window_index(coords, 1, 11, 0)        # window size beyond the key layout
+
+
+@pytest.mark.parametrize("shift", [0, 2])
+def test_headline_room(oracle_lib, hip_lib, shift):
+    scene = synth.make_room((10, 8, 3), 30, 200_000, seed=0)
+    rng = np.random.default_rng(0)
+    coords = scene.coords[rng.permutation(scene.coords.shape[0])]     # arbitrary input order
+    got = _compare(oracle_lib, coords, 1, 5, shift)
+    assert got.inverse()[got.n2n.long()].tolist()[:100] == list(range(100))
+
+
+def test_get_index01_matches_reference_formulas(oracle_lib, hip_lib):
+    """n_coords = window-local voxel + fraction, signals appended, all gathered by n2n
+    (swin3d_layers.py:800-804); pair arrays on request."""
+    import swin3d_amd
+    from helpers import n_coords_from_scene
+    rng = np.random.default_rng(4)
+    coords = random_scene(rng, 2000, extent=(15, 15, 6), batches=2)
+    frac = rng.random((2000, 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (2000, 6)).astype(np.float32)
+    args = swin3d_amd.get_index01(torch.from_numpy(coords).cuda(), 1, 5, torch.from_numpy(frac).cuda(),
+                                  torch.from_numpy(sig).cuda(), shift=2, materialize_pairs=True)
+    x_off, y_off, m2w, w_sizes, w2n, n2n, w2m, n_coords = args
+    index, scaled = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, 5, 4, "XYZ_RGB_NORM", shift=2)
+    np.testing.assert_array_equal(n2n.cpu().numpy(), index["n2n"])
+    got_scaled = swin3d_amd.scale_crse_coords(n_coords, 4, "XYZ_RGB_NORM").cpu().numpy()
+    np.testing.assert_array_equal(got_scaled, scaled)                 # bit-exact fp32
+    o_w2m, o_m2w, o_x, o_y = oracle_lib.pair_index(index["w_sizes"])
+    np.testing.assert_array_equal(x_off.cpu().numpy(), o_x)
+    np.testing.assert_array_equal(y_off.cpu().numpy(), o_y)
+    np.testing.assert_array_equal(m2w.cpu().numpy(), o_m2w)
+    np.testing.assert_array_equal(w2m.cpu().numpy(), o_w2m)
