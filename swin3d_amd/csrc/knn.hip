@@ -240,6 +240,19 @@ __global__ __launch_bounds__(kThreads) void knn_scatter_kernel(
                               __int_as_float(static_cast<int>(i)));
 }
 
+// ((dx*dx) + (dy*dy)) + (dz*dz) with d = src - query and every operation rounded to fp32 on
+// its own: contraction into fused multiply-adds is switched off for this function (the
+// compiler's default for device code is to fuse).
+__device__ __forceinline__ float dist2_unfused(float sx, float sy, float sz, float qx, float qy,
+                                               float qz)
+{
+#pragma clang fp contract(off)
+    const float dx = sx - qx, dy = sy - qy, dz = sz - qz;
+    const float xx = dx * dx, yy = dy * dy, zz = dz * dz;
+    const float xy = xx + yy;
+    return xy + zz;
+}
+
 __device__ __forceinline__ bool cand_less(float d, int i, float d2, int i2)
 {
     return d < d2 || (d == d2 && i < i2);
@@ -356,10 +369,7 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
                         const int s_begin = row[x0], s_end = row[x1 + 1];
                         for (int s = s_begin; s < s_end; ++s) {
                             const float4 p = sorted[s];
-                            const float dx = __fsub_rn(p.x, qx), dy = __fsub_rn(p.y, qy),
-                                        dz = __fsub_rn(p.z, qz);
-                            const float d2 = __fadd_rn(
-                                __fadd_rn(__fmul_rn(dx, dx), __fmul_rn(dy, dy)), __fmul_rn(dz, dz));
+                            const float d2 = dist2_unfused(p.x, p.y, p.z, qx, qy, qz);
                             const int si = __float_as_int(p.w);
                             if (cand_less(d2, si, best.worst_d(K), best.worst_i(K)))
                                 best.insert(d2, si, K);

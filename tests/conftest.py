@@ -32,6 +32,8 @@ def hip_lib():
 
 def random_scene(rng, n, extent=(12, 12, 6), batches=1, stride=1, duplicates=False):
     """n distinct voxels (batch,x,y,z) int32 inside a small box, unsorted."""
+    capacity = batches * 8 * extent[0] * extent[1] * extent[2]
+    assert duplicates or n <= 0.8 * capacity, f"{n} distinct voxels do not fit a box of {capacity} cells"
     rows = set()
     out = []
     while len(out) < n:

@@ -23,13 +23,17 @@ def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda"):
 
 
 def assert_attn_close(got, ref, dtype):
-    """fp32: |a-b| <= 1e-5 * max(|b|, 1e-2 * max|ref|)   (1e-5 relative, scale floored at 1 % of
-    the largest reference magnitude); fp16: |a-b| <= 2e-3 absolute."""
+    """fp32: |a-b| <= 1e-5 * scale, scale = max(largest |ref| over the D channels of the same
+    (voxel, head), 1e-2 * max|ref|): 1e-5 relative to the head vector the element belongs to.
+    An element-wise relative bound is not attainable in fp32: a channel that cancels to ~0 still
+    carries the rounding of logits of magnitude ~10 (one fp32 ulp there is 1e-6, and an absolute
+    logit error is a relative error of the softmax weight).  fp16: |a-b| <= 2e-3 absolute."""
     got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
     assert np.isfinite(got).all()
     err = np.abs(got - ref)
     if dtype == torch.float32:
-        tol = 1e-5 * np.maximum(np.abs(ref), 1e-2 * np.abs(ref).max())
+        row_scale = np.abs(ref).max(axis=-1, keepdims=True)
+        tol = 1e-5 * np.maximum(row_scale, 1e-2 * np.abs(ref).max()) * np.ones_like(ref)
     else:
         tol = np.full_like(ref, 2e-3)
     worst = np.unravel_index(np.argmax(err - tol), err.shape)

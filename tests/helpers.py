@@ -83,10 +83,3 @@ def to_half_and_back(case):
     case.q, case.k, case.v = h(case.q), h(case.k), h(case.v)
     case.tq, case.tk, case.tv = h(case.tq), h(case.tk), h(case.tv)
     return case
-
-
-def attn_tolerance_fp32(ref):
-    """|a - b| <= 1e-5 * max(|b|, 1e-2 * max|ref|): 1e-5 relative, with a floor on the scale so
-    that outputs which cancel to ~0 are not held to an impossible bound."""
-    ref = np.asarray(ref, np.float64)
-    return 1e-5 * np.maximum(np.abs(ref), 1e-2 * np.abs(ref).max())

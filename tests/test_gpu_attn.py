@@ -68,7 +68,8 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
     coords = coords[rng.permutation(coords.shape[0])]
     frac = rng.random((coords.shape[0], 3)).astype(np.float32)
     sig = rng.uniform(-1, 1, (coords.shape[0], 6)).astype(np.float32)
-    case = make_attn_case(oracle_lib, seed=33, n=coords.shape[0], ws=ws, quant=quant, heads=heads, dim=dim)
+    case = make_attn_case(oracle_lib, seed=33, n=coords.shape[0], ws=ws, quant=quant, heads=heads, dim=dim,
+                          extent=(12, 12, 6))
     case.coords = coords
     case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
     assert case.index["w_sizes"].tolist() == [343, 343]
