@@ -37,6 +37,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (1 = force the generic kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -77,17 +78,20 @@ def main():
     n_crse = crse.scale_crse_coords(n_coords, quant, cRSE)
     q_d, k_d, v_d = t(q), t(k), t(v)
     tq_d, tk_d, tv_d = (t(x) for x in tables)
-    sizes_d = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    c_sizes = (ctypes.c_int32 * nd)(*sizes)
     out = torch.empty_like(q_d)
     num_w, num_m = index.num_windows, index.num_pairs
+    ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, heads, dim, num_w)
+    workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
 
     def step():
         status = lib.s3d_attn_fwd(q_d.data_ptr(), k_d.data_ptr(), v_d.data_ptr(), tq_d.data_ptr(),
-                                  tk_d.data_ptr(), tv_d.data_ptr(), sizes_d.data_ptr(), nd, table_len,
+                                  tk_d.data_ptr(), tv_d.data_ptr(), c_sizes, nd, table_len,
                                   index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
                                   n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  _lib.S3D_DTYPE_F16, stream.cuda_stream)
+                                  _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
+                                  stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")
 

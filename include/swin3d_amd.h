@@ -63,8 +63,9 @@ const char *s3d_last_error_string(void);
  *
  *   q, k, v        device [N,H,D] of `dtype`, original voxel order (q pre-scaled)
  *   table_q/k/v    device [table_len] of `dtype`, layout [axis][row][h][c]
- *   table_sizes    device int32 [nd], table_sizes[n] = rows_n * H * D
- *                  (the reference's `table_offsets` tensor, fwd.cu:258,285)
+ *   table_sizes    HOST int32 [nd], table_sizes[n] = rows_n * H * D (the values of the
+ *                  reference's `table_offsets` tensor, fwd.cu:258,285; read on the host so
+ *                  that the row counts travel as kernel arguments)
  *   table_len      elements per table = sum_n table_sizes[n]
  *   w_sizes, w2n   device int32 [W]: voxels per window, exclusive prefix sum
  *   n2n            device int32 [N]: window-sorted position -> original row
@@ -74,7 +75,11 @@ const char *s3d_last_error_string(void);
  *                  (the tensor cal_max_coffs returns)
  *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
- *   D in {8,16,32}, nd in {3,6,9}, H >= 1.
+ *   flags          0, or S3D_ATTN_FORCE_GENERIC to run the VALU kernel for every case
+ *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
+ *                  (a transposed copy of the value table and the per-window work-item prefix
+ *                  of the MFMA kernel)
+ *   D in {8,16}, nd in {3,6,9}, H >= 1.
  *
  * Row index of axis n for the pair (query i, key j), all in fp32:
  *   rel = (n_coords[i][n] - n_coords[j][n]) + float(rows_n / 2)
@@ -82,12 +87,18 @@ const char *s3d_last_error_string(void);
  * (Swin3D/src/attn/attn_utils.cuh:444-450; the reference indexes one row past
  * the axis table when the clamped value equals rows_n, this library folds that
  * case onto the last row).
+ *
+ * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.
  */
+#define S3D_ATTN_FORCE_GENERIC 1
+size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,
+                                    int64_t W);
 int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_q,
                  const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
                  int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
                  const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
-                 int32_t H, int32_t D, int64_t W, int32_t dtype, void *stream);
+                 int32_t H, int32_t D, int64_t W, int32_t dtype, int32_t flags, void *workspace,
+                 size_t workspace_bytes, void *stream);
 
 /*
  * Window sort + segment offsets.

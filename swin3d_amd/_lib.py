@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libswin3d_amd.so")
 S3D_DTYPE_F32 = 0
 S3D_DTYPE_F16 = 1
 KNN_KMAX = 64
+S3D_ATTN_FORCE_GENERIC = 1
 
 _lib = None
 
@@ -23,7 +24,9 @@ _i64 = ctypes.c_int64
 SIGNATURES = {
     "s3d_version": (ctypes.c_int, []),
     "s3d_last_error_string": (ctypes.c_char_p, []),
-    "s3d_attn_fwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 + [_i64, _i32, _i32, _i64, _i32, _vp]),
+    "s3d_attn_fwd_workspace_bytes": (ctypes.c_size_t, [_vp, _i32, _i32, _i32, _i64]),
+    "s3d_attn_fwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
+                     [_i64, _i32, _i32, _i64, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_window_index_workspace_bytes": (ctypes.c_size_t, [_i64]),
     "s3d_window_index": (ctypes.c_int, [_vp, _i64, _i32, _i32, _i32] + [_vp] * 6 + [ctypes.c_size_t, _vp]),
     "s3d_knn_workspace_bytes": (ctypes.c_size_t, [_i64, _i64, _i32]),

@@ -12,12 +12,14 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libswin3d_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["api_common.hip", "attn_fwd.hip", "window_index.hip", "knn.hip"]
+SOURCES = ["api_common.hip", "attn_fwd.hip", "attn_fwd_generic.hip", "attn_fwd_mfma.hip",
+           "window_index.hip", "knn.hip"]
 
 # packed-fp32 VALU forms are disabled for every device compilation unit
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-munsafe-fp-atomics",   # LDS float adds as one ds_add_f32 instead of a compare-and-swap loop
     "-Wno-unused-command-line-argument",
 ]
 

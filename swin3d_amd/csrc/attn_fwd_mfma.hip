@@ -1,0 +1,559 @@
+// Sparse-voxel windowed self-attention forward with cRSE tables: MFMA kernel (gfx950, fp16).
+//
+// One wavefront owns one window and walks it in 32-query x 32-key tiles.  For a tile and a head
+//   S^T   = K Q^T                       one MFMA, lands directly in the logit registers
+//   QT_n  = Tq_n Q^T,  KT_n = Tk_n K^T  per signal axis n, MFMA -> LDS ("every table row
+//                                       against every query / key of the tile")
+// so that the table terms of a pair's logit become two 4-byte LDS gathers per axis
+//   L(i,j) = S(i,j) + sum_n QT_n[row_n(i,j)][i] + KT_n[j][row_n(i,j)]
+// instead of 2*D-element table row gathers.  The value side uses the transposed trick:
+//   sum_j P(i,j) Tv_n[row_n(i,j)] = sum_r H_n[r][i] Tv_n[r],  H_n[r][i] = sum_{j: row_n(i,j)=r} P(i,j)
+// a per-query histogram of the softmax weights over table rows, followed by MFMAs against a
+// transposed copy of the value table.  P V is an MFMA as well.
+//
+// The histogram is accumulated with INTEGER LDS atomics on 2^-24 fixed point (softmax weights
+// are in [0,1], at most 32 of them meet in one bin): ds_add_u32 runs at full LDS rate while
+// ds_add_f32 measured about six times slower on this part.
+//
+// Lane layout = the 32x32 MFMA accumulator layout: lane l holds query i = l % 32 and, in
+// register v, key j = 8*(v/4) + 4*(l/32) + v%4, so logits, softmax weights and the B operand
+// of the value MFMAs never move between lanes.  QT / H are stored [row][query] (bank = query,
+// conflict-free for any row pattern), KT is stored [key][row] (one key per half-wave: the
+// gathers hit consecutive words of one row).
+//
+// The row indices depend on the pair only; they are computed once per tile (fp32, in the
+// reference's operation order, Swin3D/src/attn/attn_utils.cuh:444-450) and kept as bytes in
+// registers across heads when the window has a single key tile.
+//
+// Latency: a window is a long chain of small dependent steps, so every global load is issued
+// one step ahead of its use (next head's q/k/v fragments, next axis' table fragments) and the
+// transposed value table of all heads sits in LDS, shared by the wavefronts of the workgroup.
+#include "attn_kernels.h"
+
+namespace s3d {
+namespace {
+
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+constexpr int kWaves = 8;             // wavefronts per workgroup (they share the value table in LDS)
+constexpr int kTile = 32;             // queries / keys per tile
+constexpr float kFix = 16777216.0f;   // 2^24 fixed point of the histogram
+
+// LDS operations of one wavefront execute in order; this only stops the compiler from moving
+// LDS accesses across the point where lanes exchange data (global loads stay free to move).
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+
+template <int D> struct Frag;
+template <> struct Frag<8> {
+    typedef h4 type;
+    static __device__ __forceinline__ f16v mfma(h4 a, h4 b, f16v c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x8f16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Frag<16> {
+    typedef h8 type;
+    static __device__ __forceinline__ f16v mfma(h8 a, h8 b, f16v c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// channels [ (D/2)*half, (D/2)*half + D/2 ) of one (row, head): what a lane feeds to the MFMA
+template <int D>
+__device__ __forceinline__ typename Frag<D>::type load_frag(const _Float16 *row_head, int half)
+{
+    return *reinterpret_cast<const typename Frag<D>::type *>(row_head + (D / 2) * half);
+}
+
+__device__ __forceinline__ int crse_row(float ci, float cj, int rows)
+{
+    float rel = ci - cj;
+    rel = rel + static_cast<float>(rows / 2);
+    rel = fminf(fmaxf(rel, 0.0f), static_cast<float>(rows));
+    return min(static_cast<int>(rel), rows - 1);
+}
+
+// key index held by accumulator register v of a lane in half-wave `half`
+__device__ __forceinline__ constexpr int key_of(int v, int half) { return 8 * (v / 4) + 4 * half + (v % 4); }
+
+// RMAX: rows of the largest axis table rounded up to 16 (32, 48 or 64)
+template <int RMAX> struct WaveLds {
+    static constexpr int kTiles = (RMAX + kTile - 1) / kTile;  // 32-row MFMA tiles per axis table
+    static constexpr int kQtRows = RMAX;                       // QT / H rows kept in LDS
+    static constexpr int kKtStride = RMAX + 4;                 // words per key row of KT
+    static constexpr int kCrd = kTile * kMaxAxes;
+    static constexpr int kQt = kQtRows * kTile;                // QT[row][query], reused as H[row][query]
+    static constexpr int kKt = kTile * kKtStride;
+    static constexpr int kVt = kTile * 16 / 2;                 // V tile [key][D] in halves
+    static constexpr int kWords = kCrd + kQt + kKt + kVt;
+};
+
+template <int D, int ND, int RMAX>
+__global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
+{
+    extern __shared__ float smem[];
+    typedef typename Frag<D>::type frag_t;
+    typedef WaveLds<RMAX> L;
+    constexpr int kIdxWords = (16 * ND + 3) / 4;
+    constexpr int kOut = D / 2;   // output channels a lane keeps for its query
+
+    const int H = a.H;
+    const int HD = H * D;
+    const int prow = a.padded_rows;
+
+    // transposed value table of all heads -> LDS: tvt[(h*D + c)*prow + padded row]
+    _Float16 *tvt = reinterpret_cast<_Float16 *>(smem);
+    {
+        const h8 *src = static_cast<const h8 *>(a.workspace);
+        h8 *dst = reinterpret_cast<h8 *>(smem);
+        const int chunks = HD * prow / 8;   // prow is a multiple of 16
+        for (int t = threadIdx.x; t < chunks; t += kWaves * 64) dst[t] = src[t];
+    }
+    __syncthreads();   // the only workgroup barrier; every wavefront reaches it
+    const int tvt_words = HD * prow / 2;
+
+    // the wavefront index is uniform: tell the compiler, so that everything derived from the
+    // work item (sizes, tile counts, loop bounds) lives in scalar registers and branches are scalar
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int il = lane & 31;
+    const int half = lane >> 5;
+
+    float *crd_k = smem + (tvt_words + 3) / 4 * 4 + wave * L::kWords;   // [32][ND]
+    float *qt = crd_k + L::kCrd;                                          // [kQtRows][32]
+    unsigned int *hist = reinterpret_cast<unsigned int *>(qt);
+    float *kt = qt + L::kQt;                                              // [32][kKtStride]
+    _Float16 *vt = reinterpret_cast<_Float16 *>(kt + L::kKt);             // [32][D]
+
+    const _Float16 *gq = static_cast<const _Float16 *>(a.q);
+    const _Float16 *gk = static_cast<const _Float16 *>(a.k);
+    const _Float16 *gv = static_cast<const _Float16 *>(a.v);
+    const _Float16 *gtq = static_cast<const _Float16 *>(a.table_q);
+    const _Float16 *gtk = static_cast<const _Float16 *>(a.table_k);
+    _Float16 *gout = static_cast<_Float16 *>(a.out);
+
+    const int *item_end = static_cast<const int *>(a.items);   // inclusive prefix of items per window
+    const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]);
+    const int total_waves = gridDim.x * kWaves;
+
+    const int cc = min(il, D - 1);               // channel this lane feeds to the value MFMAs
+    const bool c_valid = il < D;
+    // per-lane bases such that key slot v sits at a compile-time offset: key_of(v, half) =
+    // key_of(v, 0) + 4*half
+    const float *kt_lane = kt + 4 * half * L::kKtStride;
+    const _Float16 *vt_lane = vt + 4 * half * D + cc;
+
+    f16v zero16;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) zero16[v] = 0.0f;
+
+    for (int item = blockIdx.x * kWaves + wave; item < total_items; item += total_waves) {
+        // window of this item: first w with item_end[w] > item
+        int lo = 0, hi = static_cast<int>(a.W) - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (__builtin_amdgcn_readfirstlane(item_end[mid]) > item) hi = mid; else lo = mid + 1;
+        }
+        const int w = lo;
+        const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
+        const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
+        const int nkt = (n_w + kTile - 1) / kTile;   // key tiles (= query tiles)
+        const bool single_key_tile = nkt == 1;
+        // a single-tile window is one item (all heads, row indices cached across heads);
+        // a larger window is split into (query tile, head) items
+        const int local = item - (w > 0 ? __builtin_amdgcn_readfirstlane(item_end[w - 1]) : 0);
+        const int q0 = single_key_tile ? 0 : (local / H) * kTile;
+        const int h_first = single_key_tile ? 0 : local % H;
+        const int h_count = single_key_tile ? H : 1;
+        const int steps = h_count * nkt;             // (head, key tile) steps of this item
+
+        const bool q_valid = q0 + il < n_w;
+        const int q_pos = s0 + min(q0 + il, n_w - 1);   // lanes past the window repeat the last voxel
+        const int q_row = a.n2n[q_pos];
+        float ci[ND];
+#pragma unroll
+        for (int n = 0; n < ND; ++n) ci[n] = a.n_coords[static_cast<int64_t>(q_pos) * ND + n];
+
+        uint32_t idx[kIdxWords];
+
+        // stage the key coordinates of a key tile and derive the row indices of all pairs
+        auto build_pair_rows = [&](int k0, int nk) {
+            wave_lds_fence();
+            for (int t = lane; t < kTile * ND; t += 64) {
+                const int j = t / ND, n = t - j * ND;
+                crd_k[t] = a.n_coords[static_cast<int64_t>(s0 + k0 + min(j, nk - 1)) * ND + n];
+            }
+            wave_lds_fence();
+#pragma unroll
+            for (int t = 0; t < kIdxWords; ++t) idx[t] = 0;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int j = key_of(v, half);
+#pragma unroll
+                for (int n = 0; n < ND; ++n) {
+                    const int r = crse_row(ci[n], crd_k[j * ND + n], a.rows[n]);
+                    idx[(v * ND + n) >> 2] |= static_cast<uint32_t>(r) << (8 * ((v * ND + n) & 3));
+                }
+            }
+        };
+        if (single_key_tile) build_pair_rows(0, n_w);
+
+        // fragments of the step ahead (head h, key tile kt): issued one step early
+        frag_t qf_next, kf_next;
+        h8 vv_next;
+        auto prefetch_step = [&](int hh, int kk) {
+            const int k0 = kk * kTile;
+            const int nk = min(kTile, n_w - k0);
+            const int k_row = a.n2n[s0 + k0 + min(il, nk - 1)];
+            qf_next = load_frag<D>(gq + static_cast<int64_t>(q_row) * HD + hh * D, half);
+            kf_next = load_frag<D>(gk + static_cast<int64_t>(k_row) * HD + hh * D, half);
+            vv_next = *reinterpret_cast<const h8 *>(gv + static_cast<int64_t>(k_row) * HD + hh * D +
+                                                    (D == 16 ? 8 * half : 0));
+        };
+        prefetch_step(h_first, 0);
+
+        float m_run = -INFINITY, l_run = 0.0f;
+        float o_run[kOut];
+#pragma unroll
+        for (int t = 0; t < kOut; ++t) o_run[t] = 0.0f;
+        int h = h_first, kt_i = 0;
+        for (int step = 0; step < steps; ++step) {
+            const int k0 = kt_i * kTile;
+            const int nk = min(kTile, n_w - k0);
+            const frag_t qf = qf_next, kf = kf_next;
+            const h8 vv = vv_next;
+            if (kt_i == 0) {
+                m_run = -INFINITY;
+                l_run = 0.0f;
+#pragma unroll
+                for (int t = 0; t < kOut; ++t) o_run[t] = 0.0f;
+            }
+            // first axis' table fragments for this head, then the next step's q/k/v
+            frag_t tq_cur[L::kTiles], tk_cur[L::kTiles];
+            auto load_axis = [&](int n, frag_t *tq_dst, frag_t *tk_dst) {
+                const int rows = a.rows[n];
+#pragma unroll
+                for (int t = 0; t < L::kTiles; ++t) {
+                    const int trow = a.base[n] + min(kTile * t + il, rows - 1);
+                    tq_dst[t] = load_frag<D>(gtq + static_cast<int64_t>(trow) * HD + h * D, half);
+                    tk_dst[t] = load_frag<D>(gtk + static_cast<int64_t>(trow) * HD + h * D, half);
+                }
+            };
+            load_axis(0, tq_cur, tk_cur);
+            {
+                int hn = h, ktn = kt_i + 1;
+                if (ktn == nkt) {
+                    ktn = 0;
+                    ++hn;
+                }
+                if (step + 1 < steps) prefetch_step(hn, ktn);
+            }
+
+            if (!single_key_tile) build_pair_rows(k0, nk);
+
+            // V tile -> LDS, [key][D] halves
+            wave_lds_fence();
+            if (half * 8 < D) *reinterpret_cast<h8 *>(vt + il * D + 8 * half) = vv;
+
+            // logits: S^T[j][i] = sum_c K[j][c] Q[i][c]; copied out of the MFMA accumulator so that
+            // the per-axis updates below are plain VALU adds on VGPRs
+            float lg[16];
+            {
+                const f16v s_acc = Frag<D>::mfma(kf, qf, zero16);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    lg[v] = s_acc[v];
+                    asm volatile("" : "+v"(lg[v]));   // one VGPR each, not a 16-register tuple
+                }
+            }
+
+#pragma unroll
+            for (int n = 0; n < ND; ++n) {
+                if (a.debug_skip & 1) break;
+                frag_t tq_nxt[L::kTiles], tk_nxt[L::kTiles];
+                if (n + 1 < ND) load_axis(n + 1, tq_nxt, tk_nxt);
+                const int tiles = (a.rows[n] + kTile - 1) / kTile;
+#pragma unroll
+                for (int t = 0; t < L::kTiles; ++t) {
+                    if (t < tiles) {
+                        const f16v dq = Frag<D>::mfma(tq_cur[t], qf, zero16);   // QT[r][i]
+                        const f16v dk = Frag<D>::mfma(tk_cur[t], kf, zero16);   // KT[r][j]
+                        // registers 4g..4g+3 hold rows 32t + 8g + 4*half + (0..3); rows >= RMAX are not kept
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (kTile * t + 8 * (v / 4) + 8 <= RMAX)
+                                qt[(kTile * t + key_of(v, half)) * kTile + il] = dq[v];
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            if (kTile * t + 8 * g + 8 <= RMAX) {
+                                f4 x = {dk[4 * g], dk[4 * g + 1], dk[4 * g + 2], dk[4 * g + 3]};
+                                *reinterpret_cast<f4 *>(kt + il * L::kKtStride + kTile * t + 8 * g + 4 * half) = x;
+                            }
+                        }
+                    }
+                }
+                wave_lds_fence();
+                // straight-line over all 16 key slots: slots past the end of the tile read
+                // staged duplicates of the last key and get weight 0 below
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = (idx[(v * ND + n) >> 2] >> (8 * ((v * ND + n) & 3))) & 0xff;
+                    lg[v] += qt[r * kTile + il] + kt_lane[key_of(v, 0) * L::kKtStride + r];
+                }
+                // pin the sums here: without it the scheduler keeps the gathered values of all
+                // axes alive and adds them after the last axis (hundreds of spilled registers)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(lg[v]));
+                wave_lds_fence();
+                if (n + 1 < ND) {
+#pragma unroll
+                    for (int t = 0; t < L::kTiles; ++t) {
+                        tq_cur[t] = tq_nxt[t];
+                        tk_cur[t] = tk_nxt[t];
+                    }
+                }
+            }
+
+            // online softmax over this key tile
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (key_of(v, half) < nk) mx = fmaxf(mx, lg[v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            const float scale = __expf(m_run - m_new);
+            float p[16];
+            float psum = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                p[v] = (key_of(v, half) < nk) ? __expf(lg[v] - m_new) : 0.0f;
+                psum += p[v];
+            }
+            psum += __shfl_xor(psum, 32);
+            l_run = l_run * scale + psum;
+            m_run = m_new;
+            // 2^-24 fixed-point image of the weights for the integer histogram (0 for dead slots)
+            unsigned int pfix[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) pfix[v] = static_cast<unsigned int>(p[v] * kFix + 0.5f);
+
+            // value side: acc[c][i], c = 8*(v/4) + 4*half + v%4
+            f16v acc = zero16;
+#pragma unroll
+            for (int t = 0; t < kOut; ++t) acc[t] = o_run[t] * scale;
+
+            wave_lds_fence();   // V tile written above is visible to every lane
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {   // 16 keys per MFMA: element e <-> key key_of(8b + e, half)
+                h8 vf, pf;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const _Float16 x = vt_lane[key_of(8 * b + e, 0) * D];
+                    vf[e] = c_valid ? x : static_cast<_Float16>(0.0f);
+                    pf[e] = static_cast<_Float16>(p[8 * b + e]);
+                }
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, acc, 0, 0, 0);
+            }
+
+            const _Float16 *tvt_row = tvt + (h * D + cc) * prow;
+#pragma unroll
+            for (int n = 0; n < ND; ++n) {
+                if (a.debug_skip & 2) break;
+                const int rows16 = (a.rows[n] + 15) / 16;
+                // clear H_n
+                for (int t = lane; t < rows16 * 16 * kTile / 4; t += 64) {
+                    f4 z = {0.0f, 0.0f, 0.0f, 0.0f};
+                    *reinterpret_cast<f4 *>(qt + 4 * t) = z;
+                }
+                wave_lds_fence();
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int r = (idx[(v * ND + n) >> 2] >> (8 * ((v * ND + n) & 3))) & 0xff;
+                    atomicAdd(hist + r * kTile + il, pfix[v]);
+                }
+                wave_lds_fence();
+                for (int b = 0; b < rows16; ++b) {
+                    h8 hf;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        hf[e] = static_cast<_Float16>(
+                            static_cast<float>(hist[(16 * b + 8 * half + e) * kTile + il]) * (1.0f / kFix));
+                    h8 tf = *reinterpret_cast<const h8 *>(tvt_row + a.pbase[n] + 16 * b + 8 * half);
+                    if (!c_valid) tf = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(tf, hf, acc, 0, 0, 0);
+                }
+                wave_lds_fence();
+            }
+#pragma unroll
+            for (int t = 0; t < kOut; ++t) o_run[t] = acc[t];
+
+            if (kt_i == nkt - 1 && q_valid) {
+                const float inv = 1.0f / l_run;
+                _Float16 *orow = gout + static_cast<int64_t>(q_row) * HD + h * D;
+#pragma unroll
+                for (int g = 0; g < D / 8; ++g) {   // registers 4g..4g+3 hold channels 8g + 4*half + e
+                    h4 ov;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ov[e] = static_cast<_Float16>(o_run[4 * g + e] * inv);
+                    *reinterpret_cast<h4 *>(orow + 8 * g + 4 * half) = ov;
+                }
+                if (half == 0) {
+                    if (a.out_max) a.out_max[static_cast<int64_t>(q_row) * H + h] = m_run;
+                    if (a.out_sum) a.out_sum[static_cast<int64_t>(q_row) * H + h] = l_run;
+                }
+            }
+            if (++kt_i == nkt) {
+                kt_i = 0;
+                ++h;
+            }
+        }
+    }
+}
+
+// value table [axis][row][h][c] -> [h][c][padded row], every axis padded to a multiple of 16 rows
+__global__ void transpose_value_table_kernel(AttnArgs a)
+{
+    const int HD = a.H * a.D;
+    _Float16 *dst = static_cast<_Float16 *>(a.workspace);
+    const _Float16 *src = static_cast<const _Float16 *>(a.table_v);
+    const int64_t total = static_cast<int64_t>(HD) * a.padded_rows;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
+         t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int hc = static_cast<int>(t / a.padded_rows);
+        const int pr = static_cast<int>(t - static_cast<int64_t>(hc) * a.padded_rows);
+        _Float16 val = static_cast<_Float16>(0.0f);
+        for (int n = 0; n < a.nd; ++n) {
+            const int r = pr - a.pbase[n];
+            if (r >= 0 && r < a.rows[n]) val = src[static_cast<int64_t>(a.base[n] + r) * HD + hc];
+        }
+        dst[t] = val;
+    }
+}
+
+// inclusive prefix sum of the work items of every window: 1 for a window of at most 32 voxels,
+// (query tiles x heads) for a larger one.  One workgroup; W is at most a few hundred thousand.
+__global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
+{
+    __shared__ int part[1024];
+    int *item_end = static_cast<int *>(a.items);
+    const int W = static_cast<int>(a.W);
+    const int per = (W + 1023) / 1024;
+    const int begin = threadIdx.x * per, end = min(begin + per, W);
+    int sum = 0;
+    for (int w = begin; w < end; ++w) {
+        const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
+        sum += tiles <= 1 ? 1 : tiles * a.H;
+    }
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+        __syncthreads();
+        part[threadIdx.x] += add;
+        __syncthreads();
+    }
+    int run = part[threadIdx.x] - sum;
+    for (int w = begin; w < end; ++w) {
+        const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
+        run += tiles <= 1 ? 1 : tiles * a.H;
+        item_end[w] = run;
+    }
+}
+
+size_t lds_bytes(const AttnArgs &a, int wave_words)
+{
+    const size_t tvt_words = static_cast<size_t>(a.H) * a.D * a.padded_rows / 2;
+    return sizeof(float) * ((tvt_words + 3) / 4 * 4 + static_cast<size_t>(kWaves) * wave_words);
+}
+
+template <int D, int ND, int RMAX>
+int launch(const AttnArgs &a, hipStream_t stream)
+{
+    auto kernel = attn_fwd_mfma_kernel<D, ND, RMAX>;
+    const size_t lds = lds_bytes(a, WaveLds<RMAX>::kWords);
+    S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    const int64_t cells = static_cast<int64_t>(a.H) * a.D * a.padded_rows;
+    hipLaunchKernelGGL(transpose_value_table_kernel, dim3(static_cast<unsigned>(ceil_div(cells, 256))),
+                       dim3(256), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(window_items_kernel, dim3(1), dim3(1024), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    // persistent grid: as many workgroups as fit the chip at once (LDS-bound), never more than the
+    // windows can feed; wavefronts pull items in a strided loop
+    int device = 0, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
+    }
+    const int per_cu = static_cast<int>((160 * 1024) / lds) > 0 ? static_cast<int>((160 * 1024) / lds) : 1;
+    int64_t grid = static_cast<int64_t>(cus) * per_cu;
+    const int64_t need = ceil_div(a.W, kWaves);
+    if (grid > need) grid = need;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kWaves * 64), lds, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+int max_axis_rows(const AttnArgs &a)
+{
+    int m = 0;
+    for (int n = 0; n < a.nd; ++n) m = a.rows[n] > m ? a.rows[n] : m;
+    return m;
+}
+
+}  // namespace
+
+int attn_mfma_padded_rows(const int32_t *rows, int nd)
+{
+    int padded = 16;   // slack so that 16-row reads of the last block stay inside the table
+    for (int n = 0; n < nd; ++n) padded += (rows[n] + 15) / 16 * 16;
+    return padded;
+}
+
+bool attn_mfma_supported(const AttnArgs &a, int dtype)
+{
+    if (dtype != S3D_DTYPE_F16) return false;
+    if (a.D != 8 && a.D != 16) return false;
+    if (a.nd != 3 && a.nd != 6 && a.nd != 9) return false;
+    const int rmax = max_axis_rows(a);
+    if (rmax > 64) return false;
+    // the transposed value table of all heads must fit LDS next to the per-wavefront staging
+    const int words = rmax <= 32 ? WaveLds<32>::kWords : rmax <= 48 ? WaveLds<48>::kWords : WaveLds<64>::kWords;
+    return lds_bytes(a, words) <= 160 * 1024;
+}
+
+size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
+{
+    return align_up(sizeof(_Float16) * static_cast<size_t>(H) * D * padded_rows, 256);
+}
+
+size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W)
+{
+    return attn_mfma_table_bytes(H, D, padded_rows) + align_up(sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1), 256);
+}
+
+int launch_attn_mfma(const AttnArgs &a, hipStream_t stream)
+{
+    const int rmax = max_axis_rows(a);
+#define S3D_CASE(DD, NN)                                                         \
+    if (a.D == DD && a.nd == NN)                                                 \
+        return rmax <= 32   ? launch<DD, NN, 32>(a, stream)                      \
+               : rmax <= 48 ? launch<DD, NN, 48>(a, stream)                      \
+                            : launch<DD, NN, 64>(a, stream);
+    S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
+    S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
+#undef S3D_CASE
+    return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: MFMA kernel does not cover D=%d nd=%d", a.D, a.nd);
+}
+
+}  // namespace s3d

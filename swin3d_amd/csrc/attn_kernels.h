@@ -1,0 +1,38 @@
+// Internal interface between the attention entry point and its kernel families.
+#pragma once
+
+#include "s3d_common.h"
+
+namespace s3d {
+
+constexpr int kMaxAxes = 9;
+
+// Everything a window-attention kernel needs, by value (lives in kernel-argument SGPRs).
+struct AttnArgs {
+    const void *q, *k, *v;                 // [N,H,D]
+    const void *table_q, *table_k, *table_v;  // flat [sum rows][H][D]
+    const int32_t *w_sizes, *w2n, *n2n;
+    const float *n_coords;                 // [N,nd], window-sorted
+    void *out;                             // [N,H,D]
+    float *out_max, *out_sum;              // [N,H] or null
+    void *workspace;                       // transposed value table (MFMA path) or null
+    void *items;                           // int32 [W] work-item prefix (MFMA path) or null
+    int32_t H, D, nd, total_rows;
+    int64_t N, W;
+    int32_t rows[kMaxAxes];                // rows of each axis table
+    int32_t base[kMaxAxes];                // first row of each axis table in the flat table
+    int32_t pbase[kMaxAxes];               // first row of each axis in the padded transposed table
+    int32_t padded_rows;                   // row stride of the transposed value table
+    int32_t debug_skip;                    // TEMP ablation bits
+};
+
+// One workgroup per (window, head), tables of the head in LDS, VALU math; any dtype.
+int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
+
+// One wavefront per window, MFMA products + LDS gathers; fp16 only.
+bool attn_mfma_supported(const AttnArgs &a, int dtype);
+size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
+size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W);
+int launch_attn_mfma(const AttnArgs &a, hipStream_t stream);
+
+}  // namespace s3d

@@ -8,6 +8,7 @@ can call it unchanged.  Differences in mechanism, not in result:
   * only the combination the model uses is implemented (PosEmb.SEPARATE, TableDims.D0,
     IndexMode.INDIRECT); the backward pass is not implemented yet.
 """
+import ctypes
 import enum
 
 import torch
@@ -66,17 +67,27 @@ def _as_int32(name, t, device):
     return t.to(torch.int32).contiguous()
 
 
+def _host_table_sizes(table_sizes):
+    """The op reads the per-axis table sizes on the host.  A CUDA tensor (what the reference's
+    caller builds on every call) costs one synchronising device-to-host copy here; pass a list
+    or a CPU tensor to avoid it."""
+    if isinstance(table_sizes, torch.Tensor):
+        return [int(x) for x in table_sizes.reshape(-1).tolist()]
+    return [int(x) for x in table_sizes]
+
+
 def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
-                             n_coords, return_stats=False):
+                             n_coords, return_stats=False, force_generic=False):
     """softmax-normalised window attention, [N,H,D] in the dtype of q.
 
     q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5)
     table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
-    table_sizes    int tensor / list [nd], per-axis element counts rows*H*D
+    table_sizes    int tensor / list [nd], per-axis element counts rows*H*D (read on the host)
     w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
     n2n            [N] window-sorted position -> row of q/k/v
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
+    force_generic  run the VALU kernel even where the MFMA kernel applies (fp16)
     """
     _require_cuda("query", q)
     dev = q.device
@@ -91,10 +102,14 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
     if d not in (8, 16):
         raise ValueError(f"head_dim must be 8 or 16, got {d}")
-    table_sizes = _as_int32("table_sizes", table_sizes, dev).reshape(-1)
-    nd = table_sizes.numel()
+    sizes = _host_table_sizes(table_sizes)
+    nd = len(sizes)
     if nd not in (3, 6, 9):
         raise ValueError(f"table_sizes must have 3, 6 or 9 entries, got {nd}")
+    if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_q.numel():
+        raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
+                         f"to the table length {table_q.numel()}")
+    c_sizes = (ctypes.c_int32 * nd)(*sizes)
     table_len = table_q.numel()
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
@@ -118,14 +133,18 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     out = torch.empty_like(q)
     omax = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
+    lib = _lib.lib()
     with torch.cuda.device(dev):
+        ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, w_sizes.numel())
+        workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
-        status = _lib.lib().s3d_attn_fwd(
+        status = lib.s3d_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), table_q.data_ptr(), table_k.data_ptr(),
-            table_v.data_ptr(), table_sizes.data_ptr(), nd, table_len, w_sizes.data_ptr(),
+            table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
             w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
-            n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype], stream)
+            n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype],
+            _lib.S3D_ATTN_FORCE_GENERIC if force_generic else 0, workspace.data_ptr(), ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
     if return_stats:
         return out, omax, osum

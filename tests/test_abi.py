@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_attn_fwd", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+    for must in ("s3d_attn_fwd", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -41,7 +41,7 @@ def test_argument_errors_are_reported_without_a_device(hip_lib):
     status = hip_lib.s3d_knn(0, None, 0, None, 0, None, None, 1, None, None, 0.0, None, 0, None)
     assert status < 0
     assert b"K=0" in hip_lib.s3d_last_error_string()
-    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 1, None)
+    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 1, 0, None, 0, None)
     assert status < 0 and b"table_len" in hip_lib.s3d_last_error_string()
     try:
         _lib.check(status, "s3d_attn_fwd")

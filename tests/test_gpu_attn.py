@@ -16,6 +16,9 @@ def _check(oracle_lib, case, dtype):
     ref = oracle_lib.attn_fwd(*case.oracle_args())
     got = run_attention(case, dtype)
     assert_attn_close(got, ref, dtype)
+    if dtype == torch.float16:
+        # fp16 runs on the MFMA kernel by default; the generic kernel must agree with the oracle too
+        assert_attn_close(run_attention(case, dtype, force_generic=True), ref, dtype)
     return got, ref
 
 
