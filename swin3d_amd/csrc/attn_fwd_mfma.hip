@@ -143,7 +143,9 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 
     const int *item_end = static_cast<const int *>(a.items);   // inclusive prefix of items per window
     const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]);
-    const int total_waves = gridDim.x * kWaves;
+    // work items are handed out through a device counter (zeroed by window_items_kernel), so a
+    // wavefront that drew long items simply draws fewer of them
+    int *next_item = static_cast<int *>(a.items) + a.W;
 
     const int cc = min(il, D - 1);               // channel this lane feeds to the value MFMAs
     const bool c_valid = il < D;
@@ -156,7 +158,11 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 #pragma unroll
     for (int v = 0; v < 16; ++v) zero16[v] = 0.0f;
 
-    for (int item = blockIdx.x * kWaves + wave; item < total_items; item += total_waves) {
+    for (;;) {
+        int item = 0;
+        if (lane == 0) item = atomicAdd(next_item, 1);
+        item = __builtin_amdgcn_readfirstlane(item);
+        if (item >= total_items) break;
         // window of this item: first w with item_end[w] > item
         int lo = 0, hi = static_cast<int>(a.W) - 1;
         while (lo < hi) {
@@ -467,6 +473,7 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
         run += tiles <= 1 ? 1 : tiles * a.H;
         item_end[w] = run;
     }
+    if (threadIdx.x == 0) item_end[W] = 0;   // the work counter of the attention kernel
 }
 
 size_t lds_bytes(const AttnArgs &a, int wave_words)
@@ -539,7 +546,7 @@ size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
 
 size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W)
 {
-    return attn_mfma_table_bytes(H, D, padded_rows) + align_up(sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1), 256);
+    return attn_mfma_table_bytes(H, D, padded_rows) + align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 1), 256);
 }
 
 int launch_attn_mfma(const AttnArgs &a, hipStream_t stream)
