@@ -23,6 +23,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the dominant kernel from the FETCH_SIZE / WRITE_SIZE passes recorded in
+# profiles/attn_fwd_headline.txt: (63130 KiB * 2.00 + 32280 KiB * 1.00), factors from the 64 MiB copy
+MEASURED_TRAFFIC_BYTES = int((63130 * 2.00 + 32280 * 1.00) * 1024)
 
 
 def algorithmic_bytes(n, c, elem_bytes, nd, w, table_len):
@@ -139,9 +142,16 @@ def main():
         "kernel_ms": {"mean": kernel_ms, "median": float(np.median(launch_ms)),
                       "p10": float(np.percentile(launch_ms, 10)), "p90": float(np.percentile(launch_ms, 90))},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES if args.flags == 0 else None,
                      "algorithmic_bytes": bytes_alg},
     }
+
+    # one plain device-to-device copy of known size (64 MiB read + 64 MiB written): the yardstick
+    # that the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled against
+    probe = torch.empty(64 * 1024 * 1024, dtype=torch.uint8, device=dev)
+    torch.empty_like(probe).copy_(probe)
+    torch.cuda.synchronize()
 
     if not args.no_extras:
         result["extras"] = extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev)

@@ -98,7 +98,6 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.out_max = out_max;
     a.out_sum = out_sum;
     a.workspace = workspace;
-    a.debug_skip = flags >> 8;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype);
     if (want_mfma) {

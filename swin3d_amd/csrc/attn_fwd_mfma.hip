@@ -284,7 +284,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 
 #pragma unroll
             for (int n = 0; n < ND; ++n) {
-                if (a.debug_skip & 1) break;
                 frag_t tq_nxt[L::kTiles], tk_nxt[L::kTiles];
                 if (n + 1 < ND) load_axis(n + 1, tq_nxt, tk_nxt);
                 const int tiles = (a.rows[n] + kTile - 1) / kTile;
@@ -373,7 +372,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
             const _Float16 *tvt_row = tvt + (h * D + cc) * prow;
 #pragma unroll
             for (int n = 0; n < ND; ++n) {
-                if (a.debug_skip & 2) break;
                 const int rows16 = (a.rows[n] + 15) / 16;
                 // clear H_n
                 for (int t = lane; t < rows16 * 16 * kTile / 4; t += 64) {

@@ -23,7 +23,6 @@ struct AttnArgs {
     int32_t base[kMaxAxes];                // first row of each axis table in the flat table
     int32_t pbase[kMaxAxes];               // first row of each axis in the padded transposed table
     int32_t padded_rows;                   // row stride of the transposed value table
-    int32_t debug_skip;                    // TEMP ablation bits
 };
 
 // One workgroup per (window, head), tables of the head in LDS, VALU math; any dtype.
