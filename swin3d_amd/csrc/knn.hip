@@ -100,16 +100,24 @@ __global__ __launch_bounds__(kThreads) void knn_init_kernel(KnnPlan *plan, int32
     }
 }
 
+// Bounding box of the sources: a small grid-stride grid so that only a few hundred atomics
+// meet on the six box words (one atomic pair per wavefront and axis).
+constexpr int kBboxBlocks = 64;
+
 __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restrict__ src,
                                                             int64_t Ns, KnnPlan *plan)
 {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     int lo[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
     int hi[3] = {static_cast<int>(0x80000000u), static_cast<int>(0x80000000u),
                  static_cast<int>(0x80000000u)};
-    if (i < Ns) {
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < Ns;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
 #pragma unroll
-        for (int a = 0; a < 3; ++a) lo[a] = hi[a] = float_to_ordered(src[i * 3 + a]);
+        for (int a = 0; a < 3; ++a) {
+            const int o = float_to_ordered(src[i * 3 + a]);
+            lo[a] = min(lo[a], o);
+            hi[a] = max(hi[a], o);
+        }
     }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
@@ -348,34 +356,59 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
         for (int r = r_first; r <= r_last; ++r) {
             const int z0 = max(qc[2] - r, 0), z1 = min(qc[2] + r, plan.dim[2] - 1);
             const int y0 = max(qc[1] - r, 0), y1 = min(qc[1] + r, plan.dim[1] - 1);
-            for (int z = z0; z <= z1; ++z) {
-                const bool z_face = (z == qc[2] - r) || (z == qc[2] + r);
-                for (int y = y0; y <= y1; ++y) {
-                    const bool face = z_face || (y == qc[1] - r) || (y == qc[1] + r);
-                    const int32_t *row = cell_base + (z * plan.dim[1] + y) * plan.dim[0];
-                    // a face row spans the whole x range of the cube, an interior row only its two ends
-                    const int n_runs = (face || r == 0) ? 1 : 2;
-                    for (int run = 0; run < n_runs; ++run) {
-                        int x0, x1;
-                        if (face || r == 0) {
-                            x0 = qc[0] - r;
-                            x1 = qc[0] + r;
-                        } else {
-                            x0 = x1 = (run == 0) ? qc[0] - r : qc[0] + r;
-                        }
-                        x0 = max(x0, 0);
-                        x1 = min(x1, plan.dim[0] - 1);
-                        if (x0 > x1) continue;
-                        const int s_begin = row[x0], s_end = row[x1 + 1];
-                        for (int s = s_begin; s < s_end; ++s) {
-                            const float4 p = sorted[s];
-                            const float d2 = dist2_unfused(p.x, p.y, p.z, qx, qy, qz);
-                            const int si = __float_as_int(p.w);
-                            if (cand_less(d2, si, best.worst_d(K), best.worst_i(K)))
-                                best.insert(d2, si, K);
-                        }
+            const int ny = y1 - y0 + 1;
+            const int n_rows = (z1 - z0 + 1) * ny;   // <= 0 when the shell misses the grid in z or y
+            // source ranges of row t of the shell: a face row spans the whole x range of the cube
+            // (one contiguous run of cells), an interior row only its two end cells
+            auto row_ranges = [&](int t, int &a0, int &a1, int &b0, int &b1) {
+                const int z = z0 + t / ny, y = y0 + t % ny;
+                const bool face = r == 0 || z == qc[2] - r || z == qc[2] + r || y == qc[1] - r ||
+                                  y == qc[1] + r;
+                const int32_t *row = cell_base + (z * plan.dim[1] + y) * plan.dim[0];
+                const int xl = qc[0] - r, xh = qc[0] + r;
+                a0 = a1 = b0 = b1 = 0;
+                if (face) {
+                    const int x0 = max(xl, 0), x1 = min(xh, plan.dim[0] - 1);
+                    if (x0 <= x1) {
+                        a0 = row[x0];
+                        a1 = row[x1 + 1];
+                    }
+                } else {
+                    if (xl >= 0 && xl < plan.dim[0]) {
+                        a0 = row[xl];
+                        a1 = row[xl + 1];
+                    }
+                    if (xh >= 0 && xh < plan.dim[0]) {
+                        b0 = row[xh];
+                        b1 = row[xh + 1];
                     }
                 }
+            };
+            auto scan_sources = [&](int s_begin, int s_end) {
+                for (int s = s_begin; s < s_end; s += 2) {
+                    // two candidates per trip so that their loads are in flight together
+                    const bool two = s + 1 < s_end;
+                    const float4 p0 = sorted[s];
+                    const float4 p1 = sorted[two ? s + 1 : s];
+                    const float d0 = dist2_unfused(p0.x, p0.y, p0.z, qx, qy, qz);
+                    const float d1 = dist2_unfused(p1.x, p1.y, p1.z, qx, qy, qz);
+                    const int i0 = __float_as_int(p0.w), i1 = __float_as_int(p1.w);
+                    if (cand_less(d0, i0, best.worst_d(K), best.worst_i(K))) best.insert(d0, i0, K);
+                    if (two && cand_less(d1, i1, best.worst_d(K), best.worst_i(K))) best.insert(d1, i1, K);
+                }
+            };
+            int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+            if (n_rows > 0) row_ranges(0, a0, a1, b0, b1);
+            for (int t = 0; t < n_rows; ++t) {
+                // the next row's cell bounds are loaded while this row's sources are scanned
+                int na0 = 0, na1 = 0, nb0 = 0, nb1 = 0;
+                if (t + 1 < n_rows) row_ranges(t + 1, na0, na1, nb0, nb1);
+                scan_sources(a0, a1);
+                scan_sources(b0, b1);
+                a0 = na0;
+                a1 = na1;
+                b0 = nb0;
+                b1 = nb1;
             }
             if (best.worst_i(K) != 0x7fffffff) {
                 // everything outside the visited cube is at least `bound` away from the query
@@ -444,7 +477,9 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
     S3D_HIP_CHECK(hipGetLastError());
     if (Ns > 0) {
         const dim3 sgrid(static_cast<unsigned>(ceil_div(Ns, kThreads)));
-        hipLaunchKernelGGL(knn_bbox_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, plan);
+        const int64_t bbox_blocks = ceil_div(Ns, kThreads) < kBboxBlocks ? ceil_div(Ns, kThreads) : kBboxBlocks;
+        hipLaunchKernelGGL(knn_bbox_kernel, dim3(static_cast<unsigned>(bbox_blocks)), dim3(kThreads), 0, s,
+                           src_xyz, Ns, plan);
         S3D_HIP_CHECK(hipGetLastError());
         hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,
                            cell_size, L.cells_cap);
