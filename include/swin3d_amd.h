@@ -91,6 +91,9 @@ const char *s3d_last_error_string(void);
  * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.
  */
 #define S3D_ATTN_FORCE_GENERIC 1
+/* 1 if s3d_attn_fwd runs these shapes on the MFMA kernel (fp16, every axis table <= 64 rows),
+ * 0 if on the generic VALU kernel.  No counterpart in the reference (it has one kernel). */
+int s3d_attn_fwd_uses_mfma(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype);
 size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,
                                     int64_t W);
 int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_q,

@@ -62,6 +62,21 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
     return attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W);
 }
 
+extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
+    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype)
+{
+    using namespace s3d;
+    if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1) return 0;
+    AttnArgs a{};
+    a.H = H;
+    a.D = D;
+    a.nd = nd;
+    int64_t total = 0;
+    for (int n = 0; n < nd; ++n) total += table_sizes[n];
+    if (fill_axes(a, table_sizes, nd, total) != S3D_OK) return 0;
+    return attn_mfma_supported(a, dtype) ? 1 : 0;
+}
+
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
     const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,

@@ -97,7 +97,9 @@ template <int RMAX> struct WaveLds {
     static constexpr int kWords = kCrd + kQt + kKt + kVt;
 };
 
-template <int D, int ND, int RMAX>
+// TVT_LDS: the transposed value table of all heads is staged in LDS (it must fit next to the
+// per-wavefront staging); otherwise its fragments are read from the L2-resident workspace copy.
+template <int D, int ND, int RMAX, bool TVT_LDS>
 __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 {
     extern __shared__ float smem[];
@@ -110,16 +112,16 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
     const int HD = H * D;
     const int prow = a.padded_rows;
 
-    // transposed value table of all heads -> LDS: tvt[(h*D + c)*prow + padded row]
-    _Float16 *tvt = reinterpret_cast<_Float16 *>(smem);
-    {
+    // transposed value table of all heads: tvt[(h*D + c)*prow + padded row]
+    int tvt_words = 0;
+    if constexpr (TVT_LDS) {
         const h8 *src = static_cast<const h8 *>(a.workspace);
         h8 *dst = reinterpret_cast<h8 *>(smem);
         const int chunks = HD * prow / 8;   // prow is a multiple of 16
         for (int t = threadIdx.x; t < chunks; t += kWaves * 64) dst[t] = src[t];
+        __syncthreads();   // the only workgroup barrier; every wavefront reaches it
+        tvt_words = HD * prow / 2;
     }
-    __syncthreads();   // the only workgroup barrier; every wavefront reaches it
-    const int tvt_words = HD * prow / 2;
 
     // the wavefront index is uniform: tell the compiler, so that everything derived from the
     // work item (sizes, tile counts, loop bounds) lives in scalar registers and branches are scalar
@@ -369,10 +371,25 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, acc, 0, 0, 0);
             }
 
-            const _Float16 *tvt_row = tvt + (h * D + cc) * prow;
+            const _Float16 *tvt_row;
+            if constexpr (TVT_LDS)
+                tvt_row = reinterpret_cast<const _Float16 *>(smem) + (h * D + cc) * prow;
+            else
+                tvt_row = static_cast<const _Float16 *>(a.workspace) + static_cast<int64_t>(h * D + cc) * prow;
 #pragma unroll
             for (int n = 0; n < ND; ++n) {
                 const int rows16 = (a.rows[n] + 15) / 16;
+                // global copy of the value table: fetch this axis' fragments now, their latency hides
+                // behind the histogram; the LDS copy is read right before each MFMA instead
+                h8 tf[RMAX / 16];
+                if constexpr (!TVT_LDS) {
+#pragma unroll
+                    for (int b = 0; b < RMAX / 16; ++b) {
+                        tf[b] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                        if (b < rows16 && c_valid)
+                            tf[b] = *reinterpret_cast<const h8 *>(tvt_row + a.pbase[n] + 16 * b + 8 * half);
+                    }
+                }
                 // clear H_n
                 for (int t = lane; t < rows16 * 16 * kTile / 4; t += 64) {
                     f4 z = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -385,15 +402,25 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                     atomicAdd(hist + r * kTile + il, pfix[v]);
                 }
                 wave_lds_fence();
-                for (int b = 0; b < rows16; ++b) {
+                auto hist_frag = [&](int b) {
                     h8 hf;
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
                         hf[e] = static_cast<_Float16>(
                             static_cast<float>(hist[(16 * b + 8 * half + e) * kTile + il]) * (1.0f / kFix));
-                    h8 tf = *reinterpret_cast<const h8 *>(tvt_row + a.pbase[n] + 16 * b + 8 * half);
-                    if (!c_valid) tf = h8{0, 0, 0, 0, 0, 0, 0, 0};
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(tf, hf, acc, 0, 0, 0);
+                    return hf;
+                };
+                if constexpr (TVT_LDS) {
+                    for (int b = 0; b < rows16; ++b) {
+                        h8 t = *reinterpret_cast<const h8 *>(tvt_row + a.pbase[n] + 16 * b + 8 * half);
+                        if (!c_valid) t = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(t, hist_frag(b), acc, 0, 0, 0);
+                    }
+                } else {
+#pragma unroll
+                    for (int b = 0; b < RMAX / 16; ++b)
+                        if (b < rows16)
+                            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(tf[b], hist_frag(b), acc, 0, 0, 0);
                 }
                 wave_lds_fence();
             }
@@ -474,17 +501,19 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
     if (threadIdx.x == 0) item_end[W] = 0;   // the work counter of the attention kernel
 }
 
-size_t lds_bytes(const AttnArgs &a, int wave_words)
+size_t lds_bytes(const AttnArgs &a, int wave_words, bool tvt_lds)
 {
-    const size_t tvt_words = static_cast<size_t>(a.H) * a.D * a.padded_rows / 2;
+    const size_t tvt_words = tvt_lds ? static_cast<size_t>(a.H) * a.D * a.padded_rows / 2 : 0;
     return sizeof(float) * ((tvt_words + 3) / 4 * 4 + static_cast<size_t>(kWaves) * wave_words);
 }
 
-template <int D, int ND, int RMAX>
+constexpr size_t kLdsPerCu = 160 * 1024;
+
+template <int D, int ND, int RMAX, bool TVT_LDS>
 int launch(const AttnArgs &a, hipStream_t stream)
 {
-    auto kernel = attn_fwd_mfma_kernel<D, ND, RMAX>;
-    const size_t lds = lds_bytes(a, WaveLds<RMAX>::kWords);
+    auto kernel = attn_fwd_mfma_kernel<D, ND, RMAX, TVT_LDS>;
+    const size_t lds = lds_bytes(a, WaveLds<RMAX>::kWords, TVT_LDS);
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     const int64_t cells = static_cast<int64_t>(a.H) * a.D * a.padded_rows;
@@ -500,7 +529,7 @@ int launch(const AttnArgs &a, hipStream_t stream)
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
     }
-    const int per_cu = static_cast<int>((160 * 1024) / lds) > 0 ? static_cast<int>((160 * 1024) / lds) : 1;
+    const int per_cu = kLdsPerCu / lds > 0 ? static_cast<int>(kLdsPerCu / lds) : 1;
     int64_t grid = static_cast<int64_t>(cus) * per_cu;
     const int64_t need = ceil_div(a.W, kWaves);
     if (grid > need) grid = need;
@@ -532,9 +561,7 @@ bool attn_mfma_supported(const AttnArgs &a, int dtype)
     if (a.nd != 3 && a.nd != 6 && a.nd != 9) return false;
     const int rmax = max_axis_rows(a);
     if (rmax > 64) return false;
-    // the transposed value table of all heads must fit LDS next to the per-wavefront staging
-    const int words = rmax <= 32 ? WaveLds<32>::kWords : rmax <= 48 ? WaveLds<48>::kWords : WaveLds<64>::kWords;
-    return lds_bytes(a, words) <= 160 * 1024;
+    return true;
 }
 
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
@@ -550,14 +577,20 @@ size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W)
 int launch_attn_mfma(const AttnArgs &a, hipStream_t stream)
 {
     const int rmax = max_axis_rows(a);
+    const int words = rmax <= 32 ? WaveLds<32>::kWords : rmax <= 48 ? WaveLds<48>::kWords : WaveLds<64>::kWords;
+    const bool tvt_lds = lds_bytes(a, words, true) <= kLdsPerCu;
+#define S3D_RMAX(DD, NN, LDS)                                                    \
+    return rmax <= 32   ? launch<DD, NN, 32, LDS>(a, stream)                     \
+           : rmax <= 48 ? launch<DD, NN, 48, LDS>(a, stream)                     \
+                        : launch<DD, NN, 64, LDS>(a, stream);
 #define S3D_CASE(DD, NN)                                                         \
-    if (a.D == DD && a.nd == NN)                                                 \
-        return rmax <= 32   ? launch<DD, NN, 32>(a, stream)                      \
-               : rmax <= 48 ? launch<DD, NN, 48>(a, stream)                      \
-                            : launch<DD, NN, 64>(a, stream);
+    if (a.D == DD && a.nd == NN) {                                               \
+        if (tvt_lds) { S3D_RMAX(DD, NN, true) } else { S3D_RMAX(DD, NN, false) } \
+    }
     S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
     S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
 #undef S3D_CASE
+#undef S3D_RMAX
     return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: MFMA kernel does not cover D=%d nd=%d", a.D, a.nd);
 }
 

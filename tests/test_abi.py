@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_attn_fwd", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+    for must in ("s3d_attn_fwd", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -49,3 +49,17 @@ def test_argument_errors_are_reported_without_a_device(hip_lib):
         assert "s3d_attn_fwd failed" in str(e)
     else:
         raise AssertionError("check() must raise on a negative status")
+
+
+def test_kernel_choice_is_reported(hip_lib):
+    """fp16 Swin3D shapes (S and L, all stages) go to the MFMA kernel, fp32 to the generic one."""
+    import ctypes
+    from swin3d_amd import crse
+    for ws, heads, dim in [(5, 6, 8), (7, 6, 16), (7, 12, 16), (7, 24, 16), (5, 10, 8), (7, 40, 16)]:
+        sizes = crse.crse_table_sizes(ws, 4, heads, dim, "XYZ_RGB_NORM")
+        c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
+        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1) == 1
+        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 0) == 0
+    sizes = crse.crse_table_sizes(10, 4, 6, 8, "XYZ")          # 80-row tables: generic kernel
+    c_sizes = (ctypes.c_int32 * 3)(*sizes)
+    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, 3, 6, 8, 1) == 0

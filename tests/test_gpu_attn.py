@@ -178,3 +178,58 @@ def test_headline_size_properties(oracle_lib, hip_lib):
     assert np.abs(const - 0.5).max() <= 1e-3
     # (c) the output is a convex combination: inside [min, max] of (v + Tv) bounds
     assert got.min() >= -5 and got.max() <= 5
+
+
+def _sampled_parity(oracle_lib, case, got, dtype, n_windows, seed=0):
+    """oracle parity on a random sample of whole windows (the op ran on the full scene)."""
+    from gpu_helpers import assert_attn_close
+    rng = np.random.default_rng(seed)
+    idx = case.index
+    pick = np.sort(rng.choice(idx["W"], size=min(n_windows, idx["W"]), replace=False))
+    pos = np.concatenate([np.arange(idx["w2n"][w], idx["w2n"][w] + idx["w_sizes"][w]) for w in pick])
+    rows = idx["n2n"][pos]
+    sub_sizes = idx["w_sizes"][pick]
+    sub = oracle_lib.attn_fwd(case.q[rows], case.k[rows], case.v[rows], case.tq, case.tk, case.tv,
+                              case.table_sizes, sub_sizes, np.cumsum(sub_sizes) - sub_sizes,
+                              np.arange(rows.shape[0], dtype=np.int32), case.n_coords[pos])
+    assert_attn_close(got[rows], sub, dtype)
+
+
+@pytest.mark.parametrize("stage,heads,levels", [(2, 6, 1), (3, 12, 2), (4, 24, 3)])
+def test_deeper_stages_config3(oracle_lib, hip_lib, stage, heads, levels):
+    """Swin3D-S stages 2-4 (config 3): fp16, window 7, head_dim 16, 9 axes, the headline room
+    grid-downsampled by 2 per stage (tensor stride 2, 4, 8); shifted windows on stage 3."""
+    from gpu_helpers import run_attention
+    scene = synth.make_room((10, 8, 3), 30, 200_000, seed=0)
+    stride = 1
+    for _ in range(levels):
+        scene, _ = synth.grid_downsample(scene, 2 * stride)
+        stride *= 2
+    frac = ((scene.xyz - scene.coords[:, 1:]) / np.float32(stride)).astype(np.float32)
+    frac = np.clip(frac, 0.0, np.float32(1.0 - 2.0 ** -24))
+    sig = synth.signals(scene, "XYZ_RGB_NORM")
+    shift = 3 if stage == 3 else 0
+    index, n_coords = n_coords_from_scene(oracle_lib, scene.coords, frac, sig, stride, 7, 4, "XYZ_RGB_NORM", shift)
+    case = make_attn_case(oracle_lib, seed=stage, n=64, ws=7, quant=4, heads=heads, dim=16, extent=(4, 4, 2))
+    n = scene.coords.shape[0]
+    q, k, v, tables = synth.layer_inputs(n, heads * 16, heads, int(case.table_sizes.sum()), seed=stage, recipe="sharp")
+    case.coords, case.stride, case.index, case.n_coords = scene.coords, stride, index, n_coords
+    case.q, case.k, case.v = q, k, v
+    case.tq, case.tk, case.tv = tables
+    _sharp16(case)
+    to_half_and_back(case)
+    got = run_attention(case, torch.float16)
+    assert index["w_sizes"].max() > 32           # several key tiles per window
+    _sampled_parity(oracle_lib, case, got, torch.float16, 150)
+
+
+def test_swin3d_l_stage1_shape(oracle_lib, hip_lib):
+    """Swin3D-L stage 1 (config 5): 10 heads x 8, window 5, two scenes in one batch."""
+    from gpu_helpers import run_attention
+    a = synth.make_room((6, 5, 3), 8, 30000, seed=0)
+    b = synth.make_room((5, 4, 3), 6, 30000, seed=1)
+    scene = synth.concat_scenes([a, b])
+    case = scene_attn_case(oracle_lib, scene, 5, 4, 10, 8, "XYZ_RGB_NORM", recipe="layer")
+    to_half_and_back(case)
+    got = run_attention(case, torch.float16)
+    _sampled_parity(oracle_lib, case, got, torch.float16, 300)
