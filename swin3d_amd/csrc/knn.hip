@@ -2,9 +2,9 @@
 //
 // Replaces the brute-force kernel of Swin3D/src/knn/knn_cuda_kernel.cu:139-204
 // (one thread streaming every source of the batch through a 64-slot heap).
-// Sources are bucketed into a uniform grid (one counting sort), every query
-// thread walks cubic shells of cells around its own cell and keeps the K best
-// candidates in registers, ordered by (squared distance, source row).  A shell
+// Sources are bucketed into a uniform grid (one counting sort); a small group of
+// lanes per query walks cubic shells of cells around the query's cell and keeps
+// the K best candidates, ordered by (squared distance, source row).  A shell
 // walk stops once the K-th best distance is provably smaller than the distance
 // to anything outside the visited cube, so the result is exact and independent
 // of the visiting order: ties go to the lower source row.
@@ -266,79 +266,26 @@ __device__ __forceinline__ bool cand_less(float d, int i, float d2, int i2)
     return d < d2 || (d == d2 && i < i2);
 }
 
-template <int K>
-struct TopKRegs {
-    float d[K];
-    int id[K];
-    __device__ __forceinline__ void init(int)
-    {
-#pragma unroll
-        for (int t = 0; t < K; ++t) {
-            d[t] = INFINITY;
-            id[t] = 0x7fffffff;
-        }
-    }
-    __device__ __forceinline__ float worst_d(int) const { return d[K - 1]; }
-    __device__ __forceinline__ int worst_i(int) const { return id[K - 1]; }
-    __device__ __forceinline__ void insert(float cd, int ci, int)
-    {
-#pragma unroll
-        for (int t = K - 1; t > 0; --t) {
-            const bool before_prev = cand_less(cd, ci, d[t - 1], id[t - 1]);
-            const bool before_this = cand_less(cd, ci, d[t], id[t]);
-            const float nd = before_prev ? d[t - 1] : (before_this ? cd : d[t]);
-            const int ni = before_prev ? id[t - 1] : (before_this ? ci : id[t]);
-            d[t] = nd;
-            id[t] = ni;
-        }
-        if (cand_less(cd, ci, d[0], id[0])) {
-            d[0] = cd;
-            id[0] = ci;
-        }
-    }
-    __device__ __forceinline__ float get_d(int t) const { return d[t]; }
-    __device__ __forceinline__ int get_i(int t) const { return id[t]; }
-};
-
-// Any K up to S3D_KNN_KMAX: same ordered list, indexed at run time (lives in scratch memory).
-struct TopKAny {
-    float d[S3D_KNN_KMAX];
-    int id[S3D_KNN_KMAX];
-    __device__ __forceinline__ void init(int K)
-    {
-        for (int t = 0; t < K; ++t) {
-            d[t] = INFINITY;
-            id[t] = 0x7fffffff;
-        }
-    }
-    __device__ __forceinline__ float worst_d(int K) const { return d[K - 1]; }
-    __device__ __forceinline__ int worst_i(int K) const { return id[K - 1]; }
-    __device__ __forceinline__ void insert(float cd, int ci, int K)
-    {
-        int t = K - 1;
-        while (t > 0 && cand_less(cd, ci, d[t - 1], id[t - 1])) {
-            d[t] = d[t - 1];
-            id[t] = id[t - 1];
-            --t;
-        }
-        d[t] = cd;
-        id[t] = ci;
-    }
-    __device__ __forceinline__ float get_d(int t) const { return d[t]; }
-    __device__ __forceinline__ int get_i(int t) const { return id[t]; }
-};
-
-template <typename TopK>
+// One query per group of G lanes (G = 4, 16 or 64 >= K).  The group keeps its K best candidates
+// as ONE sorted list spread over its lanes (lane t holds the t-th best), so an insertion is a
+// compare plus a one-lane shift for the whole group instead of a K-long loop per thread, the
+// sources of a cell run are loaded G at a time (coalesced), and a 50k-query call fills the
+// chip with wavefronts instead of leaving it with a few hundred.
+template <int G>
 __global__ __launch_bounds__(kThreads) void knn_query_kernel(
     int K, const float *__restrict__ qry, int64_t Nq, const int32_t *__restrict__ query_offset,
     int B, const KnnPlan *__restrict__ plan_ptr, const int32_t *__restrict__ starts,
     const float4 *__restrict__ sorted, int32_t *__restrict__ ret_idx, float *__restrict__ ret_dist2)
 {
-    const int64_t g = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-    if (g >= Nq) return;
+    const int lane = threadIdx.x & 63;
+    const int t = lane % G;                    // position in the group's sorted list
+    const int group_shift = lane - t;          // first lane of the group inside the wavefront
+    const int64_t g_raw = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) / G;
+    const bool live = g_raw < Nq;              // groups past the last query idle along (no early
+    const int64_t g = live ? g_raw : Nq - 1;   // exit: their lanes may share a wavefront with live ones)
     const KnnPlan plan = *plan_ptr;
-    TopK best;
-    best.init(K);
+    float bd = INFINITY;
+    int bi = 0x7fffffff;
     const int b = find_batch(query_offset, B, g);
     if (b < B && plan.src_end > 0) {
         const float qx = qry[g * 3], qy = qry[g * 3 + 1], qz = qry[g * 3 + 2];
@@ -358,10 +305,10 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
             const int y0 = max(qc[1] - r, 0), y1 = min(qc[1] + r, plan.dim[1] - 1);
             const int ny = y1 - y0 + 1;
             const int n_rows = (z1 - z0 + 1) * ny;   // <= 0 when the shell misses the grid in z or y
-            // source ranges of row t of the shell: a face row spans the whole x range of the cube
+            // source ranges of row u of the shell: a face row spans the whole x range of the cube
             // (one contiguous run of cells), an interior row only its two end cells
-            auto row_ranges = [&](int t, int &a0, int &a1, int &b0, int &b1) {
-                const int z = z0 + t / ny, y = y0 + t % ny;
+            auto row_ranges = [&](int u, int &a0, int &a1, int &b0, int &b1) {
+                const int z = z0 + u / ny, y = y0 + u % ny;
                 const bool face = r == 0 || z == qc[2] - r || z == qc[2] + r || y == qc[1] - r ||
                                   y == qc[1] + r;
                 const int32_t *row = cell_base + (z * plan.dim[1] + y) * plan.dim[0];
@@ -385,24 +332,39 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
                 }
             };
             auto scan_sources = [&](int s_begin, int s_end) {
-                for (int s = s_begin; s < s_end; s += 2) {
-                    // two candidates per trip so that their loads are in flight together
-                    const bool two = s + 1 < s_end;
-                    const float4 p0 = sorted[s];
-                    const float4 p1 = sorted[two ? s + 1 : s];
-                    const float d0 = dist2_unfused(p0.x, p0.y, p0.z, qx, qy, qz);
-                    const float d1 = dist2_unfused(p1.x, p1.y, p1.z, qx, qy, qz);
-                    const int i0 = __float_as_int(p0.w), i1 = __float_as_int(p1.w);
-                    if (cand_less(d0, i0, best.worst_d(K), best.worst_i(K))) best.insert(d0, i0, K);
-                    if (two && cand_less(d1, i1, best.worst_d(K), best.worst_i(K))) best.insert(d1, i1, K);
+                for (int s0 = s_begin; s0 < s_end; s0 += G) {
+                    const int s = s0 + t;
+                    const bool have = s < s_end;
+                    const float4 p = sorted[have ? s : s_begin];
+                    const float cd = have ? dist2_unfused(p.x, p.y, p.z, qx, qy, qz) : INFINITY;
+                    const int ci = have ? __float_as_int(p.w) : 0x7fffffff;
+                    // candidates that beat the current K-th best of the group
+                    const float kth_d = __shfl(bd, K - 1, G);
+                    const int kth_i = __shfl(bi, K - 1, G);
+                    unsigned long long pass = __ballot(cand_less(cd, ci, kth_d, kth_i));
+                    pass = (pass >> group_shift) & (G == 64 ? ~0ULL : ((1ULL << G) - 1));
+                    while (pass) {
+                        const int c = __ffsll(static_cast<long long>(pass)) - 1;
+                        pass &= pass - 1;
+                        const float xd = __shfl(cd, c, G);
+                        const int xi = __shfl(ci, c, G);
+                        const float pd = __shfl_up(bd, 1, G);
+                        const int pi = __shfl_up(bi, 1, G);
+                        const bool before_prev = t > 0 && cand_less(xd, xi, pd, pi);
+                        const bool before_this = cand_less(xd, xi, bd, bi);
+                        const float nd = before_prev ? pd : (before_this ? xd : bd);
+                        const int ni = before_prev ? pi : (before_this ? xi : bi);
+                        bd = nd;
+                        bi = ni;
+                    }
                 }
             };
             int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
             if (n_rows > 0) row_ranges(0, a0, a1, b0, b1);
-            for (int t = 0; t < n_rows; ++t) {
+            for (int u = 0; u < n_rows; ++u) {
                 // the next row's cell bounds are loaded while this row's sources are scanned
                 int na0 = 0, na1 = 0, nb0 = 0, nb1 = 0;
-                if (t + 1 < n_rows) row_ranges(t + 1, na0, na1, nb0, nb1);
+                if (u + 1 < n_rows) row_ranges(u + 1, na0, na1, nb0, nb1);
                 scan_sources(a0, a1);
                 scan_sources(b0, b1);
                 a0 = na0;
@@ -410,7 +372,7 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
                 b0 = nb0;
                 b1 = nb1;
             }
-            if (best.worst_i(K) != 0x7fffffff) {
+            if (__shfl(bi, K - 1, G) != 0x7fffffff) {
                 // everything outside the visited cube is at least `bound` away from the query
                 float bound = INFINITY;
 #pragma unroll
@@ -420,15 +382,14 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
                     bound = fminf(bound, fminf(qp[a] - lo_face, hi_face - qp[a]));
                 }
                 bound -= plan.slack;
-                if (bound > 0.0f && best.worst_d(K) < bound * bound) break;
+                if (bound > 0.0f && __shfl(bd, K - 1, G) < bound * bound) break;
             }
         }
     }
-    for (int t = 0; t < K; ++t) {
-        const int si = best.get_i(t);
-        const bool filled = si != 0x7fffffff;
-        ret_idx[g * K + t] = filled ? si : -1;
-        ret_dist2[g * K + t] = filled ? best.get_d(t) : S3D_KNN_PAD_DIST2;
+    if (live && t < K) {
+        const bool filled = bi != 0x7fffffff;
+        ret_idx[g * K + t] = filled ? bi : -1;
+        ret_dist2[g * K + t] = filled ? bd : S3D_KNN_PAD_DIST2;
     }
 }
 
@@ -450,7 +411,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
     using namespace s3d;
     if (K < 1 || K > S3D_KNN_KMAX)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_knn: K=%d outside 1..%d", K, S3D_KNN_KMAX);
-    if (Ns < 0 || Nq < 0 || Ns > 0x7fffffffLL || Nq * K > 0x7fffffffffLL || B < 1 || B > kMaxBatch)
+    if (Ns < 0 || Nq < 0 || Ns > 0x7fffffffLL || Nq > 0x3fffffffLL || B < 1 || B > kMaxBatch)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_knn: Ns=%lld Nq=%lld B=%d out of range", (long long)Ns,
                     (long long)Nq, B);
     if (Nq == 0) return S3D_OK;
@@ -497,16 +458,17 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
                            cell_size, L.cells_cap);
         S3D_HIP_CHECK(hipGetLastError());
     }
-    const dim3 qgrid(static_cast<unsigned>(ceil_div(Nq, kThreads)));
-    if (K == 3)
-        hipLaunchKernelGGL(knn_query_kernel<TopKRegs<3>>, qgrid, dim3(kThreads), 0, s, K, query_xyz,
-                           Nq, query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
-    else if (K == 16)
-        hipLaunchKernelGGL(knn_query_kernel<TopKRegs<16>>, qgrid, dim3(kThreads), 0, s, K, query_xyz,
-                           Nq, query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
+    const int G = K <= 4 ? 4 : K <= 16 ? 16 : 64;   // lanes per query
+    const dim3 qgrid(static_cast<unsigned>(ceil_div(Nq * G, kThreads)));
+    if (G == 4)
+        hipLaunchKernelGGL(knn_query_kernel<4>, qgrid, dim3(kThreads), 0, s, K, query_xyz, Nq, query_offset,
+                           B, plan, starts, sorted, ret_idx, ret_dist2);
+    else if (G == 16)
+        hipLaunchKernelGGL(knn_query_kernel<16>, qgrid, dim3(kThreads), 0, s, K, query_xyz, Nq, query_offset,
+                           B, plan, starts, sorted, ret_idx, ret_dist2);
     else
-        hipLaunchKernelGGL(knn_query_kernel<TopKAny>, qgrid, dim3(kThreads), 0, s, K, query_xyz, Nq,
-                           query_offset, B, plan, starts, sorted, ret_idx, ret_dist2);
+        hipLaunchKernelGGL(knn_query_kernel<64>, qgrid, dim3(kThreads), 0, s, K, query_xyz, Nq, query_offset,
+                           B, plan, starts, sorted, ret_idx, ret_dist2);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }
