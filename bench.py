@@ -42,6 +42,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (1 = force the generic kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
+    ap.add_argument("--no-encoder", action="store_true",
+                    help="skip the Swin3D-L encoder end-to-end latency (BASELINE configs[4])")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (windows are independent; see DESIGN.md for how "
@@ -156,6 +158,9 @@ def main():
     if not args.no_extras:
         result["extras"] = extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev)
 
+    if not args.no_extras and not args.no_encoder:
+        result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)
+
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m)
 
@@ -197,6 +202,35 @@ def extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev):
         out[name] = {"ms": ms, "queries_per_s": nq / (ms * 1e-3), "sources": ns, "queries": nq,
                      "algorithmic_bytes": alg, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     return out
+
+
+def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3):
+    """BASELINE configs[4]: Swin3D-L encoder forward, fp16 attention (fp16_mode 2 under autocast),
+    random-init weights, a batch of two synthetic rooms of ~300k voxels each; attention, window
+    index and KNN on the HIP kernels, the dense layers on torch/hipBLASLt."""
+    from swin3d_amd import encoder
+    scenes = [synth.make_room((10.0, 8.0, 3.0), 30, voxels_per_scene, seed=s) for s in (0, 1)]
+    scene = synth.concat_scenes(scenes)
+    feats, signals = synth.encoder_inputs(scene)
+    vox = encoder.SparseVoxels(torch.from_numpy(scene.coords).to(dev), torch.from_numpy(feats).to(dev), 1)
+    sig = torch.from_numpy(signals).to(dev)
+    torch.manual_seed(0)
+    model = encoder.Swin3DEncoder(**encoder.SWIN3D_L, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=2)
+    model = model.to(dev).eval()
+    times = []
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        outs = model(vox, sig)          # warm-up (allocator, hipBLASLt heuristics)
+        torch.cuda.synchronize()
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            outs = model(vox, sig)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+    return {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
+            "voxels_per_stage": [int(o.coords.shape[0]) for o in outs],
+            "finite": bool(all(torch.isfinite(o.feats).all().item() for o in outs)),
+            "config": "Swin3D-L channels [80,160,320,640,640] heads [10,10,20,40,40] depths [2,4,9,4,4] "
+                      "windows [5,7,7,7,7] quant 4 cRSE XYZ_RGB_NORM, batch of 2 rooms"}
 
 
 def cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m):

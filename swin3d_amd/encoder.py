@@ -1,0 +1,268 @@
+"""Swin3D encoder on the swin3d_amd operators, without MinkowskiEngine (inference path).
+
+Everything around the two hot operators is plain PyTorch-ROCm: the sparse voxel set is a pair
+of tensors (`SparseVoxels`), coordinate lookups are sort + searchsorted on packed 64-bit keys,
+dense math (Linear / LayerNorm / GELU, the 27-offset stem convolution as one GEMM) goes to
+hipBLASLt through torch.  Window attention runs through `SelfAttnAIOFunction`, the window index
+through `get_index01`, neighbour gathering through `KNN`.
+
+What each piece mirrors in the reference (semantics, not code):
+  sparse_conv3x3x3 + BatchNorm + ReLU   MinkConvBNRelu stem            Swin3D/modules/mink_layers.py:50-80
+  pool_coordinates                      MinkowskiMaxPooling on coords  Swin3D/modules/swin3d_layers.py:284-286
+  pick_cell_representatives             GridCoordsDown                 :179-231
+  segment_offsets                       get_offset                     :234-241
+  GridKNNDownsample                     same name                      :272-315
+  WindowAttention / SwinBlock / Stage   WindowAttention, SwinTransformerBlock, BasicLayer  :382-871
+  Swin3DEncoder                         same name                      Swin3D/models/Swin3D.py:185-269
+MinkowskiEngine's output ORDER of pooled coordinates and its tie-breaking are not pinned by
+anything in the reference; here pooled voxels are sorted by (batch, x, y, z) and ties go to
+the lower row.  Stochastic depth is inference-time identity.
+"""
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
+from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
+from .sparse_dl.knn import KNN
+from .window_index import get_index01
+
+
+@dataclass
+class SparseVoxels:
+    """coords int32 [N,4] = (batch, x, y, z), x/y/z multiples of `stride`, batches contiguous and
+    ascending; feats [N,C]."""
+    coords: torch.Tensor
+    feats: torch.Tensor
+    stride: int = 1
+
+    def with_feats(self, feats):
+        return SparseVoxels(self.coords, feats, self.stride)
+
+
+_FIELD = 19            # bits per coordinate in a packed key
+_BIAS = 1 << (_FIELD - 1)
+
+
+def pack_coords(coords):
+    """int64 key, order-preserving for (batch, x, y, z) with |x|,|y|,|z| < 2^18 and batch < 64."""
+    c = coords.long()
+    key = c[:, 0]
+    for axis in (1, 2, 3):
+        key = (key << _FIELD) + (c[:, axis] + _BIAS)
+    return key
+
+
+def lookup_rows(sorted_keys, order, query_keys):
+    """row of every query key in the voxel set described by (sorted_keys, order); -1 if absent."""
+    pos = torch.searchsorted(sorted_keys, query_keys).clamp_(max=sorted_keys.numel() - 1)
+    hit = sorted_keys[pos] == query_keys
+    return torch.where(hit, order[pos], torch.full_like(pos, -1))
+
+
+def sparse_conv3x3x3(voxels, weight):
+    """Submanifold-style 3x3x3 convolution (outputs on the input voxels; missing neighbours are
+    zeros).  weight [27, Cin, Cout], offsets ordered x-major.  One gather + one GEMM."""
+    coords, feats, s = voxels.coords, voxels.feats, voxels.stride
+    n, cin = feats.shape
+    keys = pack_coords(coords)
+    sorted_keys, order = torch.sort(keys)
+    padded = torch.cat([feats, feats.new_zeros(1, cin)], 0)   # row n = zeros for missing neighbours
+    cols = []
+    for dx in (-1, 0, 1):
+        for dy in (-1, 0, 1):
+            for dz in (-1, 0, 1):
+                off = torch.tensor([0, dx * s, dy * s, dz * s], dtype=coords.dtype, device=coords.device)
+                rows = lookup_rows(sorted_keys, order, pack_coords(coords + off))
+                cols.append(padded[torch.where(rows < 0, torch.full_like(rows, n), rows)])
+    gathered = torch.cat(cols, 1)                              # [N, 27*Cin]
+    return gathered @ weight.reshape(27 * cin, -1).to(gathered.dtype)
+
+
+def pool_coordinates(coords, stride, factor):
+    """coarse voxel coordinates (floor to the coarse lattice), unique and sorted by (b,x,y,z);
+    also the coarse row of every fine voxel."""
+    step = stride * factor
+    coarse = coords.clone()
+    coarse[:, 1:] = torch.div(coords[:, 1:], step, rounding_mode="floor") * step
+    keys = pack_coords(coarse)
+    uniq, inverse = torch.unique(keys, sorted=True, return_inverse=True)
+    first = torch.full((uniq.numel(),), coords.shape[0], dtype=torch.long, device=coords.device)
+    first.scatter_reduce_(0, inverse, torch.arange(coords.shape[0], device=coords.device), reduce="amin")
+    return coarse[first], inverse
+
+
+def pick_cell_representatives(signals, cell_of_row, num_cells):
+    """For every coarse cell the fine row whose signal vector (all columns of the coordinate
+    features) is nearest to the cell mean; ties go to the lower row."""
+    sig = signals.float()
+    sums = sig.new_zeros(num_cells, sig.shape[1]).index_add_(0, cell_of_row, sig)
+    counts = sig.new_zeros(num_cells).index_add_(0, cell_of_row, sig.new_ones(sig.shape[0]))
+    mean = sums / counts.unsqueeze(1)
+    dist = (sig - mean[cell_of_row]).pow(2).sum(1).sqrt()
+    best = dist.new_full((num_cells,), float("inf")).scatter_reduce_(0, cell_of_row, dist, reduce="amin")
+    rows = torch.arange(sig.shape[0], device=sig.device)
+    cand = torch.where(dist == best[cell_of_row], rows, torch.full_like(rows, sig.shape[0]))
+    pick = torch.full((num_cells,), sig.shape[0], dtype=torch.long, device=sig.device)
+    pick.scatter_reduce_(0, cell_of_row, cand, reduce="amin")
+    return pick
+
+
+def segment_offsets(batch_column):
+    """cumulative END row of every batch element, int32 (what the KNN op takes)."""
+    counts = torch.bincount(batch_column.long())
+    return torch.cumsum(counts, 0).to(torch.int32)
+
+
+class StemConv(nn.Module):
+    """3x3x3 sparse convolution + BatchNorm + ReLU."""
+
+    def __init__(self, in_channels, out_channels):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(27, in_channels, out_channels))
+        nn.init.kaiming_normal_(self.weight.view(27 * in_channels, out_channels).t())
+        self.norm = nn.BatchNorm1d(out_channels)
+
+    def forward(self, voxels):
+        out = sparse_conv3x3x3(voxels, self.weight)
+        return voxels.with_feats(F.relu(self.norm(out.float())))
+
+
+class GridKNNDownsample(nn.Module):
+    """Coarse voxel = stride-2 cell; its feature = max over the K=16 nearest fine points of
+    Linear(LayerNorm(feature)); its coordinate signals = those of the picked representative."""
+
+    def __init__(self, in_channels, out_channels, stride=2, k=16):
+        super().__init__()
+        self.factor, self.k = stride, k
+        self.norm = nn.LayerNorm(in_channels)
+        self.linear = nn.Linear(in_channels, out_channels, bias=False)
+
+    def forward(self, voxels, signals):
+        coarse, cell_of_row = pool_coordinates(voxels.coords, voxels.stride, self.factor)
+        pick = pick_cell_representatives(signals, cell_of_row, coarse.shape[0])
+        coarse_signals = signals[pick]
+        src_xyz = signals[:, 1:4].contiguous().float()
+        qry_xyz = coarse_signals[:, 1:4].contiguous().float()
+        idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(voxels.coords[:, 0]),
+                           segment_offsets(coarse[:, 0]))
+        m, c = coarse.shape[0], voxels.feats.shape[1]
+        grouped = voxels.feats[idx.view(-1).long().clamp_(min=0)].view(m, self.k, c)
+        feats = self.linear(self.norm(grouped)).amax(dim=1)
+        return SparseVoxels(coarse, feats.float(), voxels.stride * self.factor), coarse_signals
+
+
+class WindowAttention(nn.Module):
+    """Window multi-head self-attention with cRSE tables on the fused HIP operator."""
+
+    def __init__(self, dim, window_size, quant_size, num_heads, cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.dim, self.num_heads, self.window_size, self.quant_size = dim, num_heads, window_size, quant_size
+        self.head_dim = dim // num_heads
+        self.scale = self.head_dim ** -0.5
+        self.cRSE, self.fp16_mode = cRSE, fp16_mode
+        self.table_sizes = crse_table_sizes(window_size, quant_size, num_heads, self.head_dim, cRSE)
+        rows = [sz // dim for sz in self.table_sizes]
+        for kind in ("query", "key", "value"):
+            for group, name in enumerate(("xyz", "rgb", "norm")[: crse_num_axes(cRSE) // 3]):
+                table = nn.Parameter(torch.zeros(3, rows[3 * group], num_heads, self.head_dim))
+                nn.init.trunc_normal_(table, std=0.02)
+                setattr(self, f"{kind}_{name}_table", table)
+        self.qkv = nn.Linear(dim, dim * 3)
+        self.proj = nn.Linear(dim, dim)
+
+    def _flat_table(self, kind):
+        names = ("xyz", "rgb", "norm")[: crse_num_axes(self.cRSE) // 3]
+        return torch.cat([getattr(self, f"{kind}_{n}_table").reshape(-1) for n in names])
+
+    def forward(self, feats, attn_args):
+        n = feats.shape[0]
+        _, _, m2w, w_sizes, w2n, n2n, w2m, n_coords = attn_args
+        qkv = self.qkv(feats).reshape(n, 3, self.num_heads, self.head_dim).permute(1, 0, 2, 3).contiguous()
+        query, key, value = qkv[0] * self.scale, qkv[1], qkv[2]
+        n_crse = scale_crse_coords(n_coords, self.quant_size, self.cRSE)
+        precision = (PrecisionMode.HALF_NONE, PrecisionMode.HALF_FORWARD, PrecisionMode.HALF_ALL)[self.fp16_mode]
+        out = SelfAttnAIOFunction.apply(
+            query, key, value, self._flat_table("query"), self._flat_table("key"), self._flat_table("value"),
+            self.table_sizes, [m2w, w_sizes, w2m, w2n, n2n, n_crse], PosEmb.SEPARATE, TableDims.D0,
+            IndexMode.INDIRECT, precision)
+        return self.proj(out.reshape(n, self.dim).to(feats.dtype))
+
+
+class SwinBlock(nn.Module):
+    def __init__(self, dim, num_heads, window_size, quant_size, mlp_ratio=4.0, cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.norm1 = nn.LayerNorm(dim)
+        self.attn = WindowAttention(dim, window_size, quant_size, num_heads, cRSE, fp16_mode)
+        self.norm2 = nn.LayerNorm(dim)
+        hidden = int(dim * mlp_ratio)
+        self.mlp = nn.Sequential(nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
+
+    def forward(self, feats, attn_args):
+        feats = feats + self.attn(self.norm1(feats), attn_args).float()
+        return feats + self.mlp(self.norm2(feats)).float()
+
+
+class Stage(nn.Module):
+    """`depth` Swin blocks on one resolution (regular / shifted windows alternate), then an
+    optional KNN downsample."""
+
+    def __init__(self, dim, depth, num_heads, window_size, quant_size, out_channels=None, down_stride=2,
+                 downsample=True, cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.window_size = window_size
+        self.blocks = nn.ModuleList(
+            [SwinBlock(dim, num_heads, window_size, quant_size, cRSE=cRSE, fp16_mode=fp16_mode) for _ in range(depth)])
+        self.downsample = GridKNNDownsample(dim, out_channels or dim * 2, stride=down_stride) if downsample else None
+
+    def forward(self, voxels, signals):
+        """signals [N, 4|7|10] float = (batch, xyz in voxel units, rgb, normal) of the point kept
+        in every voxel.  Returns (features at this resolution, next voxels, next signals)."""
+        local = (signals[:, 1:4].float() - voxels.coords[:, 1:].float()) / voxels.stride
+        extra = signals[:, 4:].float()
+        args = [get_index01(voxels.coords, voxels.stride, self.window_size, local, extra, shift=s)
+                for s in (0, self.window_size // 2)]
+        feats = voxels.feats
+        for i, block in enumerate(self.blocks):
+            feats = block(feats, args[i % 2])
+        voxels = voxels.with_feats(feats)
+        if self.downsample is None:
+            return voxels, voxels, signals
+        down, down_signals = self.downsample(voxels, signals)
+        return voxels, down, down_signals
+
+
+class Swin3DEncoder(nn.Module):
+    """stem -> `num_layers` stages; returns the per-stage SparseVoxels (finest first)."""
+
+    def __init__(self, depths, channels, num_heads, window_sizes, quant_size, num_layers=5, first_down_stride=2,
+                 in_channels=6, cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.stem_layer = StemConv(in_channels, channels[0])
+        self.layers = nn.ModuleList([
+            Stage(channels[i], depths[i], num_heads[i], window_sizes[i], quant_size,
+                  out_channels=channels[i + 1] if i < num_layers - 1 else None,
+                  down_stride=first_down_stride if i == 0 else 2, downsample=i < num_layers - 1,
+                  cRSE=cRSE, fp16_mode=fp16_mode)
+            for i in range(num_layers)])
+        for m in self.modules():
+            if isinstance(m, nn.Linear):
+                nn.init.trunc_normal_(m.weight, std=0.02)
+                if m.bias is not None:
+                    nn.init.zeros_(m.bias)
+
+    def forward(self, voxels, signals):
+        voxels = self.stem_layer(voxels)
+        outputs = []
+        for layer in self.layers:
+            here, voxels, signals = layer(voxels, signals)
+            outputs.append(here)
+        return outputs
+
+
+SWIN3D_S = dict(depths=[2, 4, 9, 4, 4], channels=[48, 96, 192, 384, 384], num_heads=[6, 6, 12, 24, 24],
+                window_sizes=[5, 7, 7, 7, 7], quant_size=4)
+SWIN3D_L = dict(depths=[2, 4, 9, 4, 4], channels=[80, 160, 320, 640, 640], num_heads=[10, 10, 20, 40, 40],
+                window_sizes=[5, 7, 7, 7, 7], quant_size=4)

@@ -42,6 +42,9 @@ class PrecisionMode(enum.Enum):
 
 _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_F16}
 
+# debugging / ablation switch: run the generic VALU kernel even where the MFMA kernel applies
+FORCE_GENERIC = False
+
 
 def _require_cuda(name, t, device=None):
     if not isinstance(t, torch.Tensor):
@@ -144,7 +147,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
             n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype],
-            _lib.S3D_ATTN_FORCE_GENERIC if force_generic else 0, workspace.data_ptr(), ws_bytes, stream)
+            _lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0, workspace.data_ptr(),
+            ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
     if return_stats:
         return out, omax, osum

@@ -145,3 +145,14 @@ def layer_inputs(n, channels, heads, table_len, seed=0, recipe="layer", dtype=np
     q, k, v = (np.ascontiguousarray(x).astype(dtype) for x in (q, k, v))
     tables = [t.astype(dtype) for t in tables]
     return q, k, v, tables
+
+
+def encoder_inputs(scene):
+    """Model inputs of a Scene in the reference's conventions (Swin3D/models/Swin3D.py:117-129):
+    features [N,9] = (rgb, normal, point position inside the voxel), all in [-1,1]-ish ranges, and
+    coordinate signals [N,10] = (batch, xyz in voxel units, rgb in [-1,1], normal)."""
+    rgb = scene.rgb * np.float32(2.0) - np.float32(1.0)
+    feats = np.concatenate([rgb, scene.normal, scene.frac - np.float32(0.5)], axis=1).astype(np.float32)
+    signals = np.concatenate([scene.coords[:, :1].astype(np.float32), scene.xyz, rgb, scene.normal],
+                             axis=1).astype(np.float32)
+    return feats, signals

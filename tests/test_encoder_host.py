@@ -1,0 +1,72 @@
+"""Torch-only substrate of the encoder (runs on the CPU): sparse convolution against a dense
+conv3d, coordinate pooling and the representative pick against brute force."""
+import numpy as np
+import torch
+
+from conftest import random_scene
+from swin3d_amd import encoder
+
+
+def test_sparse_conv_matches_dense_conv3d():
+    rng = np.random.default_rng(0)
+    coords = torch.from_numpy(random_scene(rng, 300, extent=(4, 4, 3), batches=2))
+    cin, cout = 5, 7
+    feats = torch.randn(300, cin, dtype=torch.float64)
+    weight = torch.randn(27, cin, cout, dtype=torch.float64)
+    got = encoder.sparse_conv3x3x3(encoder.SparseVoxels(coords, feats, 1), weight)
+    # dense volume [B, Cin, X, Y, Z] with the same voxels, zero elsewhere
+    lo = coords[:, 1:].min(0).values
+    size = (coords[:, 1:].max(0).values - lo + 1).tolist()
+    dense = torch.zeros(2, cin, *size, dtype=torch.float64)
+    c = coords.long()
+    dense[c[:, 0], :, c[:, 1] - lo[0], c[:, 2] - lo[1], c[:, 3] - lo[2]] = feats
+    w = weight.reshape(3, 3, 3, cin, cout).permute(4, 3, 0, 1, 2)      # [Cout, Cin, kx, ky, kz]
+    ref = torch.nn.functional.conv3d(dense, w, padding=1)
+    ref = ref[c[:, 0], :, c[:, 1] - lo[0], c[:, 2] - lo[1], c[:, 3] - lo[2]]
+    torch.testing.assert_close(got, ref)
+
+
+def test_sparse_conv_respects_tensor_stride():
+    coords = torch.tensor([[0, 0, 0, 0], [0, 2, 0, 0], [0, 1, 0, 0]], dtype=torch.int32)   # stride 2 lattice + a stray
+    feats = torch.eye(3, dtype=torch.float64)
+    weight = torch.zeros(27, 3, 1, dtype=torch.float64)
+    weight[(2 * 3 + 1) * 3 + 1] = 1.0            # offset (+1, 0, 0) in units of the stride
+    out = encoder.sparse_conv3x3x3(encoder.SparseVoxels(coords, feats, 2), weight)
+    # voxel (0,0,0) sees voxel (2,0,0) (row 1); nothing else has a +stride neighbour
+    assert out[:, 0].tolist() == [1.0, 0.0, 0.0]
+
+
+def test_pool_coordinates_and_representatives():
+    rng = np.random.default_rng(1)
+    coords_np = random_scene(rng, 500, extent=(6, 6, 3), batches=2, stride=2)
+    coords = torch.from_numpy(coords_np)
+    coarse, cell_of_row = encoder.pool_coordinates(coords, 2, 2)
+    cells = {}
+    for row, (b, x, y, z) in enumerate(coords_np.tolist()):
+        cells.setdefault((b, x // 4 * 4, y // 4 * 4, z // 4 * 4), []).append(row)
+    keys = sorted(cells)
+    assert coarse.tolist() == [list(k) for k in keys]                      # sorted by (b, x, y, z)
+    assert [keys[c] for c in cell_of_row.tolist()] == [(b, x // 4 * 4, y // 4 * 4, z // 4 * 4) for b, x, y, z in coords_np.tolist()]
+    signals = torch.from_numpy(rng.random((500, 10)).astype(np.float32))
+    signals[:, 0] = coords[:, 0].float()
+    signals[10] = signals[11]                                               # a tie inside one cell is possible
+    pick = encoder.pick_cell_representatives(signals, cell_of_row, coarse.shape[0])
+    sig = signals.numpy().astype(np.float64)
+    for ci, key in enumerate(keys):
+        rows = cells[key]
+        mean = signals[rows].float().mean(0).numpy()
+        d = np.sqrt(((signals[rows].float().numpy() - mean) ** 2).sum(1))
+        best = [r for r, dd in zip(rows, d) if np.isclose(dd, d.min(), rtol=1e-6, atol=1e-7)]
+        assert int(pick[ci]) in best and int(pick[ci]) in rows
+
+
+def test_segment_offsets():
+    batch = torch.tensor([0, 0, 0, 1, 1, 3], dtype=torch.int32)
+    assert encoder.segment_offsets(batch).tolist() == [3, 5, 5, 6]
+    assert encoder.segment_offsets(batch).dtype == torch.int32
+
+
+def test_pack_coords_is_order_preserving():
+    coords = torch.tensor([[0, -5, 3, 2], [0, -5, 3, 3], [0, 4, -100000, 0], [1, -200000, 0, 0], [63, 0, 0, 0]])
+    keys = encoder.pack_coords(coords)
+    assert (keys[1:] > keys[:-1]).all()

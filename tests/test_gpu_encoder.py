@@ -1,0 +1,72 @@
+"""End-to-end encoder forward on the HIP operators (GPU)."""
+import numpy as np
+import pytest
+import torch
+
+from swin3d_amd import encoder, synth
+from swin3d_amd.sparse_dl.attn import attn_coff
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(target=12000, batches=2):
+    scenes = [synth.make_room((4.0, 3.0, 2.5), 4, target, seed=s) for s in range(batches)]
+    scene = synth.concat_scenes(scenes)
+    feats, signals = synth.encoder_inputs(scene)
+    dev = torch.device("cuda")
+    vox = encoder.SparseVoxels(torch.from_numpy(scene.coords).to(dev), torch.from_numpy(feats).to(dev), 1)
+    return vox, torch.from_numpy(signals).to(dev)
+
+
+def _small_model(fp16_mode):
+    torch.manual_seed(0)
+    cfg = dict(depths=[2, 2, 2], channels=[48, 96, 192], num_heads=[6, 6, 12], window_sizes=[5, 7, 7],
+               quant_size=4, num_layers=3)
+    return encoder.Swin3DEncoder(**cfg, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=fp16_mode).cuda().eval()
+
+
+def test_encoder_forward_fp16_runs_on_both_kernels(hip_lib):
+    vox, signals = _inputs()
+    model = _small_model(fp16_mode=2)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        outs = model(vox, signals)
+        attn_coff.FORCE_GENERIC = True
+        try:
+            outs_generic = model(vox, signals)
+        finally:
+            attn_coff.FORCE_GENERIC = False
+    torch.cuda.synchronize()
+    assert [o.feats.shape[1] for o in outs] == [48, 96, 192]
+    assert [o.stride for o in outs] == [1, 2, 4]
+    assert outs[0].coords.shape[0] == vox.coords.shape[0]
+    assert outs[1].coords.shape[0] < outs[0].coords.shape[0] and outs[2].coords.shape[0] < outs[1].coords.shape[0]
+    for a, b in zip(outs, outs_generic):
+        assert torch.isfinite(a.feats).all()
+        assert torch.equal(a.coords, b.coords)
+        # two different kernels, fp16 attention inside: agreement to fp16 resolution of O(1) features
+        assert (a.feats - b.feats).abs().max().item() < 2e-2 * max(1.0, b.feats.abs().max().item())
+    # batches stay contiguous and ascending at every level, coordinates sit on the level's lattice
+    for o in outs:
+        bcol = o.coords[:, 0]
+        assert (bcol[1:] >= bcol[:-1]).all()
+        assert (o.coords[:, 1:] % o.stride == 0).all()
+
+
+def test_knn_downsample_matches_oracle_neighbours(oracle_lib, hip_lib):
+    vox, signals = _inputs(target=6000, batches=2)
+    torch.manual_seed(1)
+    down = encoder.GridKNNDownsample(9, 16).cuda().eval()
+    with torch.no_grad():
+        coarse, coarse_signals = down(vox, signals)
+    src = signals[:, 1:4].contiguous().cpu().numpy()
+    qry = coarse_signals[:, 1:4].contiguous().cpu().numpy()
+    so = encoder.segment_offsets(vox.coords[:, 0]).cpu().numpy()
+    qo = encoder.segment_offsets(coarse.coords[:, 0]).cpu().numpy()
+    idx, _ = oracle_lib.knn(16, src, qry, so, qo)
+    with torch.no_grad():
+        grouped = vox.feats[torch.from_numpy(idx).long().cuda().view(-1)].view(-1, 16, 9)
+        ref = down.linear(down.norm(grouped)).amax(dim=1)
+    torch.testing.assert_close(coarse.feats, ref.float(), rtol=1e-5, atol=1e-6)
+    # the representative of a cell is one of the cell's own points
+    cell = torch.div(coarse_signals[:, 1:4], 2, rounding_mode="floor") * 2
+    assert torch.equal(cell.int(), coarse.coords[:, 1:])
