@@ -86,7 +86,7 @@ def main():
     c_sizes = (ctypes.c_int32 * nd)(*sizes)
     out = torch.empty_like(q_d)
     num_w, num_m = index.num_windows, index.num_pairs
-    ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, heads, dim, num_w)
+    ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, heads, dim, n, num_w, index.max_window_voxels)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
 
@@ -95,7 +95,7 @@ def main():
                                   tk_d.data_ptr(), tv_d.data_ptr(), c_sizes, nd, table_len,
                                   index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
                                   n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
+                                  index.max_window_voxels, _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
                                   stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")

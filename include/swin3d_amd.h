@@ -75,10 +75,15 @@ const char *s3d_last_error_string(void);
  *                  (the tensor cal_max_coffs returns)
  *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
+ *   max_window_voxels  an upper bound of every w_sizes entry (e.g. counts[2] of s3d_window_index, or
+ *                  window^3).  It sizes the per-key-tile partial results of windows with more than 32
+ *                  voxels; a window larger than the bound would write outside the workspace, so
+ *                  the bound must hold.
  *   flags          0, or S3D_ATTN_FORCE_GENERIC to run the VALU kernel for every case
  *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
- *                  (a transposed copy of the value table and the per-window work-item prefix
- *                  of the MFMA kernel)
+ *                  (MFMA kernel: a transposed copy of the value table, the work-item prefix, and
+ *                  N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
+ *                  max_window_voxels > 32)
  *   D in {8,16}, nd in {3,6,9}, H >= 1.
  *
  * Row index of axis n for the pair (query i, key j), all in fp32:
@@ -95,13 +100,13 @@ const char *s3d_last_error_string(void);
  * 0 if on the generic VALU kernel.  No counterpart in the reference (it has one kernel). */
 int s3d_attn_fwd_uses_mfma(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype);
 size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,
-                                    int64_t W);
+                                    int64_t N, int64_t W, int32_t max_window_voxels);
 int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_q,
                  const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
                  int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
                  const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
-                 int32_t H, int32_t D, int64_t W, int32_t dtype, int32_t flags, void *workspace,
-                 size_t workspace_bytes, void *stream);
+                 int32_t H, int32_t D, int64_t W, int32_t max_window_voxels, int32_t dtype,
+                 int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Window sort + segment offsets.

@@ -50,7 +50,8 @@ int check_shape(int64_t N, int64_t W, int32_t H, int32_t D, int32_t nd, int64_t 
 }  // namespace s3d
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_bytes(
-    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int64_t W)
+    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int64_t N, int64_t W,
+    int32_t max_window_voxels)
 {
     using namespace s3d;
     if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1) return 0;
@@ -59,7 +60,8 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
         const int64_t rows = table_sizes[n] / (static_cast<int64_t>(H) * D);
         padded += (rows + 15) / 16 * 16;
     }
-    return attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W);
+    if (max_window_voxels < 1 || N < 0 || W < 0) return 0;
+    return attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
@@ -81,8 +83,9 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
     const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
     const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
-    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W, int32_t dtype,
-    int32_t flags, void *workspace, size_t workspace_bytes, void *stream)
+    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W,
+    int32_t max_window_voxels, int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes,
+    void *stream)
 {
     using namespace s3d;
     if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
@@ -116,11 +119,16 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype);
     if (want_mfma) {
-        const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W);
+        if (max_window_voxels < 1)
+            return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: max_window_voxels = %d (an upper bound of w_sizes, >= 1)",
+                        max_window_voxels);
+        const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
         if (!workspace || workspace_bytes < need)
             return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                         workspace ? workspace_bytes : size_t(0), need);
         a.items = static_cast<char *>(workspace) + attn_mfma_table_bytes(H, D, a.padded_rows);
+        a.partials = reinterpret_cast<float *>(static_cast<char *>(a.items) + attn_mfma_items_bytes(W));
+        a.max_key_tiles = attn_mfma_key_tiles(max_window_voxels);
         return launch_attn_mfma(a, s);
     }
     return launch_attn_generic(a, dtype, s);

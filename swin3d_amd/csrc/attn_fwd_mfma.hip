@@ -176,13 +176,15 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         const int nkt = (n_w + kTile - 1) / kTile;   // key tiles (= query tiles)
         const bool single_key_tile = nkt == 1;
-        // a single-tile window is one item (all heads, row indices cached across heads);
-        // a larger window is split into (query tile, head) items
+        // one item = one (query tile, key tile) pair of a window, all heads: the pair row indices
+        // are computed once and reused by every head.  A window of at most 32 voxels is a single
+        // item that writes the final output; larger windows write per-key-tile partial results
+        // (running max, sum, unnormalised output) that attn_merge_partials_kernel combines.
         const int local = item - (w > 0 ? __builtin_amdgcn_readfirstlane(item_end[w - 1]) : 0);
-        const int q0 = single_key_tile ? 0 : (local / H) * kTile;
-        const int h_first = single_key_tile ? 0 : local % H;
-        const int h_count = single_key_tile ? H : 1;
-        const int steps = h_count * nkt;             // (head, key tile) steps of this item
+        const int q0 = (local / nkt) * kTile;
+        const int kt_i = local % nkt;
+        const int k0 = kt_i * kTile;
+        const int nk = min(kTile, n_w - k0);
 
         const bool q_valid = q0 + il < n_w;
         const int q_pos = s0 + min(q0 + il, n_w - 1);   // lanes past the window repeat the last voxel
@@ -213,38 +215,28 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 }
             }
         };
-        if (single_key_tile) build_pair_rows(0, n_w);
+        build_pair_rows(k0, nk);
 
-        // fragments of the step ahead (head h, key tile kt): issued one step early
+        // fragments of the head ahead: issued one head early
+        const int k_row = a.n2n[s0 + k0 + min(il, nk - 1)];
         frag_t qf_next, kf_next;
         h8 vv_next;
-        auto prefetch_step = [&](int hh, int kk) {
-            const int k0 = kk * kTile;
-            const int nk = min(kTile, n_w - k0);
-            const int k_row = a.n2n[s0 + k0 + min(il, nk - 1)];
+        auto prefetch_head = [&](int hh) {
             qf_next = load_frag<D>(gq + static_cast<int64_t>(q_row) * HD + hh * D, half);
             kf_next = load_frag<D>(gk + static_cast<int64_t>(k_row) * HD + hh * D, half);
             vv_next = *reinterpret_cast<const h8 *>(gv + static_cast<int64_t>(k_row) * HD + hh * D +
                                                     (D == 16 ? 8 * half : 0));
         };
-        prefetch_step(h_first, 0);
+        prefetch_head(0);
 
-        float m_run = -INFINITY, l_run = 0.0f;
-        float o_run[kOut];
+        for (int h = 0; h < H; ++h) {
+            // the packed row indices are loop invariant; hide that from the optimiser, which would
+            // otherwise hoist the ~300 LDS addresses derived from them out of the head loop and
+            // spill them all
 #pragma unroll
-        for (int t = 0; t < kOut; ++t) o_run[t] = 0.0f;
-        int h = h_first, kt_i = 0;
-        for (int step = 0; step < steps; ++step) {
-            const int k0 = kt_i * kTile;
-            const int nk = min(kTile, n_w - k0);
+            for (int t = 0; t < kIdxWords; ++t) asm volatile("" : "+v"(idx[t]));
             const frag_t qf = qf_next, kf = kf_next;
             const h8 vv = vv_next;
-            if (kt_i == 0) {
-                m_run = -INFINITY;
-                l_run = 0.0f;
-#pragma unroll
-                for (int t = 0; t < kOut; ++t) o_run[t] = 0.0f;
-            }
             // first axis' table fragments for this head, then the next step's q/k/v
             frag_t tq_cur[L::kTiles], tk_cur[L::kTiles];
             auto load_axis = [&](int n, frag_t *tq_dst, frag_t *tk_dst) {
@@ -257,16 +249,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 }
             };
             load_axis(0, tq_cur, tk_cur);
-            {
-                int hn = h, ktn = kt_i + 1;
-                if (ktn == nkt) {
-                    ktn = 0;
-                    ++hn;
-                }
-                if (step + 1 < steps) prefetch_step(hn, ktn);
-            }
-
-            if (!single_key_tile) build_pair_rows(k0, nk);
+            if (h + 1 < H) prefetch_head(h + 1);
 
             // V tile -> LDS, [key][D] halves
             wave_lds_fence();
@@ -336,8 +319,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
             for (int v = 0; v < 16; ++v)
                 if (key_of(v, half) < nk) mx = fmaxf(mx, lg[v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx);
-            const float scale = __expf(m_run - m_new);
+            const float m_new = mx;
             float p[16];
             float psum = 0.0f;
 #pragma unroll
@@ -346,8 +328,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 psum += p[v];
             }
             psum += __shfl_xor(psum, 32);
-            l_run = l_run * scale + psum;
-            m_run = m_new;
             // 2^-24 fixed-point image of the weights for the integer histogram (0 for dead slots)
             unsigned int pfix[16];
 #pragma unroll
@@ -355,8 +335,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 
             // value side: acc[c][i], c = 8*(v/4) + 4*half + v%4
             f16v acc = zero16;
-#pragma unroll
-            for (int t = 0; t < kOut; ++t) acc[t] = o_run[t] * scale;
 
             wave_lds_fence();   // V tile written above is visible to every lane
 #pragma unroll
@@ -424,29 +402,74 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 }
                 wave_lds_fence();
             }
+            if (q_valid) {
+                if (single_key_tile) {
+                    const float inv = 1.0f / psum;
+                    _Float16 *orow = gout + static_cast<int64_t>(q_row) * HD + h * D;
 #pragma unroll
-            for (int t = 0; t < kOut; ++t) o_run[t] = acc[t];
-
-            if (kt_i == nkt - 1 && q_valid) {
-                const float inv = 1.0f / l_run;
-                _Float16 *orow = gout + static_cast<int64_t>(q_row) * HD + h * D;
+                    for (int g = 0; g < D / 8; ++g) {   // registers 4g..4g+3 hold channels 8g + 4*half + e
+                        h4 ov;
 #pragma unroll
-                for (int g = 0; g < D / 8; ++g) {   // registers 4g..4g+3 hold channels 8g + 4*half + e
-                    h4 ov;
+                        for (int e = 0; e < 4; ++e) ov[e] = static_cast<_Float16>(acc[4 * g + e] * inv);
+                        *reinterpret_cast<h4 *>(orow + 8 * g + 4 * half) = ov;
+                    }
+                    if (half == 0) {
+                        if (a.out_max) a.out_max[static_cast<int64_t>(q_row) * H + h] = m_new;
+                        if (a.out_sum) a.out_sum[static_cast<int64_t>(q_row) * H + h] = psum;
+                    }
+                } else {
+                    // partial of this key tile: [sorted position][key tile][head][D channels, max, sum]
+                    float *part = a.partials +
+                                  ((static_cast<int64_t>(q_pos) * a.max_key_tiles + kt_i) * H + h) * (D + 2);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) ov[e] = static_cast<_Float16>(o_run[4 * g + e] * inv);
-                    *reinterpret_cast<h4 *>(orow + 8 * g + 4 * half) = ov;
+                    for (int g = 0; g < D / 8; ++g) {
+                        f4 ov = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+                        *reinterpret_cast<f4 *>(part + 8 * g + 4 * half) = ov;
+                    }
+                    if (half == 0) {
+                        part[D] = m_new;
+                        part[D + 1] = psum;
+                    }
                 }
-                if (half == 0) {
-                    if (a.out_max) a.out_max[static_cast<int64_t>(q_row) * H + h] = m_run;
-                    if (a.out_sum) a.out_sum[static_cast<int64_t>(q_row) * H + h] = l_run;
-                }
-            }
-            if (++kt_i == nkt) {
-                kt_i = 0;
-                ++h;
             }
         }
+    }
+}
+
+// Windows of more than 32 voxels: combine the per-key-tile partial results of every (voxel, head).
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_partials_kernel(AttnArgs a)
+{
+    const int w = blockIdx.x;
+    const int n_w = a.w_sizes[w];
+    const int nkt = (n_w + kTile - 1) / kTile;
+    if (nkt <= 1) return;
+    const int s0 = a.w2n[w];
+    const int H = a.H;
+    _Float16 *gout = static_cast<_Float16 *>(a.out);
+    for (int t = threadIdx.x; t < n_w * H; t += blockDim.x) {
+        const int i = t / H, h = t - i * H;
+        const float *part = a.partials + ((static_cast<int64_t>(s0 + i) * a.max_key_tiles) * H + h) * (D + 2);
+        const int64_t tile_stride = static_cast<int64_t>(H) * (D + 2);
+        float m = -INFINITY;
+        for (int kt = 0; kt < nkt; ++kt) m = fmaxf(m, part[kt * tile_stride + D]);
+        float l = 0.0f, o[D];
+#pragma unroll
+        for (int c = 0; c < D; ++c) o[c] = 0.0f;
+        for (int kt = 0; kt < nkt; ++kt) {
+            const float *pk = part + kt * tile_stride;
+            const float wgt = __expf(pk[D] - m);
+            l += pk[D + 1] * wgt;
+#pragma unroll
+            for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
+        }
+        const int row = a.n2n[s0 + i];
+        const float inv = 1.0f / l;
+        _Float16 *orow = gout + (static_cast<int64_t>(row) * H + h) * D;
+#pragma unroll
+        for (int c = 0; c < D; ++c) orow[c] = static_cast<_Float16>(o[c] * inv);
+        if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
+        if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
     }
 }
 
@@ -470,8 +493,7 @@ __global__ void transpose_value_table_kernel(AttnArgs a)
     }
 }
 
-// inclusive prefix sum of the work items of every window: 1 for a window of at most 32 voxels,
-// (query tiles x heads) for a larger one.  One workgroup; W is at most a few hundred thousand.
+// inclusive prefix sum of the work items of every window: (query tiles x key tiles).  One workgroup; W is at most a few hundred thousand.
 __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
 {
     __shared__ int part[1024];
@@ -482,7 +504,7 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
     int sum = 0;
     for (int w = begin; w < end; ++w) {
         const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
-        sum += tiles <= 1 ? 1 : tiles * a.H;
+        sum += tiles * tiles;
     }
     part[threadIdx.x] = sum;
     __syncthreads();
@@ -495,7 +517,7 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
     int run = part[threadIdx.x] - sum;
     for (int w = begin; w < end; ++w) {
         const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
-        run += tiles <= 1 ? 1 : tiles * a.H;
+        run += tiles * tiles;
         item_end[w] = run;
     }
     if (threadIdx.x == 0) item_end[W] = 0;   // the work counter of the attention kernel
@@ -535,6 +557,9 @@ int launch(const AttnArgs &a, hipStream_t stream)
     if (grid > need) grid = need;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kWaves * 64), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
+    if (a.max_key_tiles > 1)
+        hipLaunchKernelGGL(attn_merge_partials_kernel<D>, dim3(static_cast<unsigned>(a.W)), dim3(256), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }
 
@@ -569,9 +594,21 @@ size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
     return align_up(sizeof(_Float16) * static_cast<size_t>(H) * D * padded_rows, 256);
 }
 
-size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W)
+size_t attn_mfma_items_bytes(int64_t W)
 {
-    return attn_mfma_table_bytes(H, D, padded_rows) + align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 1), 256);
+    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 1), 256);
+}
+
+int attn_mfma_key_tiles(int max_window_voxels)
+{
+    return max_window_voxels <= kTile ? 1 : (max_window_voxels + kTile - 1) / kTile;
+}
+
+size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W, int64_t N, int max_window_voxels)
+{
+    const int tiles = attn_mfma_key_tiles(max_window_voxels);
+    const size_t partials = tiles <= 1 ? 0 : sizeof(float) * static_cast<size_t>(N) * tiles * H * (D + 2);
+    return attn_mfma_table_bytes(H, D, padded_rows) + attn_mfma_items_bytes(W) + align_up(partials, 256);
 }
 
 int launch_attn_mfma(const AttnArgs &a, hipStream_t stream)

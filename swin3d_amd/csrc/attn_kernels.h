@@ -16,7 +16,9 @@ struct AttnArgs {
     void *out;                             // [N,H,D]
     float *out_max, *out_sum;              // [N,H] or null
     void *workspace;                       // transposed value table (MFMA path) or null
-    void *items;                           // int32 [W] work-item prefix (MFMA path) or null
+    void *items;                           // int32 [W+1] work-item prefix + counter (MFMA path)
+    float *partials;                       // per-key-tile partial results of multi-tile windows
+    int32_t max_key_tiles;                 // key tiles of the largest window (stride of `partials`)
     int32_t H, D, nd, total_rows;
     int64_t N, W;
     int32_t rows[kMaxAxes];                // rows of each axis table
@@ -31,7 +33,9 @@ int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
-size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W);
+size_t attn_mfma_items_bytes(int64_t W);
+int attn_mfma_key_tiles(int max_window_voxels);
+size_t attn_mfma_workspace_bytes(int H, int D, int padded_rows, int64_t W, int64_t N, int max_window_voxels);
 int launch_attn_mfma(const AttnArgs &a, hipStream_t stream);
 
 }  // namespace s3d

@@ -80,7 +80,7 @@ def _host_table_sizes(table_sizes):
 
 
 def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
-                             n_coords, return_stats=False, force_generic=False):
+                             n_coords, return_stats=False, force_generic=False, max_window_voxels=None):
     """softmax-normalised window attention, [N,H,D] in the dtype of q.
 
     q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5)
@@ -91,6 +91,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
     force_generic  run the VALU kernel even where the MFMA kernel applies (fp16)
+    max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
+                   (set by build_window_index) or, failing that, read back from the device
     """
     _require_cuda("query", q)
     dev = q.device
@@ -122,6 +124,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             raise ValueError("the three tables must have the same number of elements")
     if table_len == 0 or table_len % (h * d) != 0:
         raise ValueError(f"table length {table_len} is not a positive multiple of H*D = {h * d}")
+    w_sizes_in = w_sizes
     w_sizes = _as_int32("w_sizes", w_sizes, dev)
     w2n = _as_int32("w2n_indices", w2n, dev)
     n2n = _as_int32("n2n_indices", n2n, dev)
@@ -136,9 +139,14 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     out = torch.empty_like(q)
     omax = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
+    if max_window_voxels is None:
+        max_window_voxels = getattr(w_sizes_in, "max_window_voxels", None)
+    if max_window_voxels is None:
+        max_window_voxels = int(w_sizes.max().item()) if w_sizes.numel() else 1
+    max_window_voxels = max(int(max_window_voxels), 1)
     lib = _lib.lib()
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, w_sizes.numel())
+        ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, w_sizes.numel(), max_window_voxels)
         workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
         status = lib.s3d_attn_fwd(
@@ -146,7 +154,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
             w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
-            n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype],
+            n, h, d, w_sizes.numel(), max_window_voxels, _DTYPE_CODE[q.dtype],
             _lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0, workspace.data_ptr(),
             ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")

@@ -69,8 +69,9 @@ def build_window_index(coords, stride, window_size, shift=0):
     if err:
         raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
                          "-8192..8191)")
-    return WindowIndex(n2n, wwid, w_sizes[:num_w], w2n[:num_w], int(num_w), int(num_m), int(max_w),
-                       int(window_size))
+    sizes = w_sizes[:num_w]
+    sizes.max_window_voxels = int(max_w)   # read by the attention op (sizes its partial-result workspace)
+    return WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window_size))
 
 
 def sparse_self_attention(w_w_id, w_sizes, protocol="v1"):
