@@ -553,7 +553,8 @@ int launch(const AttnArgs &a, hipStream_t stream)
     }
     const int per_cu = kLdsPerCu / lds > 0 ? static_cast<int>(kLdsPerCu / lds) : 1;
     int64_t grid = static_cast<int64_t>(cus) * per_cu;
-    const int64_t need = ceil_div(a.W, kWaves);
+    // never more wavefronts than work items (upper bound: every window as large as the largest)
+    const int64_t need = ceil_div(a.W * a.max_key_tiles * a.max_key_tiles, kWaves);
     if (grid > need) grid = need;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kWaves * 64), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
