@@ -1,6 +1,7 @@
 // Sparse-voxel windowed self-attention forward with cRSE tables: MFMA kernel (gfx950, fp16).
 //
-// One wavefront owns one window and walks it in 32-query x 32-key tiles.  For a tile and a head
+// A wavefront draws work items from a device-side queue.  An item is one 32-query x 32-key tile
+// pair of a window and a group of heads; for the tile pair and each head of the group
 //   S^T   = K Q^T                       one MFMA, lands directly in the logit registers
 //   QT_n  = Tq_n Q^T,  KT_n = Tk_n K^T  per signal axis n, MFMA -> LDS ("every table row
 //                                       against every query / key of the tile")
@@ -12,8 +13,8 @@
 // transposed copy of the value table.  P V is an MFMA as well.
 //
 // The histogram is accumulated with INTEGER LDS atomics on 2^-24 fixed point (softmax weights
-// are in [0,1], at most 32 of them meet in one bin): ds_add_u32 runs at full LDS rate while
-// ds_add_f32 measured about six times slower on this part.
+// are in [0,1], at most 32 of them meet in one bin): a wavefront's ds_add_u32 measured about
+// 5 clocks of the LDS pipe (a 4-byte gather: 2.7), ds_add_f32 many times more.
 //
 // Lane layout = the 32x32 MFMA accumulator layout: lane l holds query i = l % 32 and, in
 // register v, key j = 8*(v/4) + 4*(l/32) + v%4, so logits, softmax weights and the B operand
@@ -21,11 +22,13 @@
 // conflict-free for any row pattern), KT is stored [key][row] (one key per half-wave: the
 // gathers hit consecutive words of one row).
 //
-// The row indices depend on the pair only; they are computed once per tile (fp32, in the
+// The row indices depend on the pair only; they are computed once per item (fp32, in the
 // reference's operation order, Swin3D/src/attn/attn_utils.cuh:444-450) and kept as bytes in
-// registers across heads when the window has a single key tile.
+// registers across the heads of the item.  A window of at most 32 voxels is finished by its item;
+// a larger one leaves one partial result (max, sum, unnormalised output) per key tile and head,
+// which attn_merge_partials_kernel combines.
 //
-// Latency: a window is a long chain of small dependent steps, so every global load is issued
+// Latency: an item is a long chain of small dependent steps, so every global load is issued
 // one step ahead of its use (next head's q/k/v fragments, next axis' table fragments) and the
 // transposed value table of all heads sits in LDS, shared by the wavefronts of the workgroup.
 #include "attn_kernels.h"
@@ -41,6 +44,7 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr int kWaves = 8;             // wavefronts per workgroup (they share the value table in LDS)
 constexpr int kTile = 32;             // queries / keys per tile
 constexpr float kFix = 16777216.0f;   // 2^24 fixed point of the histogram
+constexpr int kItemsPerWave = 2;      // heads are grouped so that a wavefront draws about this many items
 
 // LDS operations of one wavefront execute in order; this only stops the compiler from moving
 // LDS accesses across the point where lanes exchange data (global loads stay free to move).
@@ -143,8 +147,12 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
     const _Float16 *gtk = static_cast<const _Float16 *>(a.table_k);
     _Float16 *gout = static_cast<_Float16 *>(a.out);
 
-    const int *item_end = static_cast<const int *>(a.items);   // inclusive prefix of items per window
-    const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]);
+    // work list written by window_items_kernel: inclusive prefix of (query tile, key tile) pairs per
+    // window, then the work counter, the number of head groups and the heads per group
+    const int *item_end = static_cast<const int *>(a.items);
+    const int groups = __builtin_amdgcn_readfirstlane(item_end[a.W + 1]);
+    const int group_heads = __builtin_amdgcn_readfirstlane(item_end[a.W + 2]);
+    const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]) * groups;
     // work items are handed out through a device counter (zeroed by window_items_kernel), so a
     // wavefront that drew long items simply draws fewer of them
     int *next_item = static_cast<int *>(a.items) + a.W;
@@ -165,22 +173,26 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
         if (lane == 0) item = atomicAdd(next_item, 1);
         item = __builtin_amdgcn_readfirstlane(item);
         if (item >= total_items) break;
-        // window of this item: first w with item_end[w] > item
+        // item = (tile pair, head group); consecutive items share the tile pair
+        const int pair = item / groups;
+        const int h_begin = (item - pair * groups) * group_heads;
+        const int h_end = min(H, h_begin + group_heads);
+        // window of this tile pair: first w with item_end[w] > pair
         int lo = 0, hi = static_cast<int>(a.W) - 1;
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
-            if (__builtin_amdgcn_readfirstlane(item_end[mid]) > item) hi = mid; else lo = mid + 1;
+            if (__builtin_amdgcn_readfirstlane(item_end[mid]) > pair) hi = mid; else lo = mid + 1;
         }
         const int w = lo;
         const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         const int nkt = (n_w + kTile - 1) / kTile;   // key tiles (= query tiles)
         const bool single_key_tile = nkt == 1;
-        // one item = one (query tile, key tile) pair of a window, all heads: the pair row indices
-        // are computed once and reused by every head.  A window of at most 32 voxels is a single
-        // item that writes the final output; larger windows write per-key-tile partial results
+        // one item = one (query tile, key tile) pair of a window and a group of heads: the pair row
+        // indices are computed once and reused by every head of the group.  A window of at most 32
+        // voxels writes the final output; larger windows write per-key-tile partial results
         // (running max, sum, unnormalised output) that attn_merge_partials_kernel combines.
-        const int local = item - (w > 0 ? __builtin_amdgcn_readfirstlane(item_end[w - 1]) : 0);
+        const int local = pair - (w > 0 ? __builtin_amdgcn_readfirstlane(item_end[w - 1]) : 0);
         const int q0 = (local / nkt) * kTile;
         const int kt_i = local % nkt;
         const int k0 = kt_i * kTile;
@@ -227,9 +239,9 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
             vv_next = *reinterpret_cast<const h8 *>(gv + static_cast<int64_t>(k_row) * HD + hh * D +
                                                     (D == 16 ? 8 * half : 0));
         };
-        prefetch_head(0);
+        prefetch_head(h_begin);
 
-        for (int h = 0; h < H; ++h) {
+        for (int h = h_begin; h < h_end; ++h) {
             // the packed row indices are loop invariant; hide that from the optimiser, which would
             // otherwise hoist the ~300 LDS addresses derived from them out of the head loop and
             // spill them all
@@ -249,7 +261,7 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                 }
             };
             load_axis(0, tq_cur, tk_cur);
-            if (h + 1 < H) prefetch_head(h + 1);
+            if (h + 1 < h_end) prefetch_head(h + 1);
 
             // V tile -> LDS, [key][D] halves
             wave_lds_fence();
@@ -437,40 +449,45 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 }
 
 // Windows of more than 32 voxels: combine the per-key-tile partial results of every (voxel, head).
+// One thread per (sorted position, head); the window of a position is found by bisection of w2n.
 template <int D>
 __global__ __launch_bounds__(256) void attn_merge_partials_kernel(AttnArgs a)
 {
-    const int w = blockIdx.x;
-    const int n_w = a.w_sizes[w];
-    const int nkt = (n_w + kTile - 1) / kTile;
-    if (nkt <= 1) return;
-    const int s0 = a.w2n[w];
     const int H = a.H;
-    _Float16 *gout = static_cast<_Float16 *>(a.out);
-    for (int t = threadIdx.x; t < n_w * H; t += blockDim.x) {
-        const int i = t / H, h = t - i * H;
-        const float *part = a.partials + ((static_cast<int64_t>(s0 + i) * a.max_key_tiles) * H + h) * (D + 2);
-        const int64_t tile_stride = static_cast<int64_t>(H) * (D + 2);
-        float m = -INFINITY;
-        for (int kt = 0; kt < nkt; ++kt) m = fmaxf(m, part[kt * tile_stride + D]);
-        float l = 0.0f, o[D];
-#pragma unroll
-        for (int c = 0; c < D; ++c) o[c] = 0.0f;
-        for (int kt = 0; kt < nkt; ++kt) {
-            const float *pk = part + kt * tile_stride;
-            const float wgt = __expf(pk[D] - m);
-            l += pk[D + 1] * wgt;
-#pragma unroll
-            for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
-        }
-        const int row = a.n2n[s0 + i];
-        const float inv = 1.0f / l;
-        _Float16 *orow = gout + (static_cast<int64_t>(row) * H + h) * D;
-#pragma unroll
-        for (int c = 0; c < D; ++c) orow[c] = static_cast<_Float16>(o[c] * inv);
-        if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
-        if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= a.N * H) return;
+    const int pos = static_cast<int>(t / H), h = static_cast<int>(t - static_cast<int64_t>(pos) * H);
+    int lo = 0, hi = static_cast<int>(a.W) - 1;   // last window that starts at or before pos
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (a.w2n[mid] <= pos) lo = mid; else hi = mid - 1;
     }
+    const int nkt = (a.w_sizes[lo] + kTile - 1) / kTile;
+    if (nkt <= 1) return;
+    const float *part = a.partials + ((static_cast<int64_t>(pos) * a.max_key_tiles) * H + h) * (D + 2);
+    const int64_t tile_stride = static_cast<int64_t>(H) * (D + 2);
+    float m = -INFINITY;
+    for (int kt = 0; kt < nkt; ++kt) m = fmaxf(m, part[kt * tile_stride + D]);
+    float l = 0.0f, o[D];
+#pragma unroll
+    for (int c = 0; c < D; ++c) o[c] = 0.0f;
+    for (int kt = 0; kt < nkt; ++kt) {
+        const float *pk = part + kt * tile_stride;
+        const float wgt = __expf(pk[D] - m);
+        l += pk[D + 1] * wgt;
+#pragma unroll
+        for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
+    }
+    const int row = a.n2n[pos];
+    const float inv = 1.0f / l;
+    _Float16 *orow = static_cast<_Float16 *>(a.out) + (static_cast<int64_t>(row) * H + h) * D;
+    _Float16 ov[D];
+#pragma unroll
+    for (int c = 0; c < D; ++c) ov[c] = static_cast<_Float16>(o[c] * inv);
+#pragma unroll
+    for (int g = 0; g < D / 8; ++g) *reinterpret_cast<h8 *>(orow + 8 * g) = *reinterpret_cast<const h8 *>(ov + 8 * g);
+    if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
+    if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
 }
 
 // value table [axis][row][h][c] -> [h][c][padded row], every axis padded to a multiple of 16 rows
@@ -493,7 +510,9 @@ __global__ void transpose_value_table_kernel(AttnArgs a)
     }
 }
 
-// inclusive prefix sum of the work items of every window: (query tiles x key tiles).  One workgroup; W is at most a few hundred thousand.
+// Work list of the attention kernel: inclusive prefix sum of the (query tile, key tile) pairs of every
+// window, the work counter and the split of the heads into groups.  One workgroup; W is at most a few
+// hundred thousand.
 __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
 {
     __shared__ int part[1024];
@@ -520,7 +539,17 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
         run += tiles * tiles;
         item_end[w] = run;
     }
-    if (threadIdx.x == 0) item_end[W] = 0;   // the work counter of the attention kernel
+    if (threadIdx.x == 1023) {
+        // heads are split into groups when the tile pairs alone are too few to keep every wavefront
+        // of the persistent grid busy with several items (deep stages: few, large windows, many heads)
+        const int pairs = part[1023];
+        int groups = pairs > 0 ? (a.target_items + pairs - 1) / pairs : 1;
+        groups = max(1, min(groups, a.H));
+        const int group_heads = (a.H + groups - 1) / groups;
+        item_end[W] = 0;   // the work counter of the attention kernel
+        item_end[W + 1] = (a.H + group_heads - 1) / group_heads;
+        item_end[W + 2] = group_heads;
+    }
 }
 
 size_t lds_bytes(const AttnArgs &a, int wave_words, bool tvt_lds)
@@ -532,8 +561,9 @@ size_t lds_bytes(const AttnArgs &a, int wave_words, bool tvt_lds)
 constexpr size_t kLdsPerCu = 160 * 1024;
 
 template <int D, int ND, int RMAX, bool TVT_LDS>
-int launch(const AttnArgs &a, hipStream_t stream)
+int launch(const AttnArgs &args, hipStream_t stream)
 {
+    AttnArgs a = args;
     auto kernel = attn_fwd_mfma_kernel<D, ND, RMAX, TVT_LDS>;
     const size_t lds = lds_bytes(a, WaveLds<RMAX>::kWords, TVT_LDS);
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -541,8 +571,6 @@ int launch(const AttnArgs &a, hipStream_t stream)
     const int64_t cells = static_cast<int64_t>(a.H) * a.D * a.padded_rows;
     hipLaunchKernelGGL(transpose_value_table_kernel, dim3(static_cast<unsigned>(ceil_div(cells, 256))),
                        dim3(256), 0, stream, a);
-    S3D_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(window_items_kernel, dim3(1), dim3(1024), 0, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     // persistent grid: as many workgroups as fit the chip at once (LDS-bound), never more than the
     // windows can feed; wavefronts pull items in a strided loop
@@ -553,13 +581,18 @@ int launch(const AttnArgs &a, hipStream_t stream)
     }
     const int per_cu = kLdsPerCu / lds > 0 ? static_cast<int>(kLdsPerCu / lds) : 1;
     int64_t grid = static_cast<int64_t>(cus) * per_cu;
-    // never more wavefronts than work items (upper bound: every window as large as the largest)
-    const int64_t need = ceil_div(a.W * a.max_key_tiles * a.max_key_tiles, kWaves);
+    a.target_items = static_cast<int>(grid) * kWaves * kItemsPerWave;
+    hipLaunchKernelGGL(window_items_kernel, dim3(1), dim3(1024), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    // never more wavefronts than work items (upper bound: every window as large as the largest,
+    // every head an item of its own)
+    const int64_t need = ceil_div(a.W * a.max_key_tiles * a.max_key_tiles * a.H, kWaves);
     if (grid > need) grid = need;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kWaves * 64), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     if (a.max_key_tiles > 1)
-        hipLaunchKernelGGL(attn_merge_partials_kernel<D>, dim3(static_cast<unsigned>(a.W)), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL(attn_merge_partials_kernel<D>, dim3(static_cast<unsigned>(ceil_div(a.N * a.H, 256))),
+                           dim3(256), 0, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }
@@ -597,7 +630,7 @@ size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
 
 size_t attn_mfma_items_bytes(int64_t W)
 {
-    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 1), 256);
+    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 3), 256);
 }
 
 int attn_mfma_key_tiles(int max_window_voxels)

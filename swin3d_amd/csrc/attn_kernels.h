@@ -19,6 +19,7 @@ struct AttnArgs {
     void *items;                           // int32 [W+1] work-item prefix + counter (MFMA path)
     float *partials;                       // per-key-tile partial results of multi-tile windows
     int32_t max_key_tiles;                 // key tiles of the largest window (stride of `partials`)
+    int32_t target_items;                  // work items the launch wants at least (heads are split to reach it)
     int32_t H, D, nd, total_rows;
     int64_t N, W;
     int32_t rows[kMaxAxes];                // rows of each axis table
