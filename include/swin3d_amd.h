@@ -77,11 +77,11 @@ const char *s3d_last_error_string(void);
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
  *   max_window_voxels  an upper bound of every w_sizes entry (e.g. counts[2] of s3d_window_index, or
  *                  window^3).  It sizes the per-key-tile partial results of windows with more than 32
- *                  voxels; a window larger than the bound would write outside the workspace, so
- *                  the bound must hold.
+ *                  voxels; a window larger than the bound is skipped (its output rows are not
+ *                  written), so the bound must hold for a complete result.
  *   flags          0, or S3D_ATTN_FORCE_GENERIC to run the VALU kernel for every case
  *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
- *                  (MFMA kernel: a transposed copy of the value table, the work-item prefix, and
+ *                  (MFMA kernel: a transposed copy of the value table, the work list, and
  *                  N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
  *                  max_window_voxels > 32)
  *   D in {8,16}, nd in {3,6,9}, H >= 1.

@@ -188,6 +188,8 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         const int nkt = (n_w + kTile - 1) / kTile;   // key tiles (= query tiles)
         const bool single_key_tile = nkt == 1;
+        // a window beyond the caller's size bound has no room for its partial results: leave it out
+        if (nkt > a.max_key_tiles) continue;
         // one item = one (query tile, key tile) pair of a window and a group of heads: the pair row
         // indices are computed once and reused by every head of the group.  A window of at most 32
         // voxels writes the final output; larger windows write per-key-tile partial results
@@ -430,9 +432,10 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
                         if (a.out_sum) a.out_sum[static_cast<int64_t>(q_row) * H + h] = psum;
                     }
                 } else {
-                    // partial of this key tile: [sorted position][key tile][head][D channels, max, sum]
+                    // partial of this key tile: [key tile][head][sorted position][D channels, max, sum];
+                    // the 32 queries of the tile fill one contiguous run
                     float *part = a.partials +
-                                  ((static_cast<int64_t>(q_pos) * a.max_key_tiles + kt_i) * H + h) * (D + 2);
+                                  ((static_cast<int64_t>(kt_i) * H + h) * a.N + q_pos) * (D + 2);
 #pragma unroll
                     for (int g = 0; g < D / 8; ++g) {
                         f4 ov = {acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
@@ -456,16 +459,17 @@ __global__ __launch_bounds__(256) void attn_merge_partials_kernel(AttnArgs a)
     const int H = a.H;
     const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (t >= a.N * H) return;
-    const int pos = static_cast<int>(t / H), h = static_cast<int>(t - static_cast<int64_t>(pos) * H);
+    // position fastest: neighbouring threads read neighbouring partial records
+    const int h = static_cast<int>(t / a.N), pos = static_cast<int>(t - static_cast<int64_t>(h) * a.N);
     int lo = 0, hi = static_cast<int>(a.W) - 1;   // last window that starts at or before pos
     while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
         if (a.w2n[mid] <= pos) lo = mid; else hi = mid - 1;
     }
     const int nkt = (a.w_sizes[lo] + kTile - 1) / kTile;
-    if (nkt <= 1) return;
-    const float *part = a.partials + ((static_cast<int64_t>(pos) * a.max_key_tiles) * H + h) * (D + 2);
-    const int64_t tile_stride = static_cast<int64_t>(H) * (D + 2);
+    if (nkt <= 1 || nkt > a.max_key_tiles) return;
+    const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
+    const int64_t tile_stride = static_cast<int64_t>(H) * a.N * (D + 2);
     float m = -INFINITY;
     for (int kt = 0; kt < nkt; ++kt) m = fmaxf(m, part[kt * tile_stride + D]);
     float l = 0.0f, o[D];

@@ -114,6 +114,30 @@ def test_stats_outputs(oracle_lib, hip_lib):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
+def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib):
+    """max_window_voxels below the real maximum: windows beyond the bound are left out (their output
+    rows keep what the buffer held), every other window is complete, nothing is written out of bounds."""
+    import swin3d_amd
+    case = make_attn_case(oracle_lib, seed=38, n=1000, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
+    to_half_and_back(_sharp16(case))
+    w_sizes = case.index["w_sizes"]
+    assert w_sizes.max() > 32 and (w_sizes <= 32).any()
+    ref = oracle_lib.attn_fwd(*case.oracle_args())
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    h = lambda a: t(a).half()
+    i = case.index
+    got = swin3d_amd.window_attention_forward(
+        h(case.q), h(case.k), h(case.v), h(case.tq), h(case.tk), h(case.tv), t(case.table_sizes),
+        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32)
+    torch.cuda.synchronize()
+    got = got.double().cpu().numpy()
+    small = np.repeat(w_sizes <= 32, w_sizes)           # per sorted position
+    rows_small = i["n2n"][small]
+    from gpu_helpers import assert_attn_close
+    assert_attn_close(got[rows_small], ref[rows_small], torch.float16)
+
+
 def test_empty_input(hip_lib):
     import swin3d_amd
     dev = torch.device("cuda")
