@@ -36,6 +36,7 @@ def lib():
             "s3d_oracle_crse_rows",
             "s3d_oracle_attn_fwd_f64",
             "s3d_oracle_attn_fwd_f32",
+            "s3d_oracle_attn_bwd_f64",
             "s3d_oracle_knn",
             "s3d_oracle_knn_heap",
             "s3d_oracle_max_threads",
@@ -133,6 +134,29 @@ def attn_fwd(q, k, v, tq, tk, tv, table_sizes, w_sizes, w2n, n2n, n_coords, acc=
     if return_stats:
         return out, omax, osum, int(edges[0])
     return out
+
+
+def attn_bwd(q, k, v, tq, tk, tv, table_sizes, w_sizes, w2n, n2n, n_coords, dout):
+    """Attention backward in float64 -> (dq, dk, dv [N,H,D], dtq, dtk, dtv [table_len])."""
+    q, k, v, dout = (_c(x, np.float32) for x in (q, k, v, dout))
+    tq, tk, tv = (_c(x, np.float32).reshape(-1) for x in (tq, tk, tv))
+    table_sizes = _c(table_sizes, np.int32)
+    w_sizes, w2n, n2n = (_c(x, np.int32) for x in (w_sizes, w2n, n2n))
+    n_coords = _c(n_coords, np.float32)
+    n, h, d = q.shape
+    nd = table_sizes.shape[0]
+    assert dout.shape == q.shape and n_coords.shape == (n, nd)
+    assert tq.shape[0] == int(table_sizes.sum()) == tk.shape[0] == tv.shape[0]
+    assert int(w_sizes.sum()) == n and n2n.shape[0] == n
+    dq, dk, dv = (np.zeros((n, h, d), np.float64) for _ in range(3))
+    dtq, dtk, dtv = (np.zeros(tq.shape[0], np.float64) for _ in range(3))
+    rc = lib().s3d_oracle_attn_bwd_f64(
+        _p(q), _p(k), _p(v), _p(tq), _p(tk), _p(tv), _p(table_sizes), ctypes.c_int32(nd), _p(w_sizes),
+        _p(w2n), _p(n2n), _p(n_coords), _p(dout), _p(dq), _p(dk), _p(dv), _p(dtq), _p(dtk), _p(dtv),
+        ctypes.c_int64(n), ctypes.c_int32(h), ctypes.c_int32(d), ctypes.c_int64(w_sizes.shape[0]))
+    if rc != 0:
+        raise ValueError(f"s3d_oracle_attn_bwd failed: {rc}")
+    return dq, dk, dv, dtq, dtk, dtv
 
 
 def knn(k, src_xyz, query_xyz, src_offset, query_offset, heap_order=False, num_threads=None):

@@ -17,6 +17,8 @@
  *                            :111-188 (exp / accumulate pass),
  *                            Swin3D/src/attn/attn_utils.cuh:455-464 (table sum),
  *                            Swin3D/sparse_dl/attn/attn_coff.py:180-184 (raw / sum)
+ *   s3d_oracle_attn_bwd_f64  Swin3D/src/attn/self_attn_aio_bwd.cu:14-113,
+ *                            Swin3D/sparse_dl/attn/attn_coff.py:191-232
  *   s3d_oracle_knn           Swin3D/src/knn/knn_cuda_kernel.cu:139-204 with the
  *                            canonical (distance, index) order instead of heap order
  *   s3d_oracle_knn_heap      Swin3D/src/knn/knn_cuda_kernel.cu:29-62, 139-204, faithful
@@ -222,6 +224,137 @@ int s3d_oracle_crse_rows(const float *n_coords, int32_t nd, const int32_t *table
 #undef S3D_ATTN_NAME
 #undef S3D_ATTN_ACC
 #undef S3D_ATTN_EXP
+
+/*
+ * Attention backward (double accumulation).
+ *
+ * Follows Swin3D/sparse_dl/attn/attn_coff.py:191-232 and
+ * Swin3D/src/attn/self_attn_aio_bwd.cu:14-113 in the reference's own terms:
+ *   raw_i        = out_i * sum_i                                    (attn_coff.py:219)
+ *   sum_grad_i   = - sum_c raw_i[c] / sum_i^2 * dout_i[c]           (cal_exp_sum_grad_kernel, bwd.cu:38)
+ *   exp_ij       = exp(logit_ij - max_i),  norm_ij = exp_ij / sum_i (bwd.cu:91-92)
+ *   value_ij     = v_j + Tv(i,j)
+ *   dv_j, dTv rows  += dout_i * norm_ij                             (bwd.cu:99-101)
+ *   coff_grad_ij = (sum_c dout_i[c] value_ij[c] / sum_i + sum_grad_i) * exp_ij   (bwd.cu:103-106)
+ *   dk_j += coff_grad (q_i + Tk(i,j));  dq_i += coff_grad (k_j + Tq(i,j))        (bwd.cu:107-108)
+ *   dTq rows += coff_grad q_i;  dTk rows += coff_grad k_j                        (bwd.cu:109-110)
+ * max_i and sum_i are recomputed here (the reference passes the forward's tensors in).
+ * dq, dk, dv [N,H,D] and dtq, dtk, dtv [table_len] are overwritten.
+ * Pinned by automatic differentiation of an independent dense statement of the forward
+ * (tests/test_oracle_attn_bwd.py) and by central differences of the forward oracle.
+ */
+int s3d_oracle_attn_bwd_f64(const float *q, const float *k, const float *v, const float *tq, const float *tk,
+                            const float *tv, const int32_t *table_sizes, int32_t nd, const int32_t *w_sizes,
+                            const int32_t *w2n, const int32_t *n2n, const float *n_coords, const float *dout,
+                            double *dq, double *dk, double *dv, double *dtq, double *dtk, double *dtv,
+                            int64_t N, int32_t H, int32_t D, int64_t W)
+{
+    if (nd < 1 || nd > S3D_MAX_ND || H < 1 || D < 1) return -1;
+    const int32_t HD = H * D;
+    int32_t base[S3D_MAX_ND], rowsz[S3D_MAX_ND];
+    int64_t table_len = 0;
+    for (int n = 0; n < nd; ++n) {
+        if (table_sizes[n] <= 0 || table_sizes[n] % HD != 0) return -3;
+        base[n] = (int32_t)table_len;
+        rowsz[n] = table_sizes[n] / HD;
+        table_len += table_sizes[n];
+    }
+    memset(dq, 0, sizeof(double) * (size_t)N * HD);
+    memset(dk, 0, sizeof(double) * (size_t)N * HD);
+    memset(dv, 0, sizeof(double) * (size_t)N * HD);
+    memset(dtq, 0, sizeof(double) * (size_t)table_len);
+    memset(dtk, 0, sizeof(double) * (size_t)table_len);
+    memset(dtv, 0, sizeof(double) * (size_t)table_len);
+    for (int64_t w = 0; w < W; ++w) {
+        const int64_t s0 = w2n[w];
+        const int64_t n_w = w_sizes[w];
+        double *logit = (double *)malloc(sizeof(double) * (size_t)(n_w > 0 ? n_w : 1));
+        int32_t *rows = (int32_t *)malloc(sizeof(int32_t) * (size_t)(n_w > 0 ? n_w : 1) * (size_t)nd);
+        double *bq = (double *)malloc(sizeof(double) * 3 * (size_t)D);
+        double *bk = bq + D, *bv = bk + D;
+        for (int64_t a = 0; a < n_w; ++a) {
+            const int64_t i = s0 + a;
+            const int64_t qi = n2n[i];
+            for (int64_t b = 0; b < n_w; ++b) {
+                int e = 0;
+                for (int n = 0; n < nd; ++n)
+                    rows[b * nd + n] = crse_row(n_coords[i * nd + n], n_coords[(s0 + b) * nd + n], rowsz[n], &e);
+            }
+            for (int32_t h = 0; h < H; ++h) {
+                const float *qv = q + qi * HD + h * D;
+                const float *go = dout + qi * HD + h * D;
+                /* forward quantities of the row: logits, max, sum, unnormalised output */
+                double mx = -INFINITY;
+                for (int64_t b = 0; b < n_w; ++b) {
+                    const float *kv = k + (int64_t)n2n[s0 + b] * HD + h * D;
+                    double l = 0;
+                    for (int32_t c = 0; c < D; ++c) {
+                        double tq_c = 0, tk_c = 0;
+                        for (int n = 0; n < nd; ++n) {
+                            const int64_t f = (int64_t)base[n] + (int64_t)rows[b * nd + n] * HD + h * D + c;
+                            tq_c += (double)tq[f];
+                            tk_c += (double)tk[f];
+                        }
+                        l += (double)qv[c] * (double)kv[c] + (double)qv[c] * tq_c + (double)kv[c] * tk_c;
+                    }
+                    logit[b] = l;
+                    if (l > mx) mx = l;
+                }
+                double sum = 0, raw_dot = 0;
+                for (int64_t b = 0; b < n_w; ++b) sum += exp(logit[b] - mx);
+                for (int64_t b = 0; b < n_w; ++b) {
+                    const float *vv = v + (int64_t)n2n[s0 + b] * HD + h * D;
+                    const double e = exp(logit[b] - mx);
+                    for (int32_t c = 0; c < D; ++c) {
+                        double tv_c = 0;
+                        for (int n = 0; n < nd; ++n)
+                            tv_c += (double)tv[(int64_t)base[n] + (int64_t)rows[b * nd + n] * HD + h * D + c];
+                        raw_dot += e * ((double)vv[c] + tv_c) * (double)go[c];
+                    }
+                }
+                const double sum_grad = -raw_dot / (sum * sum);
+                for (int64_t b = 0; b < n_w; ++b) {
+                    const int64_t kj = n2n[s0 + b];
+                    const float *kv = k + kj * HD + h * D;
+                    const float *vv = v + kj * HD + h * D;
+                    for (int32_t c = 0; c < D; ++c) {
+                        bq[c] = bk[c] = bv[c] = 0;
+                        for (int n = 0; n < nd; ++n) {
+                            const int64_t f = (int64_t)base[n] + (int64_t)rows[b * nd + n] * HD + h * D + c;
+                            bq[c] += (double)tq[f];
+                            bk[c] += (double)tk[f];
+                            bv[c] += (double)tv[f];
+                        }
+                    }
+                    const double e = exp(logit[b] - mx);
+                    const double norm = e / sum;
+                    double pv = 0;
+                    for (int32_t c = 0; c < D; ++c) {
+                        const double vg = (double)go[c] * norm;
+                        dv[kj * HD + h * D + c] += vg;
+                        for (int n = 0; n < nd; ++n)
+                            dtv[(int64_t)base[n] + (int64_t)rows[b * nd + n] * HD + h * D + c] += vg;
+                        pv += (double)go[c] * ((double)vv[c] + bv[c]) / sum;
+                    }
+                    const double cg = (pv + sum_grad) * e;
+                    for (int32_t c = 0; c < D; ++c) {
+                        dk[kj * HD + h * D + c] += cg * ((double)qv[c] + bk[c]);
+                        dq[qi * HD + h * D + c] += cg * ((double)kv[c] + bq[c]);
+                        for (int n = 0; n < nd; ++n) {
+                            const int64_t f = (int64_t)base[n] + (int64_t)rows[b * nd + n] * HD + h * D + c;
+                            dtq[f] += cg * (double)qv[c];
+                            dtk[f] += cg * (double)kv[c];
+                        }
+                    }
+                }
+            }
+        }
+        free(logit);
+        free(rows);
+        free(bq);
+    }
+    return 0;
+}
 
 /* ------------------------------------------------------------------------- */
 /* KNN                                                                       */
