@@ -109,6 +109,35 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
                  int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Windowed self-attention backward.
+ *
+ * Replaces cal_exp_sum_grads and self_attn_indir_backward
+ * (Swin3D/src/attn/self_attn_aio_bwd.cu:14-47 and :49-113, 197-509; called from
+ * Swin3D/sparse_dl/attn/attn_coff.py:219-224) for pos_mode SEPARATE and indice_mode INDIRECT,
+ * without the O(M) pair arrays.  Arithmetic is fp32 for both dtypes.
+ *
+ *   q .. n_coords  as for s3d_attn_fwd (the forward's inputs)
+ *   out, out_max, out_sum   the forward's outputs for the same inputs (out of `dtype`, statistics fp32):
+ *                  the tensors the reference saves for backward (attn_coff.py:186-187)
+ *   dout           device [N,H,D] of `dtype`: gradient of the loss w.r.t. `out`
+ *   dq, dk, dv     device [N,H,D] of `dtype`, overwritten (every row belongs to exactly one window)
+ *   dtable_q/k/v   device FP32 [table_len], overwritten; layout of the tables
+ *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, N, W) bytes
+ *   D in {8,16}, nd in {3,6,9}, every axis table of at most 64 rows.
+ *
+ * dq, dk, dv are sums in a fixed order (deterministic); the table gradients are accumulated per
+ * wavefront and added to global memory with fp32 atomics (order varies between runs).
+ */
+size_t s3d_attn_bwd_workspace_bytes(int32_t H, int64_t N, int64_t W);
+int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
+                 const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
+                 const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords,
+                 const void *out, const float *out_max, const float *out_sum, const void *dout, void *dq,
+                 void *dk, void *dv, float *dtable_q, float *dtable_k, float *dtable_v, int64_t N,
+                 int32_t H, int32_t D, int64_t W, int32_t dtype, void *workspace, size_t workspace_bytes,
+                 void *stream);
+
+/*
  * Window sort + segment offsets.
  *
  * Replaces BasicLayer.get_map_pair / get_window_mapping

@@ -1,0 +1,579 @@
+// Sparse-voxel windowed self-attention BACKWARD with cRSE tables (gfx950): fp32 arithmetic, fp16 or fp32 I/O.
+//
+// Math (Swin3D/src/attn/self_attn_aio_bwd.cu:14-113, Swin3D/sparse_dl/attn/attn_coff.py:191-232), per
+// window, head h, query i, key j, with P = softmax weights and o the forward output:
+//   dP(i,j) = dout_i . (v_j + Tv(i,j))            dL(i,j) = P(i,j) (dP(i,j) - dout_i . o_i)
+//   dv_j  += P dout_i                              dTv[n][row_n(i,j)] += P dout_i
+//   dq_i  += dL (k_j + Tq(i,j))                    dTq[n][row_n(i,j)] += dL q_i
+//   dk_j  += dL (q_i + Tk(i,j))                    dTk[n][row_n(i,j)] += dL k_j
+// The reference adds every term with a global atomic.  Here every output element has ONE owner:
+//
+//  * a key-owned sweep gives a lane one key j and streams the window's queries through the wavefront:
+//    dk_j, dv_j accumulate in the lane's registers and are stored once;
+//  * a query-owned sweep gives a lane one query i and streams the keys: dq_i likewise;
+//  * table gradients: within one step of a sweep the streamed side is the same for all lanes (q_i and
+//    dout_i in the key-owned sweep, k_j in the query-owned one), so
+//        dTq[n][r] += (sum over lanes with row_n = r of dL) * q_i
+//    is a histogram over table rows (integer LDS atomics, one per pair and axis, on a fixed-point image
+//    scaled by the largest |dL| of the step) followed by a rank-1 update in which lane r owns row r.
+//    The wavefront keeps its table gradients in registers for all the units it processes and adds them
+//    to the global tables once, at the end (a workgroup works on one head for its whole life and keeps
+//    that head's slices of the three tables in LDS).
+//
+// Windows of at most 32 voxels put two streamed elements in one wavefront step (two 32-lane groups).
+#include "attn_kernels.h"
+
+#include <hip/hip_fp16.h>
+
+namespace s3d {
+namespace {
+
+constexpr int kBwdThreads = 256;
+constexpr int kBwdWaves = kBwdThreads / 64;
+constexpr int kChunk = 64;            // owned elements per unit = lanes of a wavefront
+constexpr float kFixP = 16777216.0f;  // 2^24: softmax weights of one query sum to at most 1
+constexpr float kFixL = 8388608.0f;   // 2^23: |dL| / max|dL| <= 1, at most 64 lanes meet in one bin
+
+struct BwdArgs {
+    const void *q, *k, *v, *table_q, *table_k, *table_v, *dout, *out;
+    const float *out_max, *out_sum;
+    const int32_t *w_sizes, *w2n, *n2n;
+    const float *n_coords;
+    void *dq, *dk, *dv;
+    float *dtq, *dtk, *dtv;
+    float *delta;     // [N,H] dout_i . o_i
+    int32_t *units;   // [W] inclusive prefix of 64-element chunks per window, then H work counters
+    int32_t H, D, nd, total_rows;
+    int64_t N, W, table_len;
+    int32_t rows[kMaxAxes];
+    int32_t base[kMaxAxes];
+};
+
+__device__ __forceinline__ void wave_lds_fence()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+
+template <int D> __device__ __forceinline__ void load_row(const float *p, float *dst)
+{
+#pragma unroll
+    for (int c = 0; c < D; c += 4) {
+        const float4 x = *reinterpret_cast<const float4 *>(p + c);
+        dst[c] = x.x; dst[c + 1] = x.y; dst[c + 2] = x.z; dst[c + 3] = x.w;
+    }
+}
+template <int D> __device__ __forceinline__ void load_row(const __half *p, float *dst)
+{
+#pragma unroll
+    for (int c = 0; c < D; c += 8) {
+        const uint4 x = *reinterpret_cast<const uint4 *>(p + c);
+        const __half2 *hh = reinterpret_cast<const __half2 *>(&x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float2 f = __half22float2(hh[e]);
+            dst[c + 2 * e] = f.x;
+            dst[c + 2 * e + 1] = f.y;
+        }
+    }
+}
+template <int D> __device__ __forceinline__ void store_row(float *p, const float *src)
+{
+#pragma unroll
+    for (int c = 0; c < D; c += 4) *reinterpret_cast<float4 *>(p + c) = make_float4(src[c], src[c + 1], src[c + 2], src[c + 3]);
+}
+template <int D> __device__ __forceinline__ void store_row(__half *p, const float *src)
+{
+#pragma unroll
+    for (int c = 0; c < D; c += 8) {
+        uint4 x;
+        __half2 *hh = reinterpret_cast<__half2 *>(&x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) hh[e] = __floats2half2_rn(src[c + 2 * e], src[c + 2 * e + 1]);
+        *reinterpret_cast<uint4 *>(p + c) = x;
+    }
+}
+__device__ __forceinline__ float as_float(float x) { return x; }
+__device__ __forceinline__ float as_float(__half x) { return __half2float(x); }
+
+__device__ __forceinline__ int crse_row(float ci, float cj, int rows)
+{
+    float rel = ci - cj;
+    rel = rel + static_cast<float>(rows / 2);
+    rel = fminf(fmaxf(rel, 0.0f), static_cast<float>(rows));
+    return min(static_cast<int>(rel), rows - 1);
+}
+
+// delta[i][h] = dout_i . o_i; the table gradients and the work counters start at zero
+template <typename T>
+__global__ void bwd_prepare_kernel(BwdArgs a)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const T *go = static_cast<const T *>(a.dout);
+    const T *o = static_cast<const T *>(a.out);
+    for (int64_t t = t0; t < a.N * a.H; t += stride) {
+        float s = 0.0f;
+        for (int c = 0; c < a.D; ++c) s += as_float(go[t * a.D + c]) * as_float(o[t * a.D + c]);
+        a.delta[t] = s;
+    }
+    for (int64_t t = t0; t < a.table_len; t += stride) {
+        a.dtq[t] = 0.0f;
+        a.dtk[t] = 0.0f;
+        a.dtv[t] = 0.0f;
+    }
+    for (int64_t t = t0; t < a.H; t += stride) a.units[a.W + t] = 0;
+}
+
+// inclusive prefix of ceil(n_w / 64) over the windows; one workgroup
+__global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
+{
+    __shared__ int part[1024];
+    const int W = static_cast<int>(a.W);
+    const int per = (W + 1023) / 1024;
+    const int begin = threadIdx.x * per, end = min(begin + per, W);
+    int sum = 0;
+    for (int w = begin; w < end; ++w) sum += (a.w_sizes[w] + kChunk - 1) / kChunk;
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+        __syncthreads();
+        part[threadIdx.x] += add;
+        __syncthreads();
+    }
+    int run = part[threadIdx.x] - sum;
+    for (int w = begin; w < end; ++w) {
+        run += (a.w_sizes[w] + kChunk - 1) / kChunk;
+        a.units[w] = run;
+    }
+}
+
+// the work counters are re-armed between sweeps
+__global__ void bwd_reset_counters_kernel(BwdArgs a)
+{
+    for (int t = threadIdx.x; t < a.H; t += blockDim.x) a.units[a.W + t] = 0;
+}
+
+// MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv; 1 = dk, dTq; 2 = dv, dTv.
+// The query-owned sweep produces dq and dTk.
+template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
+__global__ __launch_bounds__(kBwdThreads) void attn_bwd_sweep_kernel(BwdArgs a)
+{
+    constexpr bool kNeedDl = !KEY_OWNED || MODE != 2;          // dP / dL are needed
+    constexpr bool kAccA = kNeedDl;                            // dTq (key-owned) or dTk (query-owned)
+    constexpr bool kAccB = KEY_OWNED && MODE != 1;             // dTv
+    constexpr int kHistKinds = (kAccA ? 1 : 0) + (kAccB ? 1 : 0);
+    constexpr int kHistWords = kHistKinds * 2 * ND * 64;       // [kind][group][axis][row]
+
+    extern __shared__ float smem[];
+    const int H = a.H;
+    const int HD = H * D;
+    const int h = blockIdx.x % H;
+    const int cells = a.total_rows * D;
+    float *tab_q = smem;
+    float *tab_k = tab_q + cells;
+    float *tab_v = tab_k + cells;
+    int *hist_all = reinterpret_cast<int *>(tab_v + cells);
+
+    {
+        const T *gq = static_cast<const T *>(a.table_q);
+        const T *gk = static_cast<const T *>(a.table_k);
+        const T *gv = static_cast<const T *>(a.table_v);
+        for (int t = threadIdx.x; t < cells; t += kBwdThreads) {
+            const int r = t / D, c = t - r * D;
+            const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
+            tab_q[t] = as_float(gq[g]);
+            tab_k[t] = as_float(gk[g]);
+            tab_v[t] = as_float(gv[g]);
+        }
+        for (int t = threadIdx.x; t < kBwdWaves * kHistWords; t += kBwdThreads) hist_all[t] = 0;
+    }
+    __syncthreads();   // the only workgroup barrier
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    int *hist_a = hist_all + wave * kHistWords;                 // dL histogram
+    int *hist_b = hist_a + (kAccA ? 2 * ND * 64 : 0);           // P histogram
+
+    const T *gq = static_cast<const T *>(a.q);
+    const T *gk = static_cast<const T *>(a.k);
+    const T *gv = static_cast<const T *>(a.v);
+    const T *ggo = static_cast<const T *>(a.dout);
+
+    float acc_a[ND][D], acc_b[ND][D];
+#pragma unroll
+    for (int n = 0; n < ND; ++n)
+#pragma unroll
+        for (int c = 0; c < D; ++c) acc_a[n][c] = acc_b[n][c] = 0.0f;
+
+    const int *unit_end = a.units;
+    const int total_units = __builtin_amdgcn_readfirstlane(unit_end[a.W - 1]);
+    int *counter = a.units + a.W + h;
+
+    for (;;) {
+        int unit = 0;
+        if (lane == 0) unit = atomicAdd(counter, 1);
+        unit = __builtin_amdgcn_readfirstlane(unit);
+        if (unit >= total_units) break;
+        int lo = 0, hi = static_cast<int>(a.W) - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (__builtin_amdgcn_readfirstlane(unit_end[mid]) > unit) hi = mid; else lo = mid + 1;
+        }
+        const int w = lo;
+        const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
+        const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
+        const int chunk = unit - (w > 0 ? __builtin_amdgcn_readfirstlane(unit_end[w - 1]) : 0);
+        // group size: a window of at most 32 voxels streams two elements per step
+        const int gs = n_w <= 32 ? 32 : 64;
+        const int ng = 64 / gs;
+        const int grp = lane / gs;
+        const int own = chunk * kChunk + (lane - grp * gs);
+        const bool own_valid = own < n_w;
+        const int own_pos = s0 + min(own, n_w - 1);
+        const int own_row = a.n2n[own_pos];
+
+        // owned side
+        float own_x[D], own_y[D], own_c[ND], own_m = 0.0f, own_inv = 0.0f, own_delta = 0.0f;
+        if constexpr (KEY_OWNED) {
+            load_row<D>(gk + static_cast<int64_t>(own_row) * HD + h * D, own_x);   // k_j
+            if constexpr (kNeedDl) load_row<D>(gv + static_cast<int64_t>(own_row) * HD + h * D, own_y);   // v_j
+        } else {
+            load_row<D>(gq + static_cast<int64_t>(own_row) * HD + h * D, own_x);   // q_i
+            load_row<D>(ggo + static_cast<int64_t>(own_row) * HD + h * D, own_y);  // dout_i
+            own_m = a.out_max[static_cast<int64_t>(own_row) * H + h];
+            own_inv = 1.0f / a.out_sum[static_cast<int64_t>(own_row) * H + h];
+            own_delta = a.delta[static_cast<int64_t>(own_row) * H + h];
+        }
+#pragma unroll
+        for (int n = 0; n < ND; ++n) own_c[n] = a.n_coords[static_cast<int64_t>(own_pos) * ND + n];
+        float res_x[D], res_y[D];   // dk_j, dv_j  or  dq_i
+#pragma unroll
+        for (int c = 0; c < D; ++c) res_x[c] = res_y[c] = 0.0f;
+
+        const int steps = (n_w + ng - 1) / ng;
+        int st_row_next = a.n2n[s0 + min(grp, n_w - 1)];
+        for (int it = 0; it < steps; ++it) {
+            const int st = it * ng + grp;
+            const bool st_valid = st < n_w;
+            const int st_pos = s0 + min(st, n_w - 1);
+            const int st_row = st_row_next;
+            if (it + 1 < steps) st_row_next = a.n2n[s0 + min(st + ng, n_w - 1)];
+            // streamed side (the same for all lanes of a group)
+            float st_x[D], st_y[D], st_c[ND], st_m = 0.0f, st_inv = 0.0f, st_delta = 0.0f;
+            if constexpr (KEY_OWNED) {
+                load_row<D>(gq + static_cast<int64_t>(st_row) * HD + h * D, st_x);    // q_i
+                load_row<D>(ggo + static_cast<int64_t>(st_row) * HD + h * D, st_y);   // dout_i
+                st_m = a.out_max[static_cast<int64_t>(st_row) * H + h];
+                st_inv = 1.0f / a.out_sum[static_cast<int64_t>(st_row) * H + h];
+                st_delta = a.delta[static_cast<int64_t>(st_row) * H + h];
+            } else {
+                load_row<D>(gk + static_cast<int64_t>(st_row) * HD + h * D, st_x);    // k_j
+                load_row<D>(gv + static_cast<int64_t>(st_row) * HD + h * D, st_y);    // v_j
+            }
+#pragma unroll
+            for (int n = 0; n < ND; ++n) st_c[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
+
+            const float *qv = KEY_OWNED ? st_x : own_x;
+            const float *kv = KEY_OWNED ? own_x : st_x;
+            const float *vv = KEY_OWNED ? own_y : st_y;
+            const float *gov = KEY_OWNED ? st_y : own_y;
+            const float m_i = KEY_OWNED ? st_m : own_m;
+            const float inv_i = KEY_OWNED ? st_inv : own_inv;
+            const float delta_i = KEY_OWNED ? st_delta : own_delta;
+
+            int r[ND];
+            float bq[D], bk[D], bv[D];
+#pragma unroll
+            for (int c = 0; c < D; ++c) bq[c] = bk[c] = bv[c] = 0.0f;
+#pragma unroll
+            for (int n = 0; n < ND; ++n) {
+                const float ci = KEY_OWNED ? st_c[n] : own_c[n];
+                const float cj = KEY_OWNED ? own_c[n] : st_c[n];
+                r[n] = crse_row(ci, cj, a.rows[n]);
+                const int off = (a.base[n] + r[n]) * D;
+                float tq_r[D], tk_r[D];
+                load_row<D>(tab_q + off, tq_r);
+                load_row<D>(tab_k + off, tk_r);
+#pragma unroll
+                for (int c = 0; c < D; ++c) {
+                    bq[c] += tq_r[c];
+                    bk[c] += tk_r[c];
+                }
+                if constexpr (kNeedDl) {
+                    float tv_r[D];
+                    load_row<D>(tab_v + off, tv_r);
+#pragma unroll
+                    for (int c = 0; c < D; ++c) bv[c] += tv_r[c];
+                }
+            }
+            float logit = 0.0f;
+#pragma unroll
+            for (int c = 0; c < D; ++c) logit += qv[c] * kv[c] + qv[c] * bq[c] + kv[c] * bk[c];
+            const bool valid = own_valid && st_valid;
+            const float p = valid ? __expf(logit - m_i) * inv_i : 0.0f;
+            float dl = 0.0f;
+            if constexpr (kNeedDl) {
+                float dp = 0.0f;
+#pragma unroll
+                for (int c = 0; c < D; ++c) dp += gov[c] * (vv[c] + bv[c]);
+                dl = p * (dp - delta_i);
+            }
+            if constexpr (KEY_OWNED) {
+                if constexpr (MODE != 2) {
+#pragma unroll
+                    for (int c = 0; c < D; ++c) res_x[c] += dl * (qv[c] + bk[c]);   // dk_j
+                }
+                if constexpr (MODE != 1) {
+#pragma unroll
+                    for (int c = 0; c < D; ++c) res_y[c] += p * gov[c];             // dv_j
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < D; ++c) res_x[c] += dl * (kv[c] + bq[c]);       // dq_i
+            }
+
+            // table gradients: histogram of the step over table rows, then a rank-1 update (lane = row)
+            float amax = 0.0f;
+            if constexpr (kAccA) {
+                amax = fabsf(dl);
+#pragma unroll
+                for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+                if (gs == 64) amax = fmaxf(amax, __shfl_xor(amax, 32));
+                const int qd = __float2int_rn(dl * (amax > 0.0f ? kFixL / amax : 0.0f));
+                if (valid && qd != 0) {
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) atomicAdd(hist_a + (grp * ND + n) * 64 + r[n], qd);
+                }
+            }
+            if constexpr (kAccB) {
+                const int qp = __float2int_rn(p * kFixP);
+                if (valid && qp != 0) {
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) atomicAdd(hist_b + (grp * ND + n) * 64 + r[n], qp);
+                }
+            }
+            wave_lds_fence();
+            for (int g = 0; g < ng; ++g) {
+                const int src = g * gs;   // a lane of group g: its streamed registers are the group's
+                if constexpr (kAccA) {
+                    const float sc = __shfl(amax, src) * (1.0f / kFixL);
+                    float sx[D];
+#pragma unroll
+                    for (int c = 0; c < D; ++c) sx[c] = __shfl(st_x[c], src);   // q_i (key-owned) or k_j
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) {
+                        int *cell = hist_a + (g * ND + n) * 64 + lane;
+                        const float gsum = static_cast<float>(*cell) * sc;
+                        *cell = 0;
+#pragma unroll
+                        for (int c = 0; c < D; ++c) acc_a[n][c] += gsum * sx[c];
+                    }
+                }
+                if constexpr (kAccB) {
+                    float sy[D];
+#pragma unroll
+                    for (int c = 0; c < D; ++c) sy[c] = __shfl(st_y[c], src);   // dout_i
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) {
+                        int *cell = hist_b + (g * ND + n) * 64 + lane;
+                        const float psum = static_cast<float>(*cell) * (1.0f / kFixP);
+                        *cell = 0;
+#pragma unroll
+                        for (int c = 0; c < D; ++c) acc_b[n][c] += psum * sy[c];
+                    }
+                }
+            }
+            wave_lds_fence();
+        }
+
+        if (ng == 2) {
+            // the two groups own the same elements and saw alternate steps of the stream
+#pragma unroll
+            for (int c = 0; c < D; ++c) {
+                res_x[c] += __shfl_xor(res_x[c], 32);
+                res_y[c] += __shfl_xor(res_y[c], 32);
+            }
+        }
+        if (own_valid && grp == 0) {
+            if constexpr (KEY_OWNED) {
+                if constexpr (MODE != 2)
+                    store_row<D>(static_cast<T *>(a.dk) + static_cast<int64_t>(own_row) * HD + h * D, res_x);
+                if constexpr (MODE != 1)
+                    store_row<D>(static_cast<T *>(a.dv) + static_cast<int64_t>(own_row) * HD + h * D, res_y);
+            } else {
+                store_row<D>(static_cast<T *>(a.dq) + static_cast<int64_t>(own_row) * HD + h * D, res_x);
+            }
+        }
+    }
+
+    // lane = table row: add this wavefront's table gradients to the global tables
+    float *dst_a = KEY_OWNED ? a.dtq : a.dtk;
+#pragma unroll
+    for (int n = 0; n < ND; ++n) {
+        if (lane < a.rows[n]) {
+            const int64_t g = static_cast<int64_t>(a.base[n] + lane) * HD + h * D;
+#pragma unroll
+            for (int c = 0; c < D; ++c) {
+                if constexpr (kAccA) atomicAdd(dst_a + g + c, acc_a[n][c]);
+                if constexpr (kAccB) atomicAdd(a.dtv + g + c, acc_b[n][c]);
+            }
+        }
+    }
+}
+
+template <int KINDS> size_t bwd_lds_bytes(const BwdArgs &a)
+{
+    return sizeof(float) * 3 * static_cast<size_t>(a.total_rows) * a.D +
+           sizeof(int) * kBwdWaves * KINDS * 2 * static_cast<size_t>(a.nd) * 64;
+}
+
+template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
+int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
+{
+    constexpr bool need_dl = !KEY_OWNED || MODE != 2;
+    constexpr int kinds = (need_dl ? 1 : 0) + ((KEY_OWNED && MODE != 1) ? 1 : 0);
+    auto kernel = attn_bwd_sweep_kernel<T, D, ND, KEY_OWNED, MODE>;
+    const size_t lds = bwd_lds_bytes<kinds>(a);
+    if (lds > 160 * 1024)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: the tables of one head (%d rows x %d) do not fit LDS",
+                    a.total_rows, a.D);
+    S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    hipLaunchKernelGGL(bwd_reset_counters_kernel, dim3(1), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+template <typename T, int D, int ND>
+int launch_bwd(const BwdArgs &a, hipStream_t stream)
+{
+    const int64_t work = a.N * a.H + a.table_len;
+    const int prep_grid = static_cast<int>(ceil_div(work > 0 ? work : 1, 256) < 4096 ? ceil_div(work > 0 ? work : 1, 256) : 4096);
+    hipLaunchKernelGGL(bwd_prepare_kernel<T>, dim3(static_cast<unsigned>(prep_grid)), dim3(256), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(bwd_units_kernel, dim3(1), dim3(1024), 0, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    int device = 0, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
+    }
+    // a workgroup serves one head for its whole life: a multiple of H workgroups, about two per CU
+    const int per_head = (2 * cus + a.H - 1) / a.H;
+    const int grid = per_head * a.H;
+    if constexpr (D <= 8) {
+        if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
+    } else {
+        if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
+        if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
+    }
+    return launch_sweep<T, D, ND, false, 0>(a, grid, stream);
+}
+
+int fill_bwd_axes(BwdArgs &a, const int32_t *table_sizes, int nd, int64_t table_len)
+{
+    const int64_t hd = static_cast<int64_t>(a.H) * a.D;
+    int64_t total = 0;
+    int base = 0;
+    for (int n = 0; n < nd; ++n) {
+        const int64_t size = table_sizes[n];
+        if (size <= 0 || size % hd != 0)
+            return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: table_sizes[%d] = %lld is not a positive multiple of "
+                        "H*D = %lld", n, (long long)size, (long long)hd);
+        total += size;
+        a.rows[n] = static_cast<int32_t>(size / hd);
+        a.base[n] = base;
+        base += a.rows[n];
+        if (a.rows[n] > 64)
+            return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: axis table %d has %d rows (at most 64)", n, a.rows[n]);
+    }
+    for (int n = nd; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = 0;
+    if (total != table_len)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: sum(table_sizes) = %lld differs from table_len = %lld",
+                    (long long)total, (long long)table_len);
+    a.total_rows = base;
+    return S3D_OK;
+}
+
+size_t bwd_units_bytes(int64_t W, int H)
+{
+    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(H)), 256);
+}
+
+}  // namespace
+}  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_bytes(int32_t H, int64_t N,
+                                                                                      int64_t W)
+{
+    using namespace s3d;
+    if (H < 1 || N < 0 || W < 0) return 0;
+    return bwd_units_bytes(W, H) + align_up(sizeof(float) * static_cast<size_t>(N) * H, 256);
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
+    const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
+    const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
+    const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, const void *out,
+    const float *out_max, const float *out_sum, const void *dout, void *dq, void *dk, void *dv,
+    float *dtable_q, float *dtable_k, float *dtable_v, int64_t N, int32_t H, int32_t D, int64_t W,
+    int32_t dtype, void *workspace, size_t workspace_bytes, void *stream)
+{
+    using namespace s3d;
+    if (N < 0 || W < 0 || H < 1 || D < 1 || nd < 1 || table_len < 1)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: bad sizes N=%lld W=%lld H=%d D=%d nd=%d table_len=%lld",
+                    (long long)N, (long long)W, H, D, nd, (long long)table_len);
+    if (nd != 3 && nd != 6 && nd != 9)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d cRSE axes (3, 6 or 9)", nd);
+    if (D != 8 && D != 16) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8 or 16)", D);
+    if (W > 0x7fffffffLL || N > 0x7fffffffLL || H > 65535)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: N, W must fit 31 bits and H 16 bits");
+    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
+        return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: table_sizes (host) is null");
+    BwdArgs a{};
+    a.H = H;
+    a.D = D;
+    a.nd = nd;
+    a.N = N;
+    a.W = W;
+    a.table_len = table_len;
+    if (int rc = fill_bwd_axes(a, table_sizes, nd, table_len)) return rc;
+    if (!dtable_q || !dtable_k || !dtable_v)
+        return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null table-gradient pointer");
+    const size_t need = s3d_attn_bwd_workspace_bytes(H, N, W);
+    if (!workspace || workspace_bytes < need)
+        return fail(S3D_ERR_WORKSPACE, "s3d_attn_bwd: workspace %zu B < required %zu B",
+                    workspace ? workspace_bytes : size_t(0), need);
+    if (N > 0 && W > 0 &&
+        (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n2n || !n_coords || !out ||
+         !out_max || !out_sum || !dout || !dq || !dk || !dv))
+        return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null device pointer");
+    a.q = q; a.k = k; a.v = v;
+    a.table_q = table_q; a.table_k = table_k; a.table_v = table_v;
+    a.dout = dout; a.out = out; a.out_max = out_max; a.out_sum = out_sum;
+    a.w_sizes = w_sizes; a.w2n = w2n; a.n2n = n2n; a.n_coords = n_coords;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
+    a.units = static_cast<int32_t *>(workspace);
+    a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, H));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (N == 0 || W == 0) {
+        // nothing to differentiate: the table gradients are zero
+        a.N = 0;
+        hipLaunchKernelGGL((bwd_prepare_kernel<float>), dim3(64), dim3(256), 0, s, a);
+        S3D_HIP_CHECK(hipGetLastError());
+        return S3D_OK;
+    }
+#define S3D_BWD_CASE(DD, NN)                                                              \
+    if (D == DD && nd == NN)                                                              \
+        return dtype == S3D_DTYPE_F16 ? launch_bwd<__half, DD, NN>(a, s) : launch_bwd<float, DD, NN>(a, s);
+    S3D_BWD_CASE(8, 3) S3D_BWD_CASE(8, 6) S3D_BWD_CASE(8, 9)
+    S3D_BWD_CASE(16, 3) S3D_BWD_CASE(16, 6) S3D_BWD_CASE(16, 9)
+#undef S3D_BWD_CASE
+    return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: D=%d nd=%d", D, nd);
+}

@@ -1,2 +1,2 @@
 from .attn_coff import (IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims,
-                        window_attention_forward)
+                        window_attention_backward, window_attention_forward)

@@ -163,6 +163,68 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     return out
 
 
+def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n, n_coords,
+                              out, out_max, out_sum, dout):
+    """Gradients of window_attention_forward -> (dq, dk, dv [N,H,D] in the dtype of q,
+    dtable_q, dtable_k, dtable_v flat fp32).  out / out_max / out_sum are the forward's results
+    (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes."""
+    _require_cuda("query", q)
+    dev = q.device
+    if q.dim() != 3:
+        raise ValueError(f"query must be [N,H,D], got {tuple(q.shape)}")
+    n, h, d = q.shape
+    if q.dtype not in _DTYPE_CODE:
+        raise TypeError(f"unsupported feature dtype {q.dtype} (float16 or float32)")
+    for name, t in (("key", k), ("value", v), ("out", out), ("dout", dout)):
+        _require_cuda(name, t, dev)
+        if t.shape != q.shape or t.dtype != q.dtype:
+            raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
+    if d not in (8, 16):
+        raise ValueError(f"head_dim must be 8 or 16, got {d}")
+    sizes = _host_table_sizes(table_sizes)
+    nd = len(sizes)
+    if nd not in (3, 6, 9):
+        raise ValueError(f"table_sizes must have 3, 6 or 9 entries, got {nd}")
+    table_len = table_q.numel()
+    if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_len:
+        raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
+                         f"to the table length {table_len}")
+    if max(sizes) // (h * d) > 64:
+        raise NotImplementedError("attention backward supports axis tables of at most 64 rows")
+    for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
+        _require_cuda(name, t, dev)
+        if t.dtype != q.dtype or t.numel() != table_len:
+            raise ValueError(f"{name} must have the dtype of the features and {table_len} elements")
+    for name, t in (("out_max", out_max), ("out_sum", out_sum)):
+        _require_cuda(name, t, dev)
+        if t.dtype != torch.float32 or t.shape != (n, h):
+            raise ValueError(f"{name} must be float32 [{n},{h}]")
+    w_sizes = _as_int32("w_sizes", w_sizes, dev)
+    w2n = _as_int32("w2n_indices", w2n, dev)
+    n2n = _as_int32("n2n_indices", n2n, dev)
+    _require_cuda("n_coords", n_coords, dev)
+    if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
+        raise ValueError(f"n_coords must be float32 [{n},{nd}]")
+    c_sizes = (ctypes.c_int32 * nd)(*sizes)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    dtq, dtk, dtv = (torch.empty(table_len, dtype=torch.float32, device=dev) for _ in range(3))
+    lib = _lib.lib()
+    tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
+    out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
+    with torch.cuda.device(dev):
+        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, n, w_sizes.numel())
+        workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        status = lib.s3d_attn_bwd(
+            *(t.data_ptr() for t in tensors), c_sizes, nd, table_len, w_sizes.data_ptr(), w2n.data_ptr(),
+            n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(), out_max.data_ptr(), out_sum.data_ptr(),
+            dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dtq.data_ptr(), dtk.data_ptr(),
+            dtv.data_ptr(), n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype], workspace.data_ptr(), ws_bytes,
+            stream)
+    _lib.check(status, "s3d_attn_bwd")
+    return dq, dk, dv, dtq, dtk, dtv
+
+
 def _compute_dtype(precision):
     """fp32 unless autocast is on and the precision mode allows half (attn_coff.py:172-175)."""
     if torch.is_autocast_enabled() and precision != PrecisionMode.HALF_NONE:
@@ -171,7 +233,7 @@ def _compute_dtype(precision):
 
 
 class SelfAttnAIOFunction(Function):
-    """Function of all-in-one self-attention (forward only)."""
+    """Function of all-in-one self-attention (Swin3D/sparse_dl/attn/attn_coff.py:155-232)."""
 
     @staticmethod
     def forward(ctx, raw_query_feats, raw_key_feats, raw_value_feats, query_table, key_table,
@@ -186,13 +248,36 @@ class SelfAttnAIOFunction(Function):
         if c_dtype not in _DTYPE_CODE:
             raise NotImplementedError(f"compute dtype {c_dtype} is not supported (float16 / float32)")
         _, w_sizes, _, w2n, n2n, n_coords = indices
-        feats = [t.to(c_dtype).contiguous() for t in (raw_query_feats, raw_key_feats, raw_value_feats)]
-        tables = [t.to(c_dtype).contiguous() for t in (query_table, key_table, value_table)]
-        out = window_attention_forward(*feats, *tables, table_offsets, w_sizes, w2n, n2n,
-                                       n_coords.to(torch.float32).contiguous())
-        ctx.mark_non_differentiable(out)
+        raw = (raw_query_feats, raw_key_feats, raw_value_feats, query_table, key_table, value_table)
+        feats = [t.to(c_dtype).contiguous() for t in raw[:3]]
+        tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
+        n_coords = n_coords.to(torch.float32).contiguous()
+        needs_grad = any(ctx.needs_input_grad[:6])
+        res = window_attention_forward(*feats, *tables, table_offsets, w_sizes, w2n, n2n, n_coords,
+                                       return_stats=needs_grad)
+        if not needs_grad:
+            return res
+        out, omax, osum = res
+        ctx.precision = precision
+        ctx.table_sizes = _host_table_sizes(table_offsets)
+        ctx.save_for_backward(out, omax, osum, *raw, w_sizes, w2n, n2n, n_coords)
         return out
 
     @staticmethod
     def backward(ctx, *grad_outputs):
-        raise NotImplementedError("swin3d_amd implements the attention forward only")
+        """Compute dtype as in the reference (attn_coff.py:206-215): the gradient's dtype for HALF_ALL,
+        fp32 otherwise; the statistics saved by the forward are reused either way."""
+        (dout,) = grad_outputs
+        out, omax, osum = ctx.saved_tensors[:3]
+        raw = ctx.saved_tensors[3:9]
+        w_sizes, w2n, n2n, n_coords = ctx.saved_tensors[9:]
+        c_dtype = dout.dtype if ctx.precision == PrecisionMode.HALF_ALL else torch.float32
+        if c_dtype not in _DTYPE_CODE:
+            raise NotImplementedError(f"compute dtype {c_dtype} is not supported (float16 / float32)")
+        feats = [t.to(c_dtype).contiguous() for t in raw[:3]]
+        tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
+        grads = window_attention_backward(*feats, *tables, ctx.table_sizes, w_sizes, w2n, n2n, n_coords,
+                                          out.to(c_dtype), omax, osum, dout.to(c_dtype).contiguous())
+        grads = [g.to(t.dtype).reshape(t.shape) if need else None
+                 for g, t, need in zip(grads, raw, ctx.needs_input_grad[:6])]
+        return (*grads, None, None, None, None, None, None)

@@ -1,0 +1,191 @@
+"""GPU parity of the window attention backward (HIP through the C ABI) against the float64 CPU oracle.
+
+Tolerance: |got - ref| <= rel * scale with rel = 2e-5 for fp32 and 3e-3 for fp16 (fp16: the forward output
+o that enters dout.o, and dq / dk / dv themselves, are rounded to fp16); scale = largest |ref| over
+(dq, dk, dv) for those three and over the three table gradients for those."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_attn_case, scene_attn_case, to_half_and_back, n_coords_from_scene
+from swin3d_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("dq", "dk", "dv", "dtable_q", "dtable_k", "dtable_v")
+
+
+def _run(case, dout, dtype):
+    import swin3d_amd
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = lambda a: t(a).to(dtype)
+    i = case.index
+    args = (f(case.q), f(case.k), f(case.v), f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
+            t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
+    out, omax, osum = swin3d_amd.window_attention_forward(*args, return_stats=True)
+    grads = swin3d_amd.window_attention_backward(*args, out, omax, osum, f(dout))
+    torch.cuda.synchronize()
+    return [g.double().cpu().numpy() for g in grads]
+
+
+def _assert_close(got, ref, dtype):
+    """The scale of a tolerance is the largest |ref| of the GROUP a tensor belongs to (dq, dk, dv / the three
+    table gradients): dq and dk are sums of P (dP - dout.o) terms that cancel (exactly, for a single-voxel
+    window), so their rounding error is set by the size of the terms, which dv shares, not by the result."""
+    rel = 2e-5 if dtype == torch.float32 else 3e-3
+    ref = [np.asarray(r, np.float64).reshape(g.shape) for g, r in zip(got, ref)]
+    scales = [max(np.abs(r).max() for r in ref[:3])] * 3 + [max(np.abs(r).max() for r in ref[3:])] * 3
+    for name, g, r, scale in zip(NAMES, got, ref, scales):
+        assert np.isfinite(g).all(), name
+        err = np.abs(g - r).max()
+        assert err <= rel * max(scale, 1e-30), f"{name}: max err {err:.3e}, scale {scale:.3e}"
+
+
+def _check(oracle_lib, case, dtype, seed=0, dout_scale=1.0):
+    if dtype == torch.float16:
+        to_half_and_back(case)
+    rng = np.random.default_rng(seed + 900)
+    dout = (rng.standard_normal(case.q.shape) * dout_scale).astype(np.float32)
+    if dtype == torch.float16:
+        dout = dout.astype(np.float16).astype(np.float32)
+    ref = oracle_lib.attn_bwd(*case.oracle_args(), dout)
+    _assert_close(_run(case, dout, dtype), ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("cRSE", ["XYZ", "XYZ_RGB", "XYZ_RGB_NORM"])
+@pytest.mark.parametrize("heads,dim,ws", [(6, 8, 5), (3, 16, 7)])
+def test_random_scenes(oracle_lib, hip_lib, dtype, cRSE, heads, dim, ws):
+    case = make_attn_case(oracle_lib, seed=61, n=900, ws=ws, quant=4, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(10, 10, 3) if ws == 5 else (12, 12, 4))
+    if dtype == torch.float16:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+    _check(oracle_lib, case, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_room_layer_recipe(oracle_lib, hip_lib, dtype):
+    """A small synthetic room with the freshly-initialised-layer recipe (near-uniform softmax); tiny
+    gradient scale on purpose: the fixed-point histograms are scaled per step, not by a constant."""
+    scene = synth.make_room((3.0, 2.0, 1.5), 3, 4000, seed=3)
+    case = scene_attn_case(oracle_lib, scene, 5, 4, 6, 8, "XYZ_RGB_NORM", recipe="layer")
+    _check(oracle_lib, case, dtype, dout_scale=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
+    ws, quant, heads, dim = 7, 4, 2, 16
+    g = np.stack(np.meshgrid(np.arange(14), np.arange(7), np.arange(7), indexing="ij"), -1).reshape(-1, 3)
+    coords = np.concatenate([np.zeros((g.shape[0], 1), np.int64), g], 1).astype(np.int32)
+    rng = np.random.default_rng(63)
+    coords = coords[rng.permutation(coords.shape[0])]
+    frac = rng.random((coords.shape[0], 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (coords.shape[0], 6)).astype(np.float32)
+    case = make_attn_case(oracle_lib, seed=63, n=coords.shape[0], ws=ws, quant=quant, heads=heads, dim=dim,
+                          extent=(12, 12, 6))
+    case.coords = coords
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
+    if dtype == torch.float16:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+    _check(oracle_lib, case, dtype)
+
+
+def test_single_voxel_windows(oracle_lib, hip_lib):
+    coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
+    case = make_attn_case(oracle_lib, seed=64, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")
+    frac = np.random.default_rng(3).random((4, 3)).astype(np.float32)
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, np.zeros((4, 0), np.float32),
+                                                    1, 5, 4, "XYZ")
+    _check(oracle_lib, case, torch.float32)
+
+
+def test_empty_input(hip_lib):
+    import swin3d_amd
+    from swin3d_amd import crse
+    dev = torch.device("cuda")
+    q = torch.zeros((0, 6, 8), device=dev)
+    t = torch.zeros(14976, device=dev)
+    sizes = crse.crse_table_sizes(5, 4, 6, 8, "XYZ_RGB_NORM")
+    e = torch.zeros(0, dtype=torch.int32, device=dev)
+    s = torch.zeros((0, 6), device=dev)
+    grads = swin3d_amd.window_attention_backward(q, q, q, t, t, t, sizes, e, e, e, torch.zeros((0, 9), device=dev),
+                                                 q, s, s, q)
+    assert grads[0].shape == (0, 6, 8) and float(grads[3].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("precision_name", ["HALF_NONE", "HALF_ALL"])
+def test_autograd_function(oracle_lib, hip_lib, precision_name):
+    """loss.backward() through SelfAttnAIOFunction with the reference's argument list."""
+    from swin3d_amd.sparse_dl.attn.attn_coff import (SelfAttnAIOFunction, PosEmb, TableDims, IndexMode,
+                                                     PrecisionMode)
+    case = make_attn_case(oracle_lib, seed=65, n=500, ws=5, quant=4, heads=6, dim=8, extent=(8, 8, 3))
+    half = precision_name == "HALF_ALL"
+    if half:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+        to_half_and_back(case)
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    leaves = [t(a).requires_grad_(True) for a in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
+    i = case.index
+    indices = [None, t(i["w_sizes"]).long(), None, t(i["w2n"]).long(), t(i["n2n"]).long(), t(case.n_coords)]
+    rng = np.random.default_rng(66)
+    dout = rng.standard_normal(case.q.shape).astype(np.float32)
+    if half:
+        dout = dout.astype(np.float16).astype(np.float32)
+    with torch.autocast("cuda", dtype=torch.float16, enabled=half):
+        out = SelfAttnAIOFunction.apply(*leaves, case.table_sizes.tolist(), indices, PosEmb.SEPARATE,
+                                        TableDims.D0, IndexMode.INDIRECT, getattr(PrecisionMode, precision_name))
+    assert out.dtype == (torch.float16 if half else torch.float32)
+    out.backward(t(dout).to(out.dtype))
+    torch.cuda.synchronize()
+    ref = oracle_lib.attn_bwd(*case.oracle_args(), dout)
+    got = [leaf.grad.double().cpu().numpy() for leaf in leaves]
+    assert all(leaf.grad.dtype == torch.float32 for leaf in leaves)
+    _assert_close(got, ref, torch.float16 if half else torch.float32)
+
+
+def test_headline_size_properties(hip_lib):
+    """Swin3D-S stage-1 size (200k voxels, fp16): closed forms that hold for any input.
+    Softmax rows sum to one, hence per window and head  sum_j dv_j = sum_i dout_i,  and for every axis
+    sum_rows dTv[axis][row][h][c] = sum_i dout_i[h][c];  logit gradients of a row sum to zero, hence
+    sum_rows dTq[axis][row][h][c] = sum_i q_i[h][c] * 0 ... checked through linearity in dout instead:
+    bwd(2 * dout) = 2 * bwd(dout) exactly in the deterministic outputs."""
+    import swin3d_amd
+    from swin3d_amd import crse
+    dev = torch.device("cuda")
+    scene = synth.make_room((10.0, 8.0, 3.0), 30, 200_000, seed=0)
+    heads, dim, ws, quant, mode = 6, 8, 5, 4, "XYZ_RGB_NORM"
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    n = scene.coords.shape[0]
+    args = swin3d_amd.get_index01(t(scene.coords), 1, ws, t(scene.frac), t(synth.signals(scene, mode)))
+    _, _, _, w_sizes, w2n, n2n, _, n_coords = args
+    n_crse = crse.scale_crse_coords(n_coords, quant, mode)
+    sizes = crse.crse_table_sizes(ws, quant, heads, dim, mode)
+    q, k, v, tables = synth.layer_inputs(n, heads * dim, heads, int(sum(sizes)), seed=0, dtype=np.float16)
+    dout = np.random.default_rng(5).standard_normal((n, heads, dim)).astype(np.float16)
+    a = (t(q), t(k), t(v), t(tables[0]), t(tables[1]), t(tables[2]), sizes, w_sizes, w2n, n2n, n_crse)
+    out, omax, osum = swin3d_amd.window_attention_forward(*a, return_stats=True)
+    g1 = swin3d_amd.window_attention_backward(*a, out, omax, osum, t(dout))
+    g2 = swin3d_amd.window_attention_backward(*a, out, omax, osum, t(dout) * 2)
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(g).all() for g in g1)
+    for x, y in zip(g1[:3], g2[:3]):
+        # a power of two commutes with every rounding involved except the one to fp16 subnormals
+        # (spacing 2^-24) of the stored result
+        assert float((x.float() * 2 - y.float()).abs().max()) <= 2.0 ** -23
+    # sum over the keys of a window of dv = sum over its queries of dout
+    win = torch.repeat_interleave(torch.arange(w_sizes.numel(), device=dev), w_sizes.long())
+    rows = n2n.long()
+    dv_w = torch.zeros((w_sizes.numel(), heads, dim), device=dev).index_add_(0, win, g1[2][rows].float())
+    do_w = torch.zeros_like(dv_w).index_add_(0, win, t(dout)[rows].float())
+    assert float((dv_w - do_w).abs().max()) <= 3e-3 * float(do_w.abs().max())
+    total = t(dout).float().sum(0)            # [H,D]
+    off = 0
+    for size in sizes:
+        block = g1[5][off:off + size].reshape(-1, heads, dim).sum(0)
+        off += size
+        assert float((block - total).abs().max()) <= 1e-3 * float(t(dout).float().abs().sum(0).max())
