@@ -173,6 +173,14 @@ def main():
 
     if not args.no_extras:
         result["extras"] = extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev)
+        # backward of the same layer (fp16 I/O as under PrecisionMode.HALF_ALL, fp32 arithmetic)
+        fwd_args = (q_d, k_d, v_d, tq_d, tk_d, tv_d, sizes, index.w_sizes, index.w2n, index.n2n, n_crse)
+        o_d, mx_d, sm_d = swin3d_amd.window_attention_forward(*fwd_args, return_stats=True)
+        dout_d = torch.randn_like(o_d)
+        ms = _time_gpu(torch, lambda: swin3d_amd.window_attention_backward(*fwd_args, o_d, mx_d, sm_d, dout_d),
+                       reps=5, warm=2)
+        result["extras"]["attn_bwd"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3),
+                                        "vs_forward": ms / kernel_ms, "dtype": "f16 I/O, f32 arithmetic"}
 
     if not args.no_extras and not args.no_encoder:
         result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)

@@ -112,7 +112,8 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
  * Windowed self-attention backward.
  *
  * Replaces cal_exp_sum_grads and self_attn_indir_backward
- * (Swin3D/src/attn/self_attn_aio_bwd.cu:14-47 and :49-113, 197-509; called from
+ * (Swin3D/src/attn/self_attn_aio_bwd.cu:14-47 and :49-113, 197-509, exported at
+ * Swin3D/src/attn/attn_api.cpp:21,24; called from
  * Swin3D/sparse_dl/attn/attn_coff.py:219-224) for pos_mode SEPARATE and indice_mode INDIRECT,
  * without the O(M) pair arrays.  Arithmetic is fp32 for both dtypes.
  *

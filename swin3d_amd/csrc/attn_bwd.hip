@@ -97,6 +97,12 @@ template <int D> __device__ __forceinline__ void store_row(__half *p, const floa
 __device__ __forceinline__ float as_float(float x) { return x; }
 __device__ __forceinline__ float as_float(__half x) { return __half2float(x); }
 
+// value of x in lane `src` (src uniform): a scalar read instead of an LDS permute
+__device__ __forceinline__ float lane_value(float x, int src)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
+}
+
 __device__ __forceinline__ int crse_row(float ci, float cj, int rows)
 {
     float rel = ci - cj;
@@ -156,10 +162,11 @@ __global__ void bwd_reset_counters_kernel(BwdArgs a)
     for (int t = threadIdx.x; t < a.H; t += blockDim.x) a.units[a.W + t] = 0;
 }
 
-// MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv; 1 = dk, dTq; 2 = dv, dTv.
+// MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv (not launched: too many registers); 1 = dk, dTq;
+// 2 = dv, dTv.
 // The query-owned sweep produces dq and dTk.
 template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
-__global__ __launch_bounds__(kBwdThreads) void attn_bwd_sweep_kernel(BwdArgs a)
+__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_kernel(BwdArgs a)
 {
     constexpr bool kNeedDl = !KEY_OWNED || MODE != 2;          // dP / dL are needed
     constexpr bool kAccA = kNeedDl;                            // dTq (key-owned) or dTk (query-owned)
@@ -357,12 +364,12 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_sweep_kernel(BwdArgs a)
             }
             wave_lds_fence();
             for (int g = 0; g < ng; ++g) {
-                const int src = g * gs;   // a lane of group g: its streamed registers are the group's
+                const int src = __builtin_amdgcn_readfirstlane(g * gs);   // a lane of group g: its streamed registers are the group's
                 if constexpr (kAccA) {
-                    const float sc = __shfl(amax, src) * (1.0f / kFixL);
+                    const float sc = lane_value(amax, src) * (1.0f / kFixL);
                     float sx[D];
 #pragma unroll
-                    for (int c = 0; c < D; ++c) sx[c] = __shfl(st_x[c], src);   // q_i (key-owned) or k_j
+                    for (int c = 0; c < D; ++c) sx[c] = lane_value(st_x[c], src);   // q_i (key-owned) or k_j
 #pragma unroll
                     for (int n = 0; n < ND; ++n) {
                         int *cell = hist_a + (g * ND + n) * 64 + lane;
@@ -375,7 +382,7 @@ __global__ __launch_bounds__(kBwdThreads) void attn_bwd_sweep_kernel(BwdArgs a)
                 if constexpr (kAccB) {
                     float sy[D];
 #pragma unroll
-                    for (int c = 0; c < D; ++c) sy[c] = __shfl(st_y[c], src);   // dout_i
+                    for (int c = 0; c < D; ++c) sy[c] = lane_value(st_y[c], src);   // dout_i
 #pragma unroll
                     for (int n = 0; n < ND; ++n) {
                         int *cell = hist_b + (g * ND + n) * 64 + lane;
@@ -465,12 +472,10 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
     // a workgroup serves one head for its whole life: a multiple of H workgroups, about two per CU
     const int per_head = (2 * cus + a.H - 1) / a.H;
     const int grid = per_head * a.H;
-    if constexpr (D <= 8) {
-        if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
-    } else {
-        if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
-        if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
-    }
+    // two key-owned sweeps (dk + dTq, then dv + dTv): one sweep with both sets of table-gradient registers
+    // spills at two wavefronts per SIMD and measured slower
+    if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
+    if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
     return launch_sweep<T, D, ND, false, 0>(a, grid, stream);
 }
 
