@@ -192,6 +192,24 @@ int s3d_knn(int32_t K, const float *src_xyz, int64_t Ns, const float *query_xyz,
             float *ret_dist2, float cell_size, void *workspace, size_t workspace_bytes,
             void *stream);
 
+/*
+ * Inverse-distance interpolation of source features at the queries, from the result of s3d_knn.
+ *
+ * Replaces the torch statement knn_linear_interpolation
+ * (Swin3D/modules/swin3d_layers.py:53-73: K indexing passes over src_feat and the weight
+ * arithmetic, about 3*K + 4 kernels) with one gather kernel:
+ *   weight_i = 1 / (sqrt(dist2_i) + 1e-8), normalised over the K neighbours of the query
+ *   out[q]   = sum_i weight_i * src_feat[idx[q][i]]
+ *
+ *   idx, dist2   device [Nq,K] as written by s3d_knn (squared distances)
+ *   src_feat     device [Ns,C] of `dtype`        out   device [Nq,C] of `dtype`
+ * Neighbour slots padded with row -1 carry no weight (the reference's torch indexing would read the
+ * LAST source row there, with a weight of about 2e-5); a query with no neighbour at all gets zeros.
+ * Accumulation is fp32, one rounding to `dtype`.
+ */
+int s3d_knn_interpolate(const int32_t *idx, const float *dist2, int32_t K, int64_t Nq, const void *src_feat,
+                        int64_t Ns, int32_t C, int32_t dtype, void *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,6 +39,7 @@ def lib():
             "s3d_oracle_attn_bwd_f64",
             "s3d_oracle_knn",
             "s3d_oracle_knn_heap",
+            "s3d_oracle_knn_interpolate",
             "s3d_oracle_max_threads",
         ):
             getattr(_lib, name).restype = ctypes.c_int
@@ -180,3 +181,17 @@ def knn(k, src_xyz, query_xyz, src_offset, query_offset, heap_order=False, num_t
     if rc != 0:
         raise ValueError(f"s3d_oracle_knn failed: {rc}")
     return idx, d2
+
+
+def knn_interpolate(idx, dist2, src_feat):
+    """Inverse-distance interpolation from KNN results -> float64 [Nq,C]."""
+    idx = _c(idx, np.int32)
+    dist2 = _c(dist2, np.float32)
+    src_feat = _c(src_feat, np.float32)
+    nq, k = idx.shape
+    out = np.zeros((nq, src_feat.shape[1]), np.float64)
+    rc = lib().s3d_oracle_knn_interpolate(_p(idx), _p(dist2), ctypes.c_int32(k), ctypes.c_int64(nq), _p(src_feat),
+                                          ctypes.c_int32(src_feat.shape[1]), _p(out))
+    if rc != 0:
+        raise ValueError(f"s3d_oracle_knn_interpolate failed: {rc}")
+    return out

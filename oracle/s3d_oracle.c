@@ -497,6 +497,34 @@ int s3d_oracle_knn_heap(int32_t K, const float *src_xyz, int64_t Ns, const float
     return 0;
 }
 
+/*
+ * Inverse-distance interpolation over KNN results, Swin3D/modules/swin3d_layers.py:53-73:
+ *   dist = sqrt(dist2) in fp32 (Swin3D/sparse_dl/knn/knn.py:24), weight = 1 / (dist + 1e-8),
+ *   weight /= sum of the weights of the query, out = sum_i src_feat[idx_i] * weight_i.
+ * Double accumulation.  Slots padded with row -1 carry no weight (decision of this build: the
+ * reference's torch indexing reads the last source row there).
+ * Pinned by closed forms (tests/test_oracle_knn.py): constant field, coincident query,
+ * hand-computed two-neighbour weights.
+ */
+int s3d_oracle_knn_interpolate(const int32_t *idx, const float *dist2, int32_t K, int64_t Nq,
+                               const float *src_feat, int32_t C, double *out)
+{
+    if (K < 1 || C < 1 || Nq < 0) return -1;
+    for (int64_t q = 0; q < Nq; ++q) {
+        double norm = 0;
+        for (int i = 0; i < K; ++i)
+            if (idx[q * K + i] >= 0) norm += 1.0 / ((double)sqrtf(dist2[q * K + i]) + 1e-8);
+        for (int32_t c = 0; c < C; ++c) out[q * C + c] = 0;
+        for (int i = 0; i < K; ++i) {
+            const int32_t row = idx[q * K + i];
+            if (row < 0) continue;
+            const double w = (1.0 / ((double)sqrtf(dist2[q * K + i]) + 1e-8)) / norm;
+            for (int32_t c = 0; c < C; ++c) out[q * C + c] += w * (double)src_feat[(int64_t)row * C + c];
+        }
+    }
+    return 0;
+}
+
 int s3d_oracle_max_threads(void)
 {
 #ifdef _OPENMP

@@ -393,6 +393,75 @@ __global__ __launch_bounds__(kThreads) void knn_query_kernel(
     }
 }
 
+// Inverse-distance interpolation over the K nearest sources of every query
+// (Swin3D/modules/swin3d_layers.py:53-73): weight_i = 1 / (sqrt(dist2_i) + 1e-8), normalised over the K
+// neighbours, out = sum_i weight_i * src_feat[idx_i].  One thread per (query, group of VEC channels);
+// padded neighbour slots (index -1) carry no weight.  fp32 accumulation, one rounding to the output type.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kThreads) void knn_interpolate_kernel(const int32_t *__restrict__ idx,
+                                                                   const float *__restrict__ dist2, int K,
+                                                                   int64_t Nq, const T *__restrict__ feat, int C,
+                                                                   T *__restrict__ out)
+{
+    const int groups = C / VEC;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= Nq * groups) return;
+    const int64_t qi = t / groups;
+    const int c0 = static_cast<int>(t - qi * groups) * VEC;
+    float norm = 0.0f;
+    for (int i = 0; i < K; ++i)
+        if (idx[qi * K + i] >= 0) norm += 1.0f / (sqrtf(dist2[qi * K + i]) + 1e-8f);
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.0f;
+    for (int i = 0; i < K; ++i) {
+        const int row = idx[qi * K + i];
+        if (row < 0) continue;
+        const float w = (1.0f / (sqrtf(dist2[qi * K + i]) + 1e-8f)) / norm;
+        T v[VEC];
+        if constexpr (VEC == 4) {
+            if constexpr (sizeof(T) == 4)
+                *reinterpret_cast<float4 *>(v) = *reinterpret_cast<const float4 *>(feat + static_cast<int64_t>(row) * C + c0);
+            else
+                *reinterpret_cast<uint2 *>(v) = *reinterpret_cast<const uint2 *>(feat + static_cast<int64_t>(row) * C + c0);
+        } else {
+            v[0] = feat[static_cast<int64_t>(row) * C + c0];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += w * static_cast<float>(v[e]);
+    }
+    T o[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o[e] = static_cast<T>(acc[e]);
+    if constexpr (VEC == 4) {
+        if constexpr (sizeof(T) == 4)
+            *reinterpret_cast<float4 *>(out + qi * C + c0) = *reinterpret_cast<const float4 *>(o);
+        else
+            *reinterpret_cast<uint2 *>(out + qi * C + c0) = *reinterpret_cast<const uint2 *>(o);
+    } else {
+        out[qi * C + c0] = o[0];
+    }
+}
+
+template <typename T>
+int launch_interpolate(const int32_t *idx, const float *dist2, int K, int64_t Nq, const void *feat, int C, void *out,
+                       hipStream_t s)
+{
+    const T *f = static_cast<const T *>(feat);
+    T *o = static_cast<T *>(out);
+    if (C % 4 == 0) {
+        const int64_t threads = Nq * (C / 4);
+        hipLaunchKernelGGL((knn_interpolate_kernel<T, 4>), dim3(static_cast<unsigned>(ceil_div(threads, kThreads))),
+                           dim3(kThreads), 0, s, idx, dist2, K, Nq, f, C, o);
+    } else {
+        const int64_t threads = Nq * C;
+        hipLaunchKernelGGL((knn_interpolate_kernel<T, 1>), dim3(static_cast<unsigned>(ceil_div(threads, kThreads))),
+                           dim3(kThreads), 0, s, idx, dist2, K, Nq, f, C, o);
+    }
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
 }  // namespace
 }  // namespace s3d
 
@@ -471,4 +540,23 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
                            B, plan, starts, sorted, ret_idx, ret_dist2);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_knn_interpolate(
+    const int32_t *idx, const float *dist2, int32_t K, int64_t Nq, const void *src_feat, int64_t Ns, int32_t C,
+    int32_t dtype, void *out, void *stream)
+{
+    using namespace s3d;
+    if (K < 1 || K > S3D_KNN_KMAX) return fail(S3D_ERR_BAD_SHAPE, "s3d_knn_interpolate: K=%d outside 1..%d", K, S3D_KNN_KMAX);
+    if (Nq < 0 || Ns < 0 || C < 1 || Nq * static_cast<int64_t>(C) > 0x3fffffffffLL)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_knn_interpolate: Nq=%lld Ns=%lld C=%d out of range", (long long)Nq,
+                    (long long)Ns, C);
+    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
+        return fail(S3D_ERR_BAD_DTYPE, "s3d_knn_interpolate: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    if (Nq == 0) return S3D_OK;
+    if (!idx || !dist2 || !out || (Ns > 0 && !src_feat))
+        return fail(S3D_ERR_NULL_POINTER, "s3d_knn_interpolate: null device pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == S3D_DTYPE_F16 ? launch_interpolate<_Float16>(idx, dist2, K, Nq, src_feat, C, out, s)
+                                  : launch_interpolate<float>(idx, dist2, K, Nq, src_feat, C, out, s);
 }

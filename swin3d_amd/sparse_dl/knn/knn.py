@@ -62,3 +62,51 @@ class KNN(Function):
         dist = torch.sqrt(dist2)
         ctx.mark_non_differentiable(idx, dist)
         return idx, dist
+
+
+_FEAT_DTYPE = {torch.float32: 0, torch.float16: 1}
+
+
+def knn_interpolate(idx, dist2, src_feat):
+    """Inverse-distance interpolation of src_feat [Ns,C] at the queries of a knn_query result
+    (idx int32 [Nq,K], SQUARED distances fp32 [Nq,K]) -> [Nq,C] in the dtype of src_feat
+    (Swin3D/modules/swin3d_layers.py:65-72 in one kernel; padded slots carry no weight)."""
+    if not (idx.is_cuda and dist2.is_cuda and src_feat.is_cuda):
+        raise RuntimeError("idx, dist2 and src_feat must be CUDA (HIP) tensors")
+    if idx.dtype != torch.int32 or dist2.dtype != torch.float32 or idx.shape != dist2.shape or idx.dim() != 2:
+        raise ValueError("idx must be int32 [Nq,K] and dist2 float32 [Nq,K]")
+    if src_feat.dim() != 2 or src_feat.dtype not in _FEAT_DTYPE:
+        raise ValueError(f"src_feat must be float16/float32 [Ns,C], got {src_feat.dtype} {tuple(src_feat.shape)}")
+    idx, dist2, src_feat = idx.contiguous(), dist2.contiguous(), src_feat.contiguous()
+    nq, k = idx.shape
+    ns, c = src_feat.shape
+    out = torch.empty((nq, c), dtype=src_feat.dtype, device=src_feat.device)
+    with torch.cuda.device(src_feat.device):
+        stream = torch.cuda.current_stream(src_feat.device).cuda_stream
+        status = _lib.lib().s3d_knn_interpolate(idx.data_ptr(), dist2.data_ptr(), k, nq, src_feat.data_ptr(), ns, c,
+                                                _FEAT_DTYPE[src_feat.dtype], out.data_ptr(), stream)
+    _lib.check(status, "s3d_knn_interpolate")
+    return out
+
+
+class KNNInterpolate(Function):
+    """Differentiable (w.r.t. the features) inverse-distance interpolation; the forward is the fused
+    HIP kernel, the backward scatters the weighted output gradient back with torch's index_add_."""
+
+    @staticmethod
+    def forward(ctx, idx, dist2, src_feat):
+        ctx.save_for_backward(idx, dist2)
+        ctx.num_src = src_feat.shape[0]
+        return knn_interpolate(idx, dist2, src_feat)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        idx, dist2 = ctx.saved_tensors
+        valid = idx >= 0
+        weight = torch.where(valid, 1.0 / (torch.sqrt(dist2) + 1e-8), torch.zeros_like(dist2))
+        weight = weight / weight.sum(dim=1, keepdim=True).clamp_min(1e-30)
+        grad_src = torch.zeros((ctx.num_src, grad_out.shape[1]), dtype=torch.float32, device=grad_out.device)
+        rows = idx.clamp(min=0).long()
+        for i in range(idx.shape[1]):
+            grad_src.index_add_(0, rows[:, i], grad_out.float() * weight[:, i:i + 1])
+        return None, None, grad_src.to(grad_out.dtype)

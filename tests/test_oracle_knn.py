@@ -88,3 +88,36 @@ def test_distance_expression_is_unfused_fp32(oracle_lib):
     dx, dy, dz = (np.float32(src[0, a] - qry[0, a]) for a in range(3))
     expect = np.float32(np.float32(np.float32(dx * dx) + np.float32(dy * dy)) + np.float32(dz * dz))
     assert d2[0, 0] == expect
+
+
+def test_interpolate_closed_forms(oracle_lib):
+    """Pins of the inverse-distance interpolation: hand-computed weights, a constant field, a query on
+    top of a source, padded slots."""
+    # two neighbours at distances 1 and 3: weights (1/1, 1/3) / (4/3) = 0.75, 0.25
+    idx = np.array([[0, 1]], np.int32)
+    d2 = np.array([[1.0, 9.0]], np.float32)
+    feat = np.array([[8.0, -4.0], [0.0, 4.0]], np.float32)
+    np.testing.assert_allclose(oracle_lib.knn_interpolate(idx, d2, feat), [[6.0, -2.0]], rtol=1e-7)
+    # three neighbours at distances 1, 2, 4: weights 4/7, 2/7, 1/7
+    idx = np.array([[2, 0, 1]], np.int32)
+    d2 = np.array([[1.0, 4.0, 16.0]], np.float32)
+    feat = np.array([[7.0], [14.0], [21.0]], np.float32)       # rows 2, 0, 1 -> 21, 7, 14
+    np.testing.assert_allclose(oracle_lib.knn_interpolate(idx, d2, feat), [[(4 * 21 + 2 * 7 + 14) / 7.0]], rtol=1e-7)
+    # constant field stays constant; a query on a source returns that source (weight 1e8 against ~1)
+    rng = np.random.default_rng(27)
+    src, qry = _cloud(rng, 200), _cloud(rng, 50)
+    qry[:10] = src[:10]
+    one_s, one_q = np.array([200], np.int32), np.array([50], np.int32)
+    idx, d2 = oracle_lib.knn(3, src, qry, one_s, one_q)
+    const = np.full((200, 5), 3.25, np.float32)
+    np.testing.assert_allclose(oracle_lib.knn_interpolate(idx, d2, const), 3.25, rtol=1e-12)
+    feat = rng.standard_normal((200, 5)).astype(np.float32)
+    out = oracle_lib.knn_interpolate(idx, d2, feat)
+    np.testing.assert_allclose(out[:10], feat[:10], rtol=0, atol=1e-6)
+    # result lies in the convex hull of the neighbours' features
+    lo, hi = feat[idx].min(1), feat[idx].max(1)
+    assert (out >= lo - 1e-9).all() and (out <= hi + 1e-9).all()
+    # padded slots (segment with fewer sources than K) carry no weight
+    idx = np.array([[1, -1, -1]], np.int32)
+    d2 = np.array([[4.0, 2147483648.0, 2147483648.0]], np.float32)
+    np.testing.assert_allclose(oracle_lib.knn_interpolate(idx, d2, feat), feat[1:2], rtol=1e-12)
