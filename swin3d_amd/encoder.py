@@ -14,6 +14,8 @@ What each piece mirrors in the reference (semantics, not code):
   GridKNNDownsample                     same name                      :272-315
   WindowAttention / SwinBlock / Stage   WindowAttention, SwinTransformerBlock, BasicLayer  :382-871
   Swin3DEncoder                         same name                      Swin3D/models/Swin3D.py:185-269
+  query_knn_feature, knn_linear_interpolation, Upsample   same names   Swin3D/modules/swin3d_layers.py:27-73, 318-379
+  Swin3DUNet, load_state_with_same_shape                  same names   Swin3D/models/Swin3D.py:12-183
 MinkowskiEngine's output ORDER of pooled coordinates and its tie-breaking are not pinned by
 anything in the reference; here pooled voxels are sorted by (batch, x, y, z) and ties go to
 the lower row.  Stochastic depth is inference-time identity.
@@ -26,7 +28,7 @@ import torch.nn.functional as F
 
 from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
 from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
-from .sparse_dl.knn import KNN
+from .sparse_dl.knn import KNN, KNNInterpolate, knn_query
 from .window_index import get_index01
 
 
@@ -260,6 +262,135 @@ class Swin3DEncoder(nn.Module):
             here, voxels, signals = layer(voxels, signals)
             outputs.append(here)
         return outputs
+
+
+def query_knn_feature(K, src_xyz, query_xyz, src_feat, src_offset, query_offset, return_idx=False):
+    """Features of the K nearest sources of every query, [Nq,K,C] (swin3d_layers.py:27-50).  Slots
+    of segments with fewer than K sources repeat source row 0 of the gather (index clamped)."""
+    if query_xyz is None:
+        query_xyz, query_offset = src_xyz, src_offset
+    idx, _ = KNN.apply(K, src_xyz, query_xyz, src_offset, query_offset)
+    grouped = src_feat[idx.view(-1).long().clamp_(min=0)].view(query_xyz.shape[0], K, src_feat.shape[1])
+    return (grouped, idx) if return_idx else grouped
+
+
+def knn_linear_interpolation(src_xyz, query_xyz, src_feat, src_offset, query_offset, K=3):
+    """Inverse-distance interpolation of src_feat at the queries (swin3d_layers.py:53-73): one KNN
+    call and one fused gather kernel; differentiable w.r.t. src_feat."""
+    idx, dist2 = knn_query(K, src_xyz.contiguous(), query_xyz.contiguous(), src_offset, query_offset, KNN.cell_size)
+    return KNNInterpolate.apply(idx, dist2, src_feat.contiguous())
+
+
+class Upsample(nn.Module):
+    """Coarse features interpolated onto the finer voxel set and added to its projected skip features,
+    optionally followed by one attention block (swin3d_layers.py:318-379)."""
+
+    def __init__(self, in_channels, out_channels, num_heads, window_size, quant_size, attn=True, up_k=3,
+                 cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.linear1 = nn.Sequential(nn.LayerNorm(out_channels), nn.Linear(out_channels, out_channels))
+        self.linear2 = nn.Sequential(nn.LayerNorm(in_channels), nn.Linear(in_channels, out_channels))
+        self.up_k = up_k
+        self.attn = attn and window_size > 0
+        if self.attn:
+            self.block = Stage(out_channels, 1, num_heads, window_size, quant_size, downsample=False, cRSE=cRSE,
+                               fp16_mode=fp16_mode)
+
+    def forward(self, voxels, signals, voxels_up, signals_up):
+        """(voxels, signals): the coarse level; (voxels_up, signals_up): the finer level it feeds."""
+        xyz = signals[:, 1:4].detach().contiguous().float()
+        support_xyz = signals_up[:, 1:4].detach().contiguous().float()
+        feats = self.linear1(voxels_up.feats) + knn_linear_interpolation(
+            xyz, support_xyz, self.linear2(voxels.feats).float(), segment_offsets(voxels.coords[:, 0]),
+            segment_offsets(voxels_up.coords[:, 0]), K=self.up_k)
+        voxels_up = voxels_up.with_feats(feats.float())
+        if self.attn:
+            voxels_up, _, _ = self.block(voxels_up, signals_up)
+        return voxels_up
+
+
+def load_state_with_same_shape(model, weights, skip_first_conv=False, verbose=True):
+    """The subset of a checkpoint's state dict that this model can take (Swin3D/models/Swin3D.py:12-40):
+    a `module.` prefix is stripped, decoder (`upsamples`) and `classifier` entries are dropped, so is
+    `stem_layer` on request, and so is every entry whose name or shape the model does not have."""
+    if weights and next(iter(weights)).startswith("module."):
+        if verbose:
+            print("Loading multigpu weights with module. prefix...")
+        weights = {k.partition("module.")[2]: v for k, v in weights.items()}
+    model_state = model.state_dict()
+    dropped = [k for k in weights if "upsamples" in k or "classifier" in k]
+    weights = {k: v for k, v in weights.items() if "upsamples" not in k and "classifier" not in k}
+    if skip_first_conv:
+        dropped += [k for k in weights if "stem_layer" in k]
+        weights = {k: v for k, v in weights.items() if "stem_layer" not in k}
+    filtered = {k: v for k, v in weights.items() if k in model_state and v.size() == model_state[k].size()}
+    dropped += [k for k, v in weights.items() if k in model_state and v.size() != model_state[k].size()]
+    missing = [k for k in model_state if k not in weights]
+    if verbose:
+        print("Not Loading weights: " + ", ".join(dropped))
+        print("=" * 100)
+        print("Not found weights: " + ", ".join(missing))
+        print("=" * 100)
+    return filtered
+
+
+class Swin3DUNet(nn.Module):
+    """Encoder stages, the Upsample decoder and the per-voxel classifier (Swin3D/models/Swin3D.py:42-183,
+    stem_transformer=True layout)."""
+
+    def __init__(self, depths, channels, num_heads, window_sizes, quant_size, up_k=3, num_layers=5, num_classes=13,
+                 first_down_stride=2, upsample="linear", in_channels=6, cRSE="XYZ_RGB", fp16_mode=0):
+        super().__init__()
+        self.stem_layer = StemConv(in_channels, channels[0])
+        self.layers = nn.ModuleList([
+            Stage(channels[i], depths[i], num_heads[i], window_sizes[i], quant_size,
+                  out_channels=channels[i + 1] if i < num_layers - 1 else None,
+                  down_stride=first_down_stride if i == 0 else 2, downsample=i < num_layers - 1,
+                  cRSE=cRSE, fp16_mode=fp16_mode)
+            for i in range(num_layers)])
+        self.upsamples = nn.ModuleList([
+            Upsample(channels[i], channels[i - 1], num_heads[i - 1], window_sizes[i - 1], quant_size,
+                     attn="attn" in upsample, up_k=up_k, cRSE=cRSE, fp16_mode=fp16_mode)
+            for i in range(num_layers - 1, 0, -1)])
+        self.classifier = nn.Sequential(nn.Linear(channels[0], channels[0]), nn.BatchNorm1d(channels[0]),
+                                        nn.ReLU(inplace=True), nn.Linear(channels[0], num_classes))
+        self.num_classes = num_classes
+        for m in self.modules():
+            if isinstance(m, nn.Linear):
+                nn.init.trunc_normal_(m.weight, std=0.02)
+                if m.bias is not None:
+                    nn.init.zeros_(m.bias)
+
+    def forward(self, voxels, signals):
+        """-> logits [N, num_classes] on the input voxels."""
+        voxels = self.stem_layer(voxels)
+        levels = []
+        for layer in self.layers:
+            here, voxels_next, signals_next = layer(voxels, signals)
+            levels.append((here, signals))
+            voxels, signals = voxels_next, signals_next
+        voxels, signals = levels.pop()
+        for upsample in self.upsamples:
+            voxels_up, signals_up = levels.pop()
+            voxels = upsample(voxels, signals, voxels_up, signals_up)
+            signals = signals_up
+        return self.classifier(voxels.feats.float())
+
+    def load_pretrained_model(self, ckpt, skip_first_conv=True, verbose=True):
+        """Load the entries of a checkpoint that fit (Swin3D/models/Swin3D.py:173-183); the file is read
+        with a loader that executes nothing from it."""
+        import os
+        if not os.path.isfile(ckpt):
+            if verbose:
+                print("=> no weight found at '{}'".format(ckpt))
+            return []
+        checkpoint = torch.load(ckpt, map_location="cpu", weights_only=True)
+        weights = checkpoint["state_dict"] if "state_dict" in checkpoint else checkpoint
+        matched = load_state_with_same_shape(self, weights, skip_first_conv=skip_first_conv, verbose=verbose)
+        self.load_state_dict(matched, strict=False)
+        if verbose:
+            print("=> loaded weight '{}'".format(ckpt))
+        return sorted(matched)
 
 
 SWIN3D_S = dict(depths=[2, 4, 9, 4, 4], channels=[48, 96, 192, 384, 384], num_heads=[6, 6, 12, 24, 24],

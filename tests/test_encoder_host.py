@@ -70,3 +70,32 @@ def test_pack_coords_is_order_preserving():
     coords = torch.tensor([[0, -5, 3, 2], [0, -5, 3, 3], [0, 4, -100000, 0], [1, -200000, 0, 0], [63, 0, 0, 0]])
     keys = encoder.pack_coords(coords)
     assert (keys[1:] > keys[:-1]).all()
+
+
+def test_load_state_with_same_shape_filters_like_the_reference(tmp_path):
+    """Key filtering of Swin3D/models/Swin3D.py:12-40: `module.` prefix stripped, decoder / classifier /
+    (optionally) stem entries dropped, wrong shapes dropped; then load_pretrained_model on a file."""
+    from swin3d_amd import encoder
+    torch.manual_seed(0)
+    cfg = dict(depths=[1, 1], channels=[16, 32], num_heads=[2, 2], window_sizes=[5, 7], quant_size=4, num_layers=2)
+    model = encoder.Swin3DUNet(**cfg, in_channels=6, cRSE="XYZ_RGB", num_classes=5)
+    donor = encoder.Swin3DUNet(**cfg, in_channels=6, cRSE="XYZ_RGB", num_classes=5)
+    state = {"module." + k: v.clone() + 1.0 for k, v in donor.state_dict().items() if v.dtype.is_floating_point}
+    bad = "module.layers.0.blocks.0.attn.proj.weight"
+    state[bad] = torch.zeros(3, 3)                                  # wrong shape
+    state["module.not_in_model.weight"] = torch.zeros(2)            # unknown name
+    kept = encoder.load_state_with_same_shape(model, state, skip_first_conv=True, verbose=False)
+    assert kept and all(not k.startswith("module.") for k in kept)
+    assert not any("upsamples" in k or "classifier" in k or "stem_layer" in k for k in kept)
+    assert "layers.0.blocks.0.attn.proj.weight" not in kept and "not_in_model.weight" not in kept
+    assert "layers.0.blocks.0.attn.qkv.weight" in kept
+    kept_with_stem = encoder.load_state_with_same_shape(model, state, skip_first_conv=False, verbose=False)
+    assert any("stem_layer" in k for k in kept_with_stem)
+    path = tmp_path / "ckpt.pth"
+    torch.save({"state_dict": state}, path)
+    before = model.state_dict()["layers.0.blocks.0.attn.qkv.weight"].clone()
+    loaded = model.load_pretrained_model(str(path), verbose=False)
+    after = model.state_dict()["layers.0.blocks.0.attn.qkv.weight"]
+    assert "layers.0.blocks.0.attn.qkv.weight" in loaded
+    assert torch.equal(after, donor.state_dict()["layers.0.blocks.0.attn.qkv.weight"] + 1.0) and not torch.equal(after, before)
+    assert model.load_pretrained_model(str(tmp_path / "missing.pth"), verbose=False) == []

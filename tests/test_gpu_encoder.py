@@ -70,3 +70,42 @@ def test_knn_downsample_matches_oracle_neighbours(oracle_lib, hip_lib):
     # the representative of a cell is one of the cell's own points
     cell = torch.div(coarse_signals[:, 1:4], 2, rounding_mode="floor") * 2
     assert torch.equal(cell.int(), coarse.coords[:, 1:])
+
+
+def _small_unet(fp16_mode, upsample="linear_attn"):
+    torch.manual_seed(0)
+    cfg = dict(depths=[1, 1, 1], channels=[48, 96, 192], num_heads=[6, 6, 12], window_sizes=[5, 7, 7],
+               quant_size=4, num_layers=3)
+    return encoder.Swin3DUNet(**cfg, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=fp16_mode, num_classes=13,
+                              upsample=upsample).cuda()
+
+
+def test_unet_forward_and_training_step(hip_lib):
+    """Swin3DUNet: logits on the input voxels; one optimisation step in fp32 (attention backward through
+    s3d_attn_bwd, interpolation backward) lowers the loss on a fixed batch."""
+    vox, signals = _inputs(target=5000, batches=2)
+    model = _small_unet(fp16_mode=0)
+    labels = (vox.coords[:, 3] // 8 % 13).long()           # height bands: learnable from the features
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    losses = []
+    for _ in range(3):
+        opt.zero_grad()
+        logits = model(vox, signals)
+        assert logits.shape == (vox.coords.shape[0], 13) and torch.isfinite(logits).all()
+        loss = torch.nn.functional.cross_entropy(logits, labels)
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    table = model.layers[0].blocks[0].attn.query_xyz_table
+    assert table.grad is not None and torch.isfinite(table.grad).all() and float(table.grad.abs().max()) > 0
+    qkv = model.layers[1].blocks[0].attn.qkv.weight
+    assert qkv.grad is not None and float(qkv.grad.abs().max()) > 0
+    assert losses[-1] < losses[0], losses
+
+
+def test_unet_forward_fp16(hip_lib):
+    vox, signals = _inputs(target=5000, batches=1)
+    model = _small_unet(fp16_mode=2, upsample="linear").eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        logits = model(vox, signals)
+    assert logits.shape == (vox.coords.shape[0], 13) and torch.isfinite(logits).all()
