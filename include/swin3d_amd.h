@@ -124,7 +124,7 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
  *   dq, dk, dv     device [N,H,D] of `dtype`, overwritten (every row belongs to exactly one window)
  *   dtable_q/k/v   device FP32 [table_len], overwritten; layout of the tables
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, N, W) bytes
- *   D in {8,16}, nd in {3,6,9}, every axis table of at most 64 rows.
+ *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
  * dq, dk, dv are sums in a fixed order (deterministic); the table gradients are accumulated per
  * wavefront and added to global memory with fp32 atomics (order varies between runs).

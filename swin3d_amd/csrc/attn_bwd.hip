@@ -162,17 +162,20 @@ __global__ void bwd_reset_counters_kernel(BwdArgs a)
     for (int t = threadIdx.x; t < a.H; t += blockDim.x) a.units[a.W + t] = 0;
 }
 
-// MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv (not launched: too many registers); 1 = dk, dTq;
-// 2 = dv, dTv.
+// MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv (head_dim 8); 1 = dk, dTq; 2 = dv, dTv (head_dim 16:
+// both sets of table-gradient registers do not fit one wavefront).
 // The query-owned sweep produces dq and dTk.
-template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
+// BLK: 64-row blocks of the head's flat table (all axes back to back) that the wavefront's
+// table-gradient registers cover; lane l of block m owns flat row 64 m + l.
+template <typename T, int D, int ND, bool KEY_OWNED, int MODE, int BLK>
 __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_kernel(BwdArgs a)
 {
     constexpr bool kNeedDl = !KEY_OWNED || MODE != 2;          // dP / dL are needed
     constexpr bool kAccA = kNeedDl;                            // dTq (key-owned) or dTk (query-owned)
     constexpr bool kAccB = KEY_OWNED && MODE != 1;             // dTv
     constexpr int kHistKinds = (kAccA ? 1 : 0) + (kAccB ? 1 : 0);
-    constexpr int kHistWords = kHistKinds * 2 * ND * 64;       // [kind][group][axis][row]
+    constexpr int kFlat = BLK * 64;                            // flat table rows covered (>= total_rows)
+    constexpr int kHistWords = kHistKinds * 2 * kFlat;         // [kind][group][flat row]
 
     extern __shared__ float smem[];
     const int H = a.H;
@@ -202,18 +205,18 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     int *hist_a = hist_all + wave * kHistWords;                 // dL histogram
-    int *hist_b = hist_a + (kAccA ? 2 * ND * 64 : 0);           // P histogram
+    int *hist_b = hist_a + (kAccA ? 2 * kFlat : 0);             // P histogram
 
     const T *gq = static_cast<const T *>(a.q);
     const T *gk = static_cast<const T *>(a.k);
     const T *gv = static_cast<const T *>(a.v);
     const T *ggo = static_cast<const T *>(a.dout);
 
-    float acc_a[ND][D], acc_b[ND][D];
+    float acc_a[BLK][D], acc_b[BLK][D];
 #pragma unroll
-    for (int n = 0; n < ND; ++n)
+    for (int m = 0; m < BLK; ++m)
 #pragma unroll
-        for (int c = 0; c < D; ++c) acc_a[n][c] = acc_b[n][c] = 0.0f;
+        for (int c = 0; c < D; ++c) acc_a[m][c] = acc_b[m][c] = 0.0f;
 
     const int *unit_end = a.units;
     const int total_units = __builtin_amdgcn_readfirstlane(unit_end[a.W - 1]);
@@ -352,14 +355,14 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                 const int qd = __float2int_rn(dl * (amax > 0.0f ? kFixL / amax : 0.0f));
                 if (valid && qd != 0) {
 #pragma unroll
-                    for (int n = 0; n < ND; ++n) atomicAdd(hist_a + (grp * ND + n) * 64 + r[n], qd);
+                    for (int n = 0; n < ND; ++n) atomicAdd(hist_a + grp * kFlat + a.base[n] + r[n], qd);
                 }
             }
             if constexpr (kAccB) {
                 const int qp = __float2int_rn(p * kFixP);
                 if (valid && qp != 0) {
 #pragma unroll
-                    for (int n = 0; n < ND; ++n) atomicAdd(hist_b + (grp * ND + n) * 64 + r[n], qp);
+                    for (int n = 0; n < ND; ++n) atomicAdd(hist_b + grp * kFlat + a.base[n] + r[n], qp);
                 }
             }
             wave_lds_fence();
@@ -371,12 +374,12 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 #pragma unroll
                     for (int c = 0; c < D; ++c) sx[c] = lane_value(st_x[c], src);   // q_i (key-owned) or k_j
 #pragma unroll
-                    for (int n = 0; n < ND; ++n) {
-                        int *cell = hist_a + (g * ND + n) * 64 + lane;
+                    for (int m = 0; m < BLK; ++m) {
+                        int *cell = hist_a + g * kFlat + m * 64 + lane;
                         const float gsum = static_cast<float>(*cell) * sc;
                         *cell = 0;
 #pragma unroll
-                        for (int c = 0; c < D; ++c) acc_a[n][c] += gsum * sx[c];
+                        for (int c = 0; c < D; ++c) acc_a[m][c] += gsum * sx[c];
                     }
                 }
                 if constexpr (kAccB) {
@@ -384,12 +387,12 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 #pragma unroll
                     for (int c = 0; c < D; ++c) sy[c] = lane_value(st_y[c], src);   // dout_i
 #pragma unroll
-                    for (int n = 0; n < ND; ++n) {
-                        int *cell = hist_b + (g * ND + n) * 64 + lane;
+                    for (int m = 0; m < BLK; ++m) {
+                        int *cell = hist_b + g * kFlat + m * 64 + lane;
                         const float psum = static_cast<float>(*cell) * (1.0f / kFixP);
                         *cell = 0;
 #pragma unroll
-                        for (int c = 0; c < D; ++c) acc_b[n][c] += psum * sy[c];
+                        for (int c = 0; c < D; ++c) acc_b[m][c] += psum * sy[c];
                     }
                 }
             }
@@ -416,34 +419,35 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         }
     }
 
-    // lane = table row: add this wavefront's table gradients to the global tables
+    // lane l of block m = flat table row 64 m + l: add this wavefront's table gradients to the global tables
     float *dst_a = KEY_OWNED ? a.dtq : a.dtk;
 #pragma unroll
-    for (int n = 0; n < ND; ++n) {
-        if (lane < a.rows[n]) {
-            const int64_t g = static_cast<int64_t>(a.base[n] + lane) * HD + h * D;
+    for (int m = 0; m < BLK; ++m) {
+        const int row = m * 64 + lane;
+        if (row < a.total_rows) {
+            const int64_t g = static_cast<int64_t>(row) * HD + h * D;
 #pragma unroll
             for (int c = 0; c < D; ++c) {
-                if constexpr (kAccA) atomicAdd(dst_a + g + c, acc_a[n][c]);
-                if constexpr (kAccB) atomicAdd(a.dtv + g + c, acc_b[n][c]);
+                if constexpr (kAccA) atomicAdd(dst_a + g + c, acc_a[m][c]);
+                if constexpr (kAccB) atomicAdd(a.dtv + g + c, acc_b[m][c]);
             }
         }
     }
 }
 
-template <int KINDS> size_t bwd_lds_bytes(const BwdArgs &a)
+size_t bwd_lds_bytes(const BwdArgs &a, int kinds, int blk)
 {
     return sizeof(float) * 3 * static_cast<size_t>(a.total_rows) * a.D +
-           sizeof(int) * kBwdWaves * KINDS * 2 * static_cast<size_t>(a.nd) * 64;
+           sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(blk) * 64;
 }
 
-template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
-int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
+template <typename T, int D, int ND, bool KEY_OWNED, int MODE, int BLK>
+int launch_sweep_blk(const BwdArgs &a, int grid, hipStream_t stream)
 {
     constexpr bool need_dl = !KEY_OWNED || MODE != 2;
     constexpr int kinds = (need_dl ? 1 : 0) + ((KEY_OWNED && MODE != 1) ? 1 : 0);
-    auto kernel = attn_bwd_sweep_kernel<T, D, ND, KEY_OWNED, MODE>;
-    const size_t lds = bwd_lds_bytes<kinds>(a);
+    auto kernel = attn_bwd_sweep_kernel<T, D, ND, KEY_OWNED, MODE, BLK>;
+    const size_t lds = bwd_lds_bytes(a, kinds, BLK);
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: the tables of one head (%d rows x %d) do not fit LDS",
                     a.total_rows, a.D);
@@ -453,6 +457,15 @@ int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
+}
+
+// the usual tables (quant 4: 32-row colour / normal axes) fit 2/3 of ND blocks; any table fits ND blocks
+template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
+int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
+{
+    constexpr int kSmall = 2 * ND / 3;
+    if (a.total_rows <= 64 * kSmall) return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, kSmall>(a, grid, stream);
+    return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, ND>(a, grid, stream);
 }
 
 template <typename T, int D, int ND>
@@ -472,10 +485,13 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
     // a workgroup serves one head for its whole life: a multiple of H workgroups, about two per CU
     const int per_head = (2 * cus + a.H - 1) / a.H;
     const int grid = per_head * a.H;
-    // two key-owned sweeps (dk + dTq, then dv + dTv): one sweep with both sets of table-gradient registers
-    // spills at two wavefronts per SIMD and measured slower
-    if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
-    if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
+    if constexpr (D <= 8) {
+        // one key-owned sweep when both sets of table-gradient registers fit two wavefronts per SIMD
+        if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
+    } else {
+        if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
+        if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
+    }
     return launch_sweep<T, D, ND, false, 0>(a, grid, stream);
 }
 
@@ -493,14 +509,14 @@ int fill_bwd_axes(BwdArgs &a, const int32_t *table_sizes, int nd, int64_t table_
         a.rows[n] = static_cast<int32_t>(size / hd);
         a.base[n] = base;
         base += a.rows[n];
-        if (a.rows[n] > 64)
-            return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: axis table %d has %d rows (at most 64)", n, a.rows[n]);
     }
     for (int n = nd; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = 0;
     if (total != table_len)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: sum(table_sizes) = %lld differs from table_len = %lld",
                     (long long)total, (long long)table_len);
     a.total_rows = base;
+    if (base > 64 * nd)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d table rows per head (at most %d)", base, 64 * nd);
     return S3D_OK;
 }
 

@@ -189,8 +189,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_len:
         raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
                          f"to the table length {table_len}")
-    if max(sizes) // (h * d) > 64:
-        raise NotImplementedError("attention backward supports axis tables of at most 64 rows")
+    if sum(sizes) // (h * d) > 64 * nd:
+        raise NotImplementedError(f"attention backward supports at most {64 * nd} table rows per head")
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
         if t.dtype != q.dtype or t.numel() != table_len:
