@@ -181,7 +181,10 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int H = a.H;
     const int HD = H * D;
     const int h = blockIdx.x % H;
-    const int cells = a.total_rows * D;
+    // fp32 table slices of the head, rows padded by 16 bytes: with a 32- or 64-byte row stride a wavefront's
+    // 16-byte gathers of different rows would fall on 4 or 2 of the eight 4-bank groups
+    constexpr int kRowStride = D + 4;
+    const int cells = a.total_rows * kRowStride;
     float *tab_q = smem;
     float *tab_k = tab_q + cells;
     float *tab_v = tab_k + cells;
@@ -191,12 +194,12 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         const T *gq = static_cast<const T *>(a.table_q);
         const T *gk = static_cast<const T *>(a.table_k);
         const T *gv = static_cast<const T *>(a.table_v);
-        for (int t = threadIdx.x; t < cells; t += kBwdThreads) {
+        for (int t = threadIdx.x; t < a.total_rows * D; t += kBwdThreads) {
             const int r = t / D, c = t - r * D;
             const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
-            tab_q[t] = as_float(gq[g]);
-            tab_k[t] = as_float(gk[g]);
-            tab_v[t] = as_float(gv[g]);
+            tab_q[r * kRowStride + c] = as_float(gq[g]);
+            tab_k[r * kRowStride + c] = as_float(gk[g]);
+            tab_v[r * kRowStride + c] = as_float(gv[g]);
         }
         for (int t = threadIdx.x; t < kBwdWaves * kHistWords; t += kBwdThreads) hist_all[t] = 0;
     }
@@ -303,7 +306,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                 const float ci = KEY_OWNED ? st_c[n] : own_c[n];
                 const float cj = KEY_OWNED ? own_c[n] : st_c[n];
                 r[n] = crse_row(ci, cj, a.rows[n]);
-                const int off = (a.base[n] + r[n]) * D;
+                const int off = (a.base[n] + r[n]) * kRowStride;
                 float tq_r[D], tk_r[D];
                 load_row<D>(tab_q + off, tq_r);
                 load_row<D>(tab_k + off, tk_r);
@@ -437,7 +440,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 
 size_t bwd_lds_bytes(const BwdArgs &a, int kinds, int blk)
 {
-    return sizeof(float) * 3 * static_cast<size_t>(a.total_rows) * a.D +
+    return sizeof(float) * 3 * static_cast<size_t>(a.total_rows) * (a.D + 4) +
            sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(blk) * 64;
 }
 
