@@ -96,7 +96,7 @@ def main():
                                   tk_d.data_ptr(), tv_d.data_ptr(), c_sizes, nd, table_len,
                                   index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
                                   n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  index.max_window_voxels, _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
+                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
                                   stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")

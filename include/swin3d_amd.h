@@ -61,7 +61,7 @@ const char *s3d_last_error_string(void);
  * indice_mode INDIRECT (2), in ONE pass and without the O(M) pair arrays
  * m2w_indices / w2m_offsets.
  *
- *   q, k, v        device [N,H,D] of `dtype`, original voxel order (q pre-scaled)
+ *   q, k, v        device [N,H,D] of `dtype`, original voxel order (q pre-scaled); see qkv_row_stride
  *   table_q/k/v    device [table_len] of `dtype`, layout [axis][row][h][c]
  *   table_sizes    HOST int32 [nd], table_sizes[n] = rows_n * H * D (the values of the
  *                  reference's `table_offsets` tensor, fwd.cu:258,285; read on the host so
@@ -79,6 +79,10 @@ const char *s3d_last_error_string(void);
  *                  window^3).  It sizes the per-key-tile partial results of windows with more than 32
  *                  voxels; a window larger than the bound is skipped (its output rows are not
  *                  written), so the bound must hold for a complete result.
+ *   qkv_row_stride elements between consecutive voxel rows of q, k and v (0 = H*D, dense).  A multiple
+ *                  of 8 that is >= H*D: with 3*H*D and q, k, v pointing H*D apart the kernels read the
+ *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
+ *                  place, without the reference's reshape / permute / contiguous copy.
  *   flags          0, or S3D_ATTN_FORCE_GENERIC to run the VALU kernel for every case
  *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
  *                  (MFMA kernel: a transposed copy of the value table, the work list, and
@@ -105,8 +109,8 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
                  const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
                  int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
                  const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
-                 int32_t H, int32_t D, int64_t W, int32_t max_window_voxels, int32_t dtype,
-                 int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
+                 int32_t H, int32_t D, int64_t W, int32_t max_window_voxels, int64_t qkv_row_stride,
+                 int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Windowed self-attention backward.

@@ -84,14 +84,18 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
     const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
     float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W,
-    int32_t max_window_voxels, int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes,
-    void *stream)
+    int32_t max_window_voxels, int64_t qkv_row_stride, int32_t dtype, int32_t flags, void *workspace,
+    size_t workspace_bytes, void *stream)
 {
     using namespace s3d;
     if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
     if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
         return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_fwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
     if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_fwd: table_sizes (host) is null");
+    // rows of q, k, v are read with 16-byte loads: the stride must keep them aligned
+    if (qkv_row_stride != 0 && (qkv_row_stride < static_cast<int64_t>(H) * D || qkv_row_stride % 8 != 0))
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: qkv_row_stride = %lld (0, or a multiple of 8 that is >= H*D = %d)",
+                    (long long)qkv_row_stride, H * D);
     AttnArgs a{};
     a.H = H;
     a.D = D;
@@ -105,6 +109,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.q = q;
     a.k = k;
     a.v = v;
+    a.row_stride = qkv_row_stride == 0 ? static_cast<int64_t>(H) * D : qkv_row_stride;
     a.table_q = table_q;
     a.table_k = table_k;
     a.table_v = table_v;

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_window_head_kernel(
     AxisRows<ND> axes, int total_rows, const int32_t *__restrict__ w_sizes,
     const int32_t *__restrict__ w2n, const int32_t *__restrict__ n2n,
     const float *__restrict__ n_coords, T *__restrict__ out, float *__restrict__ out_max,
-    float *__restrict__ out_sum, int H)
+    float *__restrict__ out_sum, int H, int64_t row_stride)
 {
     extern __shared__ float smem[];
     float *tab_q = smem;                         // [total_rows][D]
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_window_head_kernel(
         int q_row = 0;
         if (valid_q) {
             q_row = n2n[s0 + i];
-            const T *qp = q + static_cast<int64_t>(q_row) * HD + h * D;
+            const T *qp = q + static_cast<int64_t>(q_row) * row_stride + h * D;
 #pragma unroll
             for (int c = 0; c < D; ++c) qv[c] = to_float(qp[c]);
 #pragma unroll
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_window_head_kernel(
             __syncthreads();  // previous chunk (and the table staging) fully consumed / written
             for (int idx = tid; idx < kend * D; idx += kThreads) {
                 const int jj = idx / D, c = idx % D;
-                const int64_t g = static_cast<int64_t>(n2n[s0 + k0 + jj]) * HD + h * D + c;
+                const int64_t g = static_cast<int64_t>(n2n[s0 + k0 + jj]) * row_stride + h * D + c;
                 key_s[idx] = to_float(k[g]);
                 val_s[idx] = to_float(v[g]);
             }
@@ -216,7 +216,7 @@ int launch_window_head(const AttnArgs &a, hipStream_t stream)
                        static_cast<const T *>(a.k), static_cast<const T *>(a.v),
                        static_cast<const T *>(a.table_q), static_cast<const T *>(a.table_k),
                        static_cast<const T *>(a.table_v), axes, a.total_rows, a.w_sizes, a.w2n, a.n2n,
-                       a.n_coords, static_cast<T *>(a.out), a.out_max, a.out_sum, a.H);
+                       a.n_coords, static_cast<T *>(a.out), a.out_max, a.out_sum, a.H, a.row_stride);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }

@@ -236,9 +236,9 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
         frag_t qf_next, kf_next;
         h8 vv_next;
         auto prefetch_head = [&](int hh) {
-            qf_next = load_frag<D>(gq + static_cast<int64_t>(q_row) * HD + hh * D, half);
-            kf_next = load_frag<D>(gk + static_cast<int64_t>(k_row) * HD + hh * D, half);
-            vv_next = *reinterpret_cast<const h8 *>(gv + static_cast<int64_t>(k_row) * HD + hh * D +
+            qf_next = load_frag<D>(gq + static_cast<int64_t>(q_row) * a.row_stride + hh * D, half);
+            kf_next = load_frag<D>(gk + static_cast<int64_t>(k_row) * a.row_stride + hh * D, half);
+            vv_next = *reinterpret_cast<const h8 *>(gv + static_cast<int64_t>(k_row) * a.row_stride + hh * D +
                                                     (D == 16 ? 8 * half : 0));
         };
         prefetch_head(h_begin);

@@ -9,7 +9,8 @@ constexpr int kMaxAxes = 9;
 
 // Everything a window-attention kernel needs, by value (lives in kernel-argument SGPRs).
 struct AttnArgs {
-    const void *q, *k, *v;                 // [N,H,D]
+    const void *q, *k, *v;                 // [N,H,D], voxel rows `row_stride` elements apart
+    int64_t row_stride;
     const void *table_q, *table_k, *table_v;  // flat [sum rows][H][D]
     const int32_t *w_sizes, *w2n, *n2n;
     const float *n_coords;                 // [N,nd], window-sorted

@@ -182,15 +182,21 @@ class WindowAttention(nn.Module):
     def forward(self, feats, attn_args):
         n = feats.shape[0]
         _, _, m2w, w_sizes, w2n, n2n, w2m, n_coords = attn_args
-        qkv = self.qkv(feats).reshape(n, 3, self.num_heads, self.head_dim).permute(1, 0, 2, 3).contiguous()
-        query, key, value = qkv[0] * self.scale, qkv[1], qkv[2]
+        # q scale folded into the projection (a C x C multiply instead of an N x C one); q, k, v stay
+        # slices of the [N, 3C] projection output, which the attention kernels read in place
+        scale = torch.ones(3 * self.dim, dtype=self.qkv.weight.dtype, device=self.qkv.weight.device)
+        scale[: self.dim] = self.scale
+        bias = None if self.qkv.bias is None else self.qkv.bias * scale
+        qkv = F.linear(feats, self.qkv.weight * scale.unsqueeze(1), bias).view(n, 3, self.num_heads, self.head_dim)
+        query, key, value = qkv[:, 0], qkv[:, 1], qkv[:, 2]
         n_crse = scale_crse_coords(n_coords, self.quant_size, self.cRSE)
         precision = (PrecisionMode.HALF_NONE, PrecisionMode.HALF_FORWARD, PrecisionMode.HALF_ALL)[self.fp16_mode]
         out = SelfAttnAIOFunction.apply(
             query, key, value, self._flat_table("query"), self._flat_table("key"), self._flat_table("value"),
             self.table_sizes, [m2w, w_sizes, w2m, w2n, n2n, n_crse], PosEmb.SEPARATE, TableDims.D0,
             IndexMode.INDIRECT, precision)
-        return self.proj(out.reshape(n, self.dim).to(feats.dtype))
+        out = out.reshape(n, self.dim)
+        return self.proj(out if torch.is_autocast_enabled() else out.to(feats.dtype))
 
 
 class SwinBlock(nn.Module):
@@ -203,8 +209,8 @@ class SwinBlock(nn.Module):
         self.mlp = nn.Sequential(nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
 
     def forward(self, feats, attn_args):
-        feats = feats + self.attn(self.norm1(feats), attn_args).float()
-        return feats + self.mlp(self.norm2(feats)).float()
+        feats = feats + self.attn(self.norm1(feats), attn_args)      # fp32 + fp16 promotes to fp32
+        return feats + self.mlp(self.norm2(feats))
 
 
 class Stage(nn.Module):

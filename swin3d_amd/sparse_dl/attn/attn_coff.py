@@ -6,7 +6,8 @@ can call it unchanged.  Differences in mechanism, not in result:
   * one fused HIP pass (s3d_attn_fwd) instead of cal_max_coffs + self_attn_forward + divide;
   * slots 0 and 2 of `indices` (the O(pairs) m2w / w2m arrays) are ignored and may be None;
   * only the combination the model uses is implemented (PosEmb.SEPARATE, TableDims.D0,
-    IndexMode.INDIRECT); the backward pass is not implemented yet.
+    IndexMode.INDIRECT);
+  * q, k, v may be strided views of the qkv projection output (read in place).
 """
 import ctypes
 import enum
@@ -46,15 +47,32 @@ _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_
 FORCE_GENERIC = False
 
 
-def _require_cuda(name, t, device=None):
+def _require_cuda(name, t, device=None, strided_rows=False):
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a CUDA (HIP) tensor")
     if device is not None and t.device != device:
         raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+    if strided_rows and _row_stride(t) is not None:
+        return
     if not t.is_contiguous():
         raise RuntimeError(f"{name} must be contiguous")
+
+
+def _row_stride(t):
+    """Row stride (elements) of an [N,H,D] tensor whose (H,D) block is dense and whose rows are a multiple
+    of 8 elements apart with 16-byte aligned storage: what the forward kernels read in place, e.g. the
+    q / k / v slices of the [N, 3*H*D] output of the qkv projection.  None for any other layout."""
+    if t.dim() != 3:
+        return None
+    n, h, d = t.shape
+    s0, s1, s2 = t.stride()
+    if n <= 1:
+        s0 = max(s0, h * d)
+    if s2 != 1 or s1 != d or s0 < h * d or s0 % 8 or (t.storage_offset() * t.element_size()) % 16:
+        return None
+    return s0
 
 
 def _as_int32(name, t, device):
@@ -83,7 +101,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
                              n_coords, return_stats=False, force_generic=False, max_window_voxels=None):
     """softmax-normalised window attention, [N,H,D] in the dtype of q.
 
-    q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5)
+    q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5); dense, or views with
+                   a dense (H,D) block and one common row stride (slices of a [N,3*H*D] projection output)
     table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
     table_sizes    int tensor / list [nd], per-axis element counts rows*H*D (read on the host)
     w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
@@ -94,7 +113,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
                    (set by build_window_index) or, failing that, read back from the device
     """
-    _require_cuda("query", q)
+    _require_cuda("query", q, strided_rows=True)
     dev = q.device
     if q.dim() != 3:
         raise ValueError(f"query must be [N,H,D], got {tuple(q.shape)}")
@@ -102,9 +121,14 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     if q.dtype not in _DTYPE_CODE:
         raise TypeError(f"unsupported feature dtype {q.dtype} (float16 or float32)")
     for name, t in (("key", k), ("value", v)):
-        _require_cuda(name, t, dev)
+        _require_cuda(name, t, dev, strided_rows=True)
         if t.shape != q.shape or t.dtype != q.dtype:
             raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
+    # q, k, v are read in place when they share one row stride (views of one projection output)
+    strides = {_row_stride(t) for t in (q, k, v)}
+    if len(strides) != 1 or None in strides:
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    row_stride = _row_stride(q)
     if d not in (8, 16):
         raise ValueError(f"head_dim must be 8 or 16, got {d}")
     sizes = _host_table_sizes(table_sizes)
@@ -136,7 +160,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
         raise ValueError(f"n_coords must be float32 [{n},{nd}], got {n_coords.dtype} {tuple(n_coords.shape)}")
 
-    out = torch.empty_like(q)
+    out = torch.empty((n, h, d), dtype=q.dtype, device=dev)
     omax = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     if max_window_voxels is None:
@@ -154,7 +178,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
             w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
-            n, h, d, w_sizes.numel(), max_window_voxels, _DTYPE_CODE[q.dtype],
+            n, h, d, w_sizes.numel(), max_window_voxels, row_stride, _DTYPE_CODE[q.dtype],
             _lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0, workspace.data_ptr(),
             ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
@@ -249,7 +273,8 @@ class SelfAttnAIOFunction(Function):
             raise NotImplementedError(f"compute dtype {c_dtype} is not supported (float16 / float32)")
         _, w_sizes, _, w2n, n2n, n_coords = indices
         raw = (raw_query_feats, raw_key_feats, raw_value_feats, query_table, key_table, value_table)
-        feats = [t.to(c_dtype).contiguous() for t in raw[:3]]
+        feats = [t.to(c_dtype) for t in raw[:3]]
+        feats = [t if _row_stride(t) is not None else t.contiguous() for t in feats]
         tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
         n_coords = n_coords.to(torch.float32).contiguous()
         needs_grad = any(ctx.needs_input_grad[:6])

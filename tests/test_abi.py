@@ -41,7 +41,7 @@ def test_argument_errors_are_reported_without_a_device(hip_lib):
     status = hip_lib.s3d_knn(0, None, 0, None, 0, None, None, 1, None, None, 0.0, None, 0, None)
     assert status < 0
     assert b"K=0" in hip_lib.s3d_last_error_string()
-    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 125, 1, 0, None, 0, None)
+    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 125, 0, 1, 0, None, 0, None)
     assert status < 0 and b"table_len" in hip_lib.s3d_last_error_string()
     try:
         _lib.check(status, "s3d_attn_fwd")

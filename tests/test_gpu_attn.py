@@ -138,6 +138,39 @@ def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib):
     assert_attn_close(got[rows_small], ref[rows_small], torch.float16)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_strided_qkv_views_are_read_in_place(oracle_lib, hip_lib, dtype):
+    """q, k, v as slices of one [N, 3*H*D] buffer (the layout of the qkv projection output): same result as
+    dense copies, on both kernels, and no copy is made (checked through the data pointers the op sees)."""
+    import swin3d_amd
+    from gpu_helpers import assert_attn_close
+    case = make_attn_case(oracle_lib, seed=39, n=1200, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
+    if dtype == torch.float16:
+        to_half_and_back(_sharp16(case))
+    ref = oracle_lib.attn_fwd(*case.oracle_args())
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    n, h, d = case.q.shape
+    packed = torch.stack([t(case.q), t(case.k), t(case.v)], dim=1).to(dtype).contiguous()    # [N,3,H,D]
+    q, k, v = packed[:, 0], packed[:, 1], packed[:, 2]
+    assert not q.is_contiguous() and q.stride(0) == 3 * h * d
+    i = case.index
+    f = lambda a: t(a).to(dtype)
+    for force_generic in (False, True):
+        got = swin3d_amd.window_attention_forward(q, k, v, f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
+                                                  t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
+                                                  force_generic=force_generic)
+        torch.cuda.synchronize()
+        assert got.is_contiguous() and got.shape == (n, h, d)
+        assert_attn_close(got.double().cpu().numpy(), ref, dtype)
+    # a row stride the kernels cannot read (not a multiple of 8 elements) is rejected, as non-contiguous
+    # input is by the reference's CHECK_INPUT
+    odd = torch.zeros((n, 3 * h * d + 3), dtype=dtype, device=dev)[:, : h * d].view(n, h, d)
+    with pytest.raises(RuntimeError):
+        swin3d_amd.window_attention_forward(odd, odd, odd, f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
+                                            t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
+
+
 def test_empty_input(hip_lib):
     import swin3d_amd
     dev = torch.device("cuda")
