@@ -102,7 +102,7 @@ __global__ __launch_bounds__(kThreads) void knn_init_kernel(KnnPlan *plan, int32
 
 // Bounding box of the sources: a small grid-stride grid so that only a few hundred atomics
 // meet on the six box words (one atomic pair per wavefront and axis).
-constexpr int kBboxBlocks = 64;
+constexpr int kBboxBlocks = 128;
 
 __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restrict__ src,
                                                             int64_t Ns, KnnPlan *plan)
@@ -126,12 +126,22 @@ __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restr
             hi[a] = max(hi[a], __shfl_down(hi[a], off));
         }
     }
+    // one set of global atomics per workgroup: they all land on the same six words and serialise
+    __shared__ int part[kThreads / 64][6];
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
         for (int a = 0; a < 3; ++a) {
-            atomicMin(&plan->lo[a], lo[a]);
-            atomicMax(&plan->hi[a], hi[a]);
+            part[threadIdx.x >> 6][a] = lo[a];
+            part[threadIdx.x >> 6][3 + a] = hi[a];
         }
+    }
+    __syncthreads();
+    if (threadIdx.x < 6) {
+        int v = part[0][threadIdx.x];
+        for (int w = 1; w < kThreads / 64; ++w)
+            v = threadIdx.x < 3 ? min(v, part[w][threadIdx.x]) : max(v, part[w][threadIdx.x]);
+        if (threadIdx.x < 3) atomicMin(&plan->lo[threadIdx.x], v);
+        else atomicMax(&plan->hi[threadIdx.x - 3], v);
     }
 }
 
