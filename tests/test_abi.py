@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_attn_fwd", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+    for must in ("s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -49,6 +49,33 @@ def test_argument_errors_are_reported_without_a_device(hip_lib):
         assert "s3d_attn_fwd failed" in str(e)
     else:
         raise AssertionError("check() must raise on a negative status")
+
+
+def test_more_argument_errors_without_a_device(hip_lib):
+    """Rejected before any launch: a row stride the kernels cannot read, the backward's table-row limit and
+    missing workspace, the interpolation's K and dtype."""
+    import ctypes
+    from swin3d_amd import crse
+    sizes = crse.crse_table_sizes(5, 4, 6, 8, "XYZ_RGB_NORM")
+    c_sizes = (ctypes.c_int32 * 9)(*sizes)
+    total = sum(sizes)
+    st = hip_lib.s3d_attn_fwd(*([None] * 6), c_sizes, 9, total, *([None] * 7), 10, 6, 8, 1, 125, 50, 1, 0, None, 0, None)
+    assert st < 0 and b"qkv_row_stride" in hip_lib.s3d_last_error_string()
+    # backward: workspace missing
+    st = hip_lib.s3d_attn_bwd(*([None] * 6), c_sizes, 9, total, *([None] * 14), 10, 6, 8, 1, 1, None, 0, None)
+    assert st < 0 and (b"gradient pointer" in hip_lib.s3d_last_error_string()
+                       or b"workspace" in hip_lib.s3d_last_error_string())
+    # backward: more table rows per head than its registers cover (window 10 at quant 8)
+    big = crse.crse_table_sizes(10, 8, 6, 8, "XYZ_RGB_NORM")
+    c_big = (ctypes.c_int32 * 9)(*big)
+    st = hip_lib.s3d_attn_bwd(*([None] * 6), c_big, 9, sum(big), *([None] * 14), 10, 6, 8, 1, 1, None, 0, None)
+    assert st < 0 and b"table rows per head" in hip_lib.s3d_last_error_string()
+    assert hip_lib.s3d_attn_bwd_workspace_bytes(6, 1000, 40) >= 4 * (40 + 6) + 4 * 6000
+    st = hip_lib.s3d_knn_interpolate(None, None, 0, 10, None, 10, 8, 0, None, None)
+    assert st < 0 and b"K=0" in hip_lib.s3d_last_error_string()
+    st = hip_lib.s3d_knn_interpolate(None, None, 3, 10, None, 10, 8, 7, None, None)
+    assert st < 0 and b"dtype" in hip_lib.s3d_last_error_string()
+    assert hip_lib.s3d_knn_interpolate(None, None, 3, 0, None, 10, 8, 0, None, None) == 0   # nothing to do
 
 
 def test_kernel_choice_is_reported(hip_lib):
