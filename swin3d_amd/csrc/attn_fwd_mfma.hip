@@ -147,13 +147,13 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
     const _Float16 *gtk = static_cast<const _Float16 *>(a.table_k);
     _Float16 *gout = static_cast<_Float16 *>(a.out);
 
-    // work list written by window_items_kernel: inclusive prefix of (query tile, key tile) pairs per
+    // work list written by attn_prepare_kernel: inclusive prefix of (query tile, key tile) pairs per
     // window, then the work counter, the number of head groups and the heads per group
     const int *item_end = static_cast<const int *>(a.items);
     const int groups = __builtin_amdgcn_readfirstlane(item_end[a.W + 1]);
     const int group_heads = __builtin_amdgcn_readfirstlane(item_end[a.W + 2]);
     const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]) * groups;
-    // work items are handed out through a device counter (zeroed by window_items_kernel), so a
+    // work items are handed out through a device counter (zeroed by attn_prepare_kernel), so a
     // wavefront that drew long items simply draws fewer of them
     int *next_item = static_cast<int *>(a.items) + a.W;
 
@@ -494,32 +494,32 @@ __global__ __launch_bounds__(256) void attn_merge_partials_kernel(AttnArgs a)
     if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
 }
 
-// value table [axis][row][h][c] -> [h][c][padded row], every axis padded to a multiple of 16 rows
-__global__ void transpose_value_table_kernel(AttnArgs a)
+// Set-up of one attention launch, one kernel:
+//  * workgroup 0 writes the work list: inclusive prefix sum of the (query tile, key tile) pairs of every
+//    window (W is at most a few hundred thousand), the work counter and the split of the heads into groups;
+//  * the other workgroups transpose the value table [axis][row][h][c] -> [h][c][padded row], every axis
+//    padded to a multiple of 16 rows.
+__global__ __launch_bounds__(1024) void attn_prepare_kernel(AttnArgs a)
 {
-    const int HD = a.H * a.D;
-    _Float16 *dst = static_cast<_Float16 *>(a.workspace);
-    const _Float16 *src = static_cast<const _Float16 *>(a.table_v);
-    const int64_t total = static_cast<int64_t>(HD) * a.padded_rows;
-    for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < total;
-         t += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        const int hc = static_cast<int>(t / a.padded_rows);
-        const int pr = static_cast<int>(t - static_cast<int64_t>(hc) * a.padded_rows);
-        _Float16 val = static_cast<_Float16>(0.0f);
-        for (int n = 0; n < a.nd; ++n) {
-            const int r = pr - a.pbase[n];
-            if (r >= 0 && r < a.rows[n]) val = src[static_cast<int64_t>(a.base[n] + r) * HD + hc];
+    if (blockIdx.x > 0) {
+        const int HD = a.H * a.D;
+        _Float16 *dst = static_cast<_Float16 *>(a.workspace);
+        const _Float16 *src = static_cast<const _Float16 *>(a.table_v);
+        const int64_t total = static_cast<int64_t>(HD) * a.padded_rows;
+        for (int64_t t = static_cast<int64_t>(blockIdx.x - 1) * blockDim.x + threadIdx.x; t < total;
+             t += static_cast<int64_t>(gridDim.x - 1) * blockDim.x) {
+            const int hc = static_cast<int>(t / a.padded_rows);
+            const int pr = static_cast<int>(t - static_cast<int64_t>(hc) * a.padded_rows);
+            _Float16 val = static_cast<_Float16>(0.0f);
+            for (int n = 0; n < a.nd; ++n) {
+                const int r = pr - a.pbase[n];
+                if (r >= 0 && r < a.rows[n]) val = src[static_cast<int64_t>(a.base[n] + r) * HD + hc];
+            }
+            dst[t] = val;
         }
-        dst[t] = val;
+        return;
     }
-}
-
-// Work list of the attention kernel: inclusive prefix sum of the (query tile, key tile) pairs of every
-// window, the work counter and the split of the heads into groups.  One workgroup; W is at most a few
-// hundred thousand.
-__global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
-{
-    __shared__ int part[1024];
+    __shared__ int wave_total[16];
     int *item_end = static_cast<int *>(a.items);
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
@@ -529,15 +529,26 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
         const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
         sum += tiles * tiles;
     }
-    part[threadIdx.x] = sum;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
-        __syncthreads();
-        part[threadIdx.x] += add;
-        __syncthreads();
+    // inclusive scan over the 1024 threads: shuffles inside a wavefront, then the 16 wavefront totals
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = sum;
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
     }
-    int run = part[threadIdx.x] - sum;
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        int v = wave_total[threadIdx.x];
+        for (int off = 1; off < 16; off <<= 1) {
+            const int up = __shfl_up(v, off);
+            if (threadIdx.x >= off) v += up;
+        }
+        wave_total[threadIdx.x] = v;
+    }
+    __syncthreads();
+    incl += wave > 0 ? wave_total[wave - 1] : 0;
+    int run = incl - sum;
     for (int w = begin; w < end; ++w) {
         const int tiles = (a.w_sizes[w] + kTile - 1) / kTile;
         run += tiles * tiles;
@@ -546,7 +557,7 @@ __global__ __launch_bounds__(1024) void window_items_kernel(AttnArgs a)
     if (threadIdx.x == 1023) {
         // heads are split into groups when the tile pairs alone are too few to keep every wavefront
         // of the persistent grid busy with several items (deep stages: few, large windows, many heads)
-        const int pairs = part[1023];
+        const int pairs = incl;
         int groups = pairs > 0 ? (a.target_items + pairs - 1) / pairs : 1;
         groups = max(1, min(groups, a.H));
         const int group_heads = (a.H + groups - 1) / groups;
@@ -572,10 +583,6 @@ int launch(const AttnArgs &args, hipStream_t stream)
     const size_t lds = lds_bytes(a, WaveLds<RMAX>::kWords, TVT_LDS);
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    const int64_t cells = static_cast<int64_t>(a.H) * a.D * a.padded_rows;
-    hipLaunchKernelGGL(transpose_value_table_kernel, dim3(static_cast<unsigned>(ceil_div(cells, 256))),
-                       dim3(256), 0, stream, a);
-    S3D_HIP_CHECK(hipGetLastError());
     // persistent grid: as many workgroups as fit the chip at once (LDS-bound), never more than the
     // windows can feed; wavefronts pull items in a strided loop
     int device = 0, cus = 256;
@@ -586,7 +593,9 @@ int launch(const AttnArgs &args, hipStream_t stream)
     const int per_cu = kLdsPerCu / lds > 0 ? static_cast<int>(kLdsPerCu / lds) : 1;
     int64_t grid = static_cast<int64_t>(cus) * per_cu;
     a.target_items = static_cast<int>(grid) * kWaves * kItemsPerWave;
-    hipLaunchKernelGGL(window_items_kernel, dim3(1), dim3(1024), 0, stream, a);
+    const int64_t cells = static_cast<int64_t>(a.H) * a.D * a.padded_rows;
+    hipLaunchKernelGGL(attn_prepare_kernel, dim3(1 + static_cast<unsigned>(ceil_div(cells, 1024))), dim3(1024), 0,
+                       stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     // never more wavefronts than work items (upper bound: every window as large as the largest,
     // every head an item of its own)
