@@ -171,6 +171,21 @@ def test_strided_qkv_views_are_read_in_place(oracle_lib, hip_lib, dtype):
                                             t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("ws,quant,heads,dim,cRSE", [
+    (3, 4, 4, 8, "XYZ_RGB_NORM"),     # 24 / 32-row axis tables: the 32-row kernel variant
+    (4, 4, 2, 16, "XYZ_RGB"),         # 32-row tables, head_dim 16, six axes
+    (4, 8, 3, 8, "XYZ_RGB_NORM"),     # quant 8: 64-row tables on every axis (576 rows per head)
+    (8, 4, 2, 16, "XYZ"),             # window 8: 64-row tables, windows up to 512 voxels
+])
+def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, heads, dim, cRSE):
+    case = make_attn_case(oracle_lib, seed=40 + ws, n=700, ws=ws, quant=quant, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(8, 8, 3))
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
 def test_empty_input(hip_lib):
     import swin3d_amd
     dev = torch.device("cuda")

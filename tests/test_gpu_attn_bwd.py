@@ -93,6 +93,22 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
     _check(oracle_lib, case, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("ws,quant,heads,dim,cRSE", [
+    (3, 4, 4, 8, "XYZ_RGB_NORM"),     # small tables
+    (4, 8, 3, 8, "XYZ_RGB_NORM"),     # quant 8: 576 table rows per head, nine 64-row register blocks
+    (8, 4, 2, 16, "XYZ"),             # window 8, head_dim 16, three axes
+    (4, 4, 2, 16, "XYZ_RGB"),         # six axes
+])
+def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, heads, dim, cRSE):
+    case = make_attn_case(oracle_lib, seed=70 + ws, n=600, ws=ws, quant=quant, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(8, 8, 3))
+    if dtype == torch.float16:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+    _check(oracle_lib, case, dtype)
+
+
 def test_single_voxel_windows(oracle_lib, hip_lib):
     coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
     case = make_attn_case(oracle_lib, seed=64, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")
