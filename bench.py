@@ -44,11 +44,11 @@ def main():
     ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (1 = force the generic kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-encoder", action="store_true",
-                    help="skip the Swin3D-L encoder end-to-end latency (BASELINE configs[4])")
+                    help="skip the Swin3D-L encoder end-to-end latency")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (windows are independent; see DESIGN.md for how "
-              "the path would shard); --gpus must be 1", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU (windows are independent, so the path would shard over "
+              "windows or scenes without any exchange); --gpus must be 1", file=sys.stderr)
         return 2
 
     import torch
@@ -64,7 +64,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    # ---- workload: BASELINE.json configs[1] -------------------------------------------------
+    # ---- workload: the Swin3D-S stage-1 layer on a 200k-voxel synthetic room ------------------------
     heads, dim, ws, quant, cRSE = 6, 8, 5, 4, "XYZ_RGB_NORM"
     channels = heads * dim
     scene = synth.make_room((10.0, 8.0, 3.0), 30, 200_000, seed=0)
@@ -137,7 +137,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "Swin3D-S stage-1 window attention fwd, synthetic 10x8x3 m room, fp16, "
-                        "C=48 H=6 D=8 window=5 quant=4 cRSE=XYZ_RGB_NORM (BASELINE configs[1])",
+                        "C=48 H=6 D=8 window=5 quant=4 cRSE=XYZ_RGB_NORM (configs[1] of the baseline description)",
             "voxels": n, "windows": num_w, "pairs": num_m,
             "mean_window_voxels": n / max(num_w, 1), "max_window_voxels": index.max_window_voxels,
         },
@@ -251,7 +251,7 @@ def extras_cpu(oracle, synth, scene, ws):
 
 
 def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3):
-    """BASELINE configs[4]: Swin3D-L encoder forward, fp16 attention (fp16_mode 2 under autocast),
+    """Swin3D-L encoder forward, fp16 attention (fp16_mode 2 under autocast),
     random-init weights, a batch of two synthetic rooms of ~300k voxels each; attention, window
     index and KNN on the HIP kernels, the dense layers on torch/hipBLASLt."""
     from swin3d_amd import encoder
