@@ -109,3 +109,60 @@ def test_unet_forward_fp16(hip_lib):
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
         logits = model(vox, signals)
     assert logits.shape == (vox.coords.shape[0], 13) and torch.isfinite(logits).all()
+
+
+def test_window_attention_module_argument_prep(oracle_lib, hip_lib):
+    """WindowAttention (fp32) against a float64 statement of the reference's argument prep
+    (Swin3D/modules/swin3d_layers.py:502-541: q, k, v = split(Linear(feats)), q *= D^-0.5, tables = cat of the
+    flattened (3, rows, H, D) parameters in the order xyz, rgb, norm, signals scaled by quant / 2*quant) fed to
+    the attention oracle, then the output projection.  Forward and the gradients of a linear loss."""
+    from swin3d_amd import crse
+    vox, signals = _inputs(target=2500, batches=1)
+    torch.manual_seed(3)
+    ws, quant, dim, heads = 5, 4, 48, 6
+    attn = encoder.WindowAttention(dim, ws, quant, heads, cRSE="XYZ_RGB_NORM", fp16_mode=0).cuda()
+    for kind in ("query", "key", "value"):
+        for name in ("xyz", "rgb", "norm"):
+            torch.nn.init.normal_(getattr(attn, f"{kind}_{name}_table"), std=0.3)
+    n = vox.coords.shape[0]
+    feats = torch.randn(n, dim, device="cuda", requires_grad=True)
+    local = (signals[:, 1:4].float() - vox.coords[:, 1:].float())
+    args = encoder.get_index01(vox.coords, 1, ws, local, signals[:, 4:].float(), shift=0)
+    out = attn(feats, args)
+    grad_out = torch.randn_like(out)
+    out.backward(grad_out)
+    torch.cuda.synchronize()
+
+    # float64 statement on the host
+    f64 = lambda t: t.detach().double().cpu().numpy()
+    x = f64(feats)
+    qkv = x @ f64(attn.qkv.weight).T + f64(attn.qkv.bias)
+    d = dim // heads
+    q = (qkv[:, :dim] * d ** -0.5).reshape(n, heads, d)
+    k = qkv[:, dim:2 * dim].reshape(n, heads, d)
+    v = qkv[:, 2 * dim:].reshape(n, heads, d)
+    flat = lambda kind: np.concatenate([f64(getattr(attn, f"{kind}_{nm}_table")).reshape(-1) for nm in ("xyz", "rgb", "norm")])
+    sizes = crse.crse_table_sizes(ws, quant, heads, d, "XYZ_RGB_NORM")
+    _, _, _, w_sizes, w2n, n2n, _, n_coords = args
+    scale = np.array([quant] * 3 + [2 * quant] * 6, np.float32)
+    n_crse = (n_coords.cpu().numpy().astype(np.float32) * scale).astype(np.float32)
+    idx = [t.cpu().numpy() for t in (w_sizes, w2n, n2n)]
+    to32 = lambda a: a.astype(np.float32)
+    # the oracle takes fp32 inputs: feed it the fp32 roundings the module itself produces
+    o = oracle_lib.attn_fwd(to32(q), to32(k), to32(v), to32(flat("query")), to32(flat("key")), to32(flat("value")),
+                            sizes, *idx, n_crse)
+    ref = o.reshape(n, dim) @ f64(attn.proj.weight).T + f64(attn.proj.bias)
+    np.testing.assert_allclose(f64(out), ref, rtol=2e-4, atol=2e-5 * np.abs(ref).max())
+
+    # gradients: d out / d attention output = grad_out @ W_proj; the oracle backward gives dq, dk, dv and the tables
+    dattn = (f64(grad_out) @ f64(attn.proj.weight)).reshape(n, heads, d)
+    dq, dk, dv, dtq, dtk, dtv = oracle_lib.attn_bwd(to32(q), to32(k), to32(v), to32(flat("query")), to32(flat("key")),
+                                                    to32(flat("value")), sizes, *idx, n_crse, to32(dattn))
+    dqkv = np.concatenate([dq.reshape(n, dim) * d ** -0.5, dk.reshape(n, dim), dv.reshape(n, dim)], axis=1)
+    ref_dfeats = dqkv @ f64(attn.qkv.weight)
+    np.testing.assert_allclose(f64(feats.grad), ref_dfeats, rtol=1e-3, atol=1e-4 * np.abs(ref_dfeats).max())
+    rows_xyz = sizes[0] // dim
+    got_xyz = f64(attn.key_xyz_table.grad).reshape(-1)
+    np.testing.assert_allclose(got_xyz, dtk[: 3 * rows_xyz * dim], rtol=1e-3, atol=1e-4 * np.abs(dtk).max())
+    got_norm = f64(attn.value_norm_table.grad).reshape(-1)
+    np.testing.assert_allclose(got_norm, dtv[-got_norm.size:], rtol=1e-3, atol=1e-4 * np.abs(dtv).max())
