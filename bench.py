@@ -181,6 +181,7 @@ def main():
                        reps=5, warm=2)
         result["extras"]["attn_bwd"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3),
                                         "vs_forward": ms / kernel_ms, "dtype": "f16 I/O, f32 arithmetic"}
+        result["extras"]["other_shapes"] = other_shapes(torch, swin3d_amd, synth, crse, scene, dev)
 
     if not args.no_extras and not args.no_encoder:
         result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)
@@ -228,6 +229,32 @@ def extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev):
         alg = 12 * ns + 12 * nq + 8 * k * nq
         out[name] = {"ms": ms, "queries_per_s": nq / (ms * 1e-3), "sources": ns, "queries": nq,
                      "algorithmic_bytes": alg, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+    return out
+
+
+def other_shapes(torch, swin3d_amd, synth, crse, scene, dev):
+    """Forward and backward of deeper-stage layers (window 7, all nine cRSE axes) on the same room
+    grid-downsampled once (tensor stride 2): head_dim 16 and a 12-head head_dim 8 layer."""
+    coarse, _ = synth.grid_downsample(scene, 2)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    frac = np.clip((coarse.xyz - coarse.coords[:, 1:]) / np.float32(2), 0, 0.999).astype(np.float32)
+    mode, ws, quant = "XYZ_RGB_NORM", 7, 4
+    index_args = swin3d_amd.get_index01(t(coarse.coords), 2, ws, t(frac), t(synth.signals(coarse, mode)))
+    _, _, _, w_sizes, w2n, n2n, _, n_coords = index_args
+    n_crse = crse.scale_crse_coords(n_coords, quant, mode)
+    n = coarse.coords.shape[0]
+    pairs = int((w_sizes.long() ** 2).sum())
+    out = {"voxels": n, "windows": int(w_sizes.numel()), "pairs": pairs}
+    for heads, dim in ((6, 16), (12, 8)):
+        sizes = crse.crse_table_sizes(ws, quant, heads, dim, mode)
+        q, k, v, tables = synth.layer_inputs(n, heads * dim, heads, int(sum(sizes)), seed=0, dtype=np.float16)
+        a = (t(q), t(k), t(v), *[t(x) for x in tables], sizes, w_sizes, w2n, n2n, n_crse)
+        fwd = _time_gpu(torch, lambda: swin3d_amd.window_attention_forward(*a), reps=10)
+        o, mx, sm = swin3d_amd.window_attention_forward(*a, return_stats=True)
+        dout = torch.randn_like(o)
+        bwd = _time_gpu(torch, lambda: swin3d_amd.window_attention_backward(*a, o, mx, sm, dout), reps=3, warm=1)
+        out[f"H{heads}_D{dim}_window7"] = {"fwd_ms": fwd, "bwd_ms": bwd,
+                                          "fwd_ps_per_pair_head": fwd * 1e9 / (pairs * heads)}
     return out
 
 
