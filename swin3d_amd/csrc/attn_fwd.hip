@@ -61,7 +61,9 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
         padded += (rows + 15) / 16 * 16;
     }
     if (max_window_voxels < 1 || N < 0 || W < 0) return 0;
-    return attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
+    const size_t mfma = attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
+    const size_t generic = attn_generic_workspace_bytes(H, W);
+    return mfma > generic ? mfma : generic;
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
@@ -136,5 +138,10 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         a.max_key_tiles = attn_mfma_key_tiles(max_window_voxels);
         return launch_attn_mfma(a, s);
     }
+    const size_t need = attn_generic_workspace_bytes(H, W);
+    if (!workspace || workspace_bytes < need)
+        return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
+                    workspace ? workspace_bytes : size_t(0), need);
+    a.items = static_cast<char *>(workspace) + align_up(sizeof(int32_t) * static_cast<size_t>(H), 256);
     return launch_attn_generic(a, dtype, s);
 }

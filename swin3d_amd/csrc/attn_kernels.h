@@ -29,7 +29,9 @@ struct AttnArgs {
     int32_t padded_rows;                   // row stride of the transposed value table
 };
 
-// One workgroup per (window, head), tables of the head in LDS, VALU math; any dtype.
+// Persistent workgroups, one head each with its table slices in LDS; lane = query, keys streamed; VALU math,
+// any dtype.  Needs a.workspace (per-head counters) and a.items (chunk prefix) inside the caller's workspace.
+size_t attn_generic_workspace_bytes(int H, int64_t W);
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
