@@ -62,7 +62,7 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
     }
     if (max_window_voxels < 1 || N < 0 || W < 0) return 0;
     const size_t mfma = attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
-    const size_t generic = attn_generic_workspace_bytes(H, W);
+    const size_t generic = attn_generic_workspace_bytes(H, D, W, N, max_window_voxels);
     return mfma > generic ? mfma : generic;
 }
 
@@ -125,10 +125,10 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype);
+    if (max_window_voxels < 1)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: max_window_voxels = %d (an upper bound of w_sizes, >= 1)",
+                    max_window_voxels);
     if (want_mfma) {
-        if (max_window_voxels < 1)
-            return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: max_window_voxels = %d (an upper bound of w_sizes, >= 1)",
-                        max_window_voxels);
         const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
         if (!workspace || workspace_bytes < need)
             return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
@@ -138,10 +138,11 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         a.max_key_tiles = attn_mfma_key_tiles(max_window_voxels);
         return launch_attn_mfma(a, s);
     }
-    const size_t need = attn_generic_workspace_bytes(H, W);
+    const size_t need = attn_generic_workspace_bytes(H, D, W, N, max_window_voxels);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
-    a.items = static_cast<char *>(workspace) + align_up(sizeof(int32_t) * static_cast<size_t>(H), 256);
+    a.partials = attn_generic_partials(workspace, H, W, N, max_window_voxels);
+    a.max_key_tiles = attn_generic_key_blocks(max_window_voxels);
     return launch_attn_generic(a, dtype, s);
 }

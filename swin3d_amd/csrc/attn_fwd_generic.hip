@@ -24,6 +24,13 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWavesPerGroup = kThreads / 64;
 constexpr int kChunk = 64;   // queries per unit = lanes of a wavefront
+constexpr int kKeys = 2;    // streamed keys per loop iteration
+// Work distribution.  Atomics on one cache line retire one after the other (about 12 ns each on this part),
+// so a single counter per head bounds a launch of 50 000 units to 0.6 ms whatever the units cost.  Every head
+// has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues; a wavefront
+// draws from the queue it starts on and moves to the next one when that is empty.
+constexpr int kQueues = 8;
+constexpr int kCounterStride = 64;   // ints between counters (256 bytes)
 
 template <int D> __device__ __forceinline__ void load_row(const float *p, float *dst)
 {
@@ -81,11 +88,15 @@ template <int D> struct Slice<float, D> {
         for (int c = 0; c < D; ++c) acc += x[c] * o.x[c];
         return acc;
     }
-    __device__ __forceinline__ void add_to(float *sum, float) const
+    // acc += p * x
+    __device__ __forceinline__ void fma_to(float *acc, float p) const
     {
 #pragma unroll
-        for (int c = 0; c < D; ++c) sum[c] += x[c];
+        for (int c = 0; c < D; ++c) acc[c] += p * x[c];
     }
+    // fp32 logits: one short partial sum per table row keeps the rounding of the (2*D*ND + D)-term sum at the
+    // level of a tree sum
+    static constexpr bool kChainLogit = false;
 };
 template <int D> struct Slice<__half, D> {
     half2_t x[D / 2];
@@ -100,40 +111,71 @@ template <int D> struct Slice<__half, D> {
         for (int e = 0; e < D / 2; ++e) acc = __builtin_amdgcn_fdot2(x[e], o.x[e], acc, false);
         return acc;
     }
-    // sum += x, widened inside a mixed-precision FMA (x * one + sum, `one` opaque to the optimiser: a plain
-    // add would be a conversion plus an add per element)
-    __device__ __forceinline__ void add_to(float *sum, float one) const
+    // acc += p * x, widened inside a mixed-precision FMA
+    __device__ __forceinline__ void fma_to(float *acc, float p) const
     {
 #pragma unroll
         for (int e = 0; e < D / 2; ++e) {
-            sum[2 * e] = __builtin_fmaf(static_cast<float>(x[e][0]), one, sum[2 * e]);
-            sum[2 * e + 1] = __builtin_fmaf(static_cast<float>(x[e][1]), one, sum[2 * e + 1]);
+            acc[2 * e] = __builtin_fmaf(static_cast<float>(x[e][0]), p, acc[2 * e]);
+            acc[2 * e + 1] = __builtin_fmaf(static_cast<float>(x[e][1]), p, acc[2 * e + 1]);
         }
     }
+    // fp16 I/O: the whole logit is one chain of dot-product accumulations
+    static constexpr bool kChainLogit = true;
 };
 
 // Row of the axis table hit by a pair; fp32 arithmetic in the reference's operation order (subtract, add
-// half the row count, clamp to [0, rows], truncate), with the upper edge folded onto the last row.
-__device__ __forceinline__ int crse_row(float ci, float cj, int rows)
+// half the row count, clamp, truncate).  The reference clamps to [0, rows] and folds the upper edge onto
+// the last row after truncation; clamping to [0, largest float below rows] gives the same row for every
+// input with one median-of-three and no integer minimum.
+__device__ __forceinline__ float crse_upper(int rows)
+{
+    return __int_as_float(__float_as_int(static_cast<float>(rows)) - 1);
+}
+__device__ __forceinline__ int crse_row(float ci, float cj, float half_rows, float upper)
 {
     float rel = ci - cj;
-    rel = rel + static_cast<float>(rows / 2);
-    rel = fminf(fmaxf(rel, 0.0f), static_cast<float>(rows));
-    return min(static_cast<int>(rel), rows - 1);
+    rel = rel + half_rows;
+    return static_cast<int>(__builtin_amdgcn_fmed3f(rel, 0.0f, upper));
 }
 
-// inclusive prefix of ceil(n_w / 64) over the windows (into a.items) and the per-head work counters
-// (at the start of a.workspace); one workgroup
+// key blocks a window of n voxels is split into (units stream at most kChunk keys), and their even size
+__host__ __device__ inline int key_blocks(int n) { return (n + kChunk - 1) / kChunk; }
+__host__ __device__ inline int key_block_size(int n) { const int b = key_blocks(n); return (n + b - 1) / b; }
+
+// byte offsets inside the workspace: the queue counters, the unit count, the unit descriptors, the partial results
+__host__ __device__ inline size_t ws_total_offset(int H) { return sizeof(int32_t) * static_cast<size_t>(H) * kQueues * kCounterStride; }
+__host__ __device__ inline size_t ws_units_offset(int H) { return ws_total_offset(H) + 256; }
+__host__ __device__ inline size_t ws_max_units(int64_t W, int64_t N, int max_blocks)
+{
+    return (static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / kChunk) * max_blocks;
+}
+__host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
+{
+    return ws_units_offset(H) + (sizeof(int2) * ws_max_units(W, N, max_blocks) + 255) / 256 * 256;
+}
+
+// Unit list of the launch, in window order: one descriptor (window, query chunk | key block << 16) per unit,
+// the unit count, and the queue counters at zero; one workgroup.  A unit is 64 queries of a window against
+// one block of at most 64 of its keys: the longest unit bounds the tail of the launch, so windows of more
+// than 64 voxels are split along the keys as well and leave partial results that a second kernel combines.
+// Windows beyond the caller's size bound get no units.
 __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
 {
     __shared__ int wave_total[16];
-    int *unit_end = static_cast<int *>(a.items);
-    int *counters = static_cast<int *>(a.workspace);
+    char *ws = static_cast<char *>(a.workspace);
+    int *counters = reinterpret_cast<int *>(ws);
+    int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
+    int2 *units = reinterpret_cast<int2 *>(ws + ws_units_offset(a.H));
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
     const int begin = threadIdx.x * per, end = min(begin + per, W);
+    auto units_of = [&](int n) {
+        const int blocks = key_blocks(n);
+        return blocks > a.max_key_tiles ? 0 : blocks * blocks;
+    };
     int sum = 0;
-    for (int w = begin; w < end; ++w) sum += (a.w_sizes[w] + kChunk - 1) / kChunk;
+    for (int w = begin; w < end; ++w) sum += units_of(a.w_sizes[w]);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int incl = sum;
     for (int off = 1; off < 64; off <<= 1) {
@@ -153,23 +195,65 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
     __syncthreads();
     int run = incl + (wave > 0 ? wave_total[wave - 1] : 0) - sum;
     for (int w = begin; w < end; ++w) {
-        run += (a.w_sizes[w] + kChunk - 1) / kChunk;
-        unit_end[w] = run;
+        const int n = a.w_sizes[w];
+        const int blocks = key_blocks(n);
+        if (units_of(n) == 0) continue;
+        for (int c = 0; c < blocks; ++c)
+            for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
     }
-    for (int t = threadIdx.x; t < a.H; t += 1024) counters[t] = 0;
+    if (threadIdx.x == 1023) *total = wave_total[15];
+    for (int t = threadIdx.x; t < a.H * kQueues; t += 1024) counters[t * kCounterStride] = 0;
 }
 
-// elements of T between table rows in LDS
+// Windows of more than 64 voxels: combine the per-key-block partial results (unnormalised output, running
+// maximum, sum) of every (voxel, head).  One thread per (sorted position, head), position fastest.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
+{
+    const int H = a.H;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= a.N * H) return;
+    const int h = static_cast<int>(t / a.N), pos = static_cast<int>(t - static_cast<int64_t>(h) * a.N);
+    int lo = 0, hi = static_cast<int>(a.W) - 1;   // last window that starts at or before pos
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (a.w2n[mid] <= pos) lo = mid; else hi = mid - 1;
+    }
+    const int blocks = key_blocks(a.w_sizes[lo]);
+    if (blocks <= 1 || blocks > a.max_key_tiles) return;
+    const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
+    const int64_t block_stride = static_cast<int64_t>(H) * a.N * (D + 2);
+    float m = -INFINITY;
+    for (int kb = 0; kb < blocks; ++kb) m = fmaxf(m, part[kb * block_stride + D]);
+    float l = 0.0f, o[D];
+#pragma unroll
+    for (int c = 0; c < D; ++c) o[c] = 0.0f;
+    for (int kb = 0; kb < blocks; ++kb) {
+        const float *pk = part + kb * block_stride;
+        const float wgt = __expf(pk[D] - m);
+        l += pk[D + 1] * wgt;
+#pragma unroll
+        for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
+    }
+    const int row = a.n2n[pos];
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int c = 0; c < D; ++c) o[c] *= inv;
+    store_row<D>(static_cast<T *>(a.out) + (static_cast<int64_t>(row) * H + h) * D, o);
+    if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
+    if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
+}
+
+// Elements of T between table rows in LDS.  A row holds the head's slices of the three tables back to back
+// (q-side, k-side, v-side: one address per pair and axis); a row length that is a multiple of 32 bytes is
+// padded by 16 bytes so that a wavefront's 16-byte gathers of different rows spread over all bank groups.
 template <typename T, int D> __host__ __device__ constexpr int table_row_stride()
 {
-    return D * sizeof(T) == 16 ? D : D + 16 / static_cast<int>(sizeof(T));
+    return 3 * D + ((3 * D * static_cast<int>(sizeof(T)) / 4) % 8 == 0 ? 16 / static_cast<int>(sizeof(T)) : 0);
 }
 
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
-template <typename T, int D> __host__ __device__ constexpr int groups_per_cu()
-{
-    return (D <= 8 ? 3 : 2) + (sizeof(T) == 2 ? 1 : 0);
-}
+template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() { return sizeof(T) == 4 && D > 8 ? 3 : 4; }
 
 template <typename T, int D, int ND>
 __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sweep_kernel(AttnArgs a)
@@ -178,14 +262,9 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
     const int H = a.H;
     const int HD = H * D;
     const int h = blockIdx.x % H;
-    // table slices of the head in the I/O type; rows longer than 16 bytes are padded by 16 bytes: with a 32- or
-    // 64-byte row stride a wavefront's 16-byte gathers of different rows would fall on 4 or 2 of the eight
-    // 4-bank groups
+    // table slices of the head in the I/O type, interleaved per row
     constexpr int kRowStride = table_row_stride<T, D>();
-    const int cells = a.total_rows * kRowStride;
-    T *tab_q = reinterpret_cast<T *>(smem);
-    T *tab_k = tab_q + cells;
-    T *tab_v = tab_k + cells;
+    T *tab = reinterpret_cast<T *>(smem);
     {
         const T *gq = static_cast<const T *>(a.table_q);
         const T *gk = static_cast<const T *>(a.table_k);
@@ -193,37 +272,53 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
         for (int t = threadIdx.x; t < a.total_rows * D; t += kThreads) {
             const int r = t / D, c = t - r * D;
             const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
-            tab_q[r * kRowStride + c] = gq[g];
-            tab_k[r * kRowStride + c] = gk[g];
-            tab_v[r * kRowStride + c] = gv[g];
+            tab[r * kRowStride + c] = gq[g];
+            tab[r * kRowStride + D + c] = gk[g];
+            tab[r * kRowStride + 2 * D + c] = gv[g];
         }
     }
     __syncthreads();   // the only workgroup barrier
 
     const int lane = threadIdx.x & 63;
-    float one = 1.0f;
-    asm volatile("" : "+v"(one));
     const T *gq = static_cast<const T *>(a.q);
     const T *gk = static_cast<const T *>(a.k);
     const T *gv = static_cast<const T *>(a.v);
-    const int *unit_end = static_cast<const int *>(a.items);
-    const int total_units = __builtin_amdgcn_readfirstlane(unit_end[a.W - 1]);
-    int *counter = static_cast<int *>(a.workspace) + h;
+    const char *ws = static_cast<const char *>(a.workspace);
+    const int2 *units = reinterpret_cast<const int2 *>(ws + ws_units_offset(H));
+    const int total_units = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(ws + ws_total_offset(H)));
+    int *counters = static_cast<int *>(a.workspace) + h * kQueues * kCounterStride;
+    float half_rows[ND], upper[ND];
+    int base_off[ND];
+#pragma unroll
+    for (int n = 0; n < ND; ++n) {
+        half_rows[n] = static_cast<float>(a.rows[n] / 2);
+        upper[n] = crse_upper(a.rows[n]);
+        base_off[n] = a.base[n] * kRowStride;
+    }
 
+    int queue = (blockIdx.x / H) % kQueues;
+    int tried = 0;       // queues found empty so far
+    int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
+    if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
     for (;;) {
-        int unit = 0;
-        if (lane == 0) unit = atomicAdd(counter, 1);
-        unit = __builtin_amdgcn_readfirstlane(unit);
-        if (unit >= total_units) break;
-        int lo = 0, hi = static_cast<int>(a.W) - 1;
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (__builtin_amdgcn_readfirstlane(unit_end[mid]) > unit) hi = mid; else lo = mid + 1;
+        int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        while (unit >= total_units && ++tried < kQueues) {
+            queue = (queue + 1) % kQueues;
+            if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+            unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
         }
-        const int w = lo;
+        if (unit >= total_units) break;
+        if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+        const int2 desc = units[unit];
+        const int w = __builtin_amdgcn_readfirstlane(desc.x);
+        const int chunk = __builtin_amdgcn_readfirstlane(desc.y) & 0xffff;
+        const int kb = __builtin_amdgcn_readfirstlane(desc.y) >> 16;
         const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
-        const int chunk = unit - (w > 0 ? __builtin_amdgcn_readfirstlane(unit_end[w - 1]) : 0);
+        // the unit's keys: block kb of the window's even split into blocks of at most 64
+        const int blocks = key_blocks(n_w);
+        const int k_begin = kb * key_block_size(n_w);
+        const int n_k = min(key_block_size(n_w), n_w - k_begin);
         // a window of at most 32 voxels streams two keys per step (lanes l and l + 32 own the same query)
         const int gs = n_w <= 32 ? 32 : 64;
         const int ng = 64 / gs;
@@ -242,44 +337,69 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
         for (int c = 0; c < D; ++c) acc[c] = 0.0f;
         float m = -INFINITY, l = 0.0f;
 
-        const int steps = (n_w + ng - 1) / ng;
-        int st_row_next = a.n2n[s0 + min(grp, n_w - 1)];
-        for (int it = 0; it < steps; ++it) {
-            const int st = it * ng + grp;
-            const bool st_valid = st < n_w;
-            const int st_pos = s0 + min(st, n_w - 1);
-            const int st_row = st_row_next;
-            if (it + 1 < steps) st_row_next = a.n2n[s0 + min(st + ng, n_w - 1)];
-            Slice<T, D> kv, v_in;
-            float vv[D], cj[ND];
-            kv.load(gk + static_cast<int64_t>(st_row) * a.row_stride + h * D);
-            v_in.load(gv + static_cast<int64_t>(st_row) * a.row_stride + h * D);
+        // kKeys streamed keys per iteration: their loads and dependent chains interleave, which hides the
+        // LDS and cache round trips a single chain would wait out one after the other
+        const int steps = (n_k + ng - 1) / ng;
+        const int k0 = s0 + k_begin;
+        int row_next[kKeys];
 #pragma unroll
-            for (int n = 0; n < ND; ++n) cj[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
+        for (int u = 0; u < kKeys; ++u) row_next[u] = a.n2n[k0 + min(u * ng + grp, n_k - 1)];
+        for (int it = 0; it < steps; it += kKeys) {
+            Slice<T, D> kv[kKeys], v_in[kKeys];
+            float logit[kKeys];
+            int off[kKeys][ND];
+            bool valid[kKeys];
 #pragma unroll
-            for (int c = 0; c < D; ++c) vv[c] = 0.0f;
-            v_in.add_to(vv, one);
-
-            float logit = qv.dot(kv, 0.0f);
+            for (int u = 0; u < kKeys; ++u) {
+                const int st = (it + u) * ng + grp;
+                valid[u] = st < n_k;
+                const int st_pos = k0 + min(st, n_k - 1);
+                const int st_row = row_next[u];
+                row_next[u] = a.n2n[k0 + min(st + kKeys * ng, n_k - 1)];
+                kv[u].load(gk + static_cast<int64_t>(st_row) * a.row_stride + h * D);
+                v_in[u].load(gv + static_cast<int64_t>(st_row) * a.row_stride + h * D);
+                float cj[ND];
 #pragma unroll
-            for (int n = 0; n < ND; ++n) {
-                const int off = (a.base[n] + crse_row(ci[n], cj[n], a.rows[n])) * kRowStride;
-                Slice<T, D> tq_r, tk_r, tv_r;
-                tq_r.load(tab_q + off);
-                tk_r.load(tab_k + off);
-                tv_r.load(tab_v + off);
-                // short partial sums per axis, added to the logit as two terms: keeps the fp32 rounding of the
-                // (up to 2*D*ND + D)-term logit at the level of a tree sum
-                logit += qv.dot(tq_r, 0.0f) + kv.dot(tk_r, 0.0f);
-                tv_r.add_to(vv, one);
+                for (int n = 0; n < ND; ++n) cj[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
+#pragma unroll
+                for (int n = 0; n < ND; ++n)
+                    off[u][n] = base_off[n] + __umul24(crse_row(ci[n], cj[n], half_rows[n], upper[n]), kRowStride);
             }
-            if (st_valid) {
-                const float m_new = fmaxf(m, logit);
-                const float scale = __expf(m - m_new);   // exp(-inf) = 0 on the first key
-                const float p = __expf(logit - m_new);
-                l = l * scale + p;
 #pragma unroll
-                for (int c = 0; c < D; ++c) acc[c] = acc[c] * scale + p * vv[c];
+            for (int u = 0; u < kKeys; ++u) {
+                logit[u] = qv.dot(kv[u], 0.0f);
+#pragma unroll
+                for (int n = 0; n < ND; ++n) {
+                    Slice<T, D> tq_r, tk_r;
+                    tq_r.load(tab + off[u][n]);
+                    tk_r.load(tab + off[u][n] + D);
+                    if (Slice<T, D>::kChainLogit) logit[u] = kv[u].dot(tk_r, qv.dot(tq_r, logit[u]));
+                    else logit[u] += kv[u].dot(tk_r, qv.dot(tq_r, 0.0f));
+                }
+            }
+            if (valid[0]) {   // slot 0 is the lowest key of the iteration
+                float m_new = fmaxf(m, logit[0]);
+#pragma unroll
+                for (int u = 1; u < kKeys; ++u) {
+                    logit[u] = valid[u] ? logit[u] : -INFINITY;
+                    m_new = fmaxf(m_new, logit[u]);
+                }
+                const float scale = __expf(m - m_new);   // exp(-inf) = 0 on the first key
+                l *= scale;
+#pragma unroll
+                for (int c = 0; c < D; ++c) acc[c] *= scale;
+#pragma unroll
+                for (int u = 0; u < kKeys; ++u) {
+                    const float p = __expf(logit[u] - m_new);
+                    l += p;
+                    v_in[u].fma_to(acc, p);
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) {
+                        Slice<T, D> tv_r;
+                        tv_r.load(tab + off[u][n] + 2 * D);
+                        tv_r.fma_to(acc, p);
+                    }
+                }
                 m = m_new;
             }
         }
@@ -295,12 +415,20 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
             m = m_all;
         }
         if (own_valid && grp == 0) {
-            const float inv = 1.0f / l;
+            if (blocks == 1) {
+                const float inv = 1.0f / l;
 #pragma unroll
-            for (int c = 0; c < D; ++c) acc[c] *= inv;
-            store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + h * D, acc);
-            if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h] = m;
-            if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h] = l;
+                for (int c = 0; c < D; ++c) acc[c] *= inv;
+                store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + h * D, acc);
+                if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h] = m;
+                if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h] = l;
+            } else {
+                float *part = a.partials + ((static_cast<int64_t>(kb) * H + h) * a.N + own_pos) * (D + 2);
+#pragma unroll
+                for (int c = 0; c < D; ++c) part[c] = acc[c];
+                part[D] = m;
+                part[D + 1] = l;
+            }
         }
     }
 }
@@ -308,7 +436,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
 template <typename T, int D, int ND>
 int launch_sweep(const AttnArgs &a, hipStream_t stream)
 {
-    const size_t lds = align_up(sizeof(T) * 3 * static_cast<size_t>(a.total_rows) * table_row_stride<T, D>(), 16);
+    const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride<T, D>(), 16);
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
@@ -329,6 +457,12 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
     const int per_head = (per_cu * cus + a.H - 1) / a.H;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_head * a.H)), dim3(kThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
+    if (a.max_key_tiles > 1) {
+        const int64_t threads = a.N * a.H;
+        hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256),
+                           0, stream, a);
+        S3D_HIP_CHECK(hipGetLastError());
+    }
     return S3D_OK;
 }
 
@@ -346,11 +480,21 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream)
 
 }  // namespace
 
-size_t attn_generic_workspace_bytes(int H, int64_t W)
+int attn_generic_key_blocks(int max_window_voxels) { return key_blocks(max_window_voxels > 0 ? max_window_voxels : 1); }
+
+size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels)
 {
-    // per-head work counters, then the prefix of 64-query chunks per window
-    return align_up(sizeof(int32_t) * static_cast<size_t>(H), 256) +
-           align_up(sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1), 256);
+    // queue counters, the unit count, the unit descriptors, and one partial record per (key block, head,
+    // voxel) when some window may be split along its keys
+    const int blocks = attn_generic_key_blocks(max_window_voxels);
+    const size_t partials = blocks <= 1 ? 0 : sizeof(float) * static_cast<size_t>(N) * blocks * H * (D + 2);
+    return ws_partials_offset(H, W, N, blocks) + align_up(partials, 256);
+}
+
+float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels)
+{
+    return reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                     ws_partials_offset(H, W, N, attn_generic_key_blocks(max_window_voxels)));
 }
 
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream)

@@ -16,7 +16,7 @@ struct AttnArgs {
     const float *n_coords;                 // [N,nd], window-sorted
     void *out;                             // [N,H,D]
     float *out_max, *out_sum;              // [N,H] or null
-    void *workspace;                       // transposed value table (MFMA path) or null
+    void *workspace;                       // the caller's workspace
     void *items;                           // int32 [W+1] work-item prefix + counter (MFMA path)
     float *partials;                       // per-key-tile partial results of multi-tile windows
     int32_t max_key_tiles;                 // key tiles of the largest window (stride of `partials`)
@@ -30,8 +30,10 @@ struct AttnArgs {
 };
 
 // Persistent workgroups, one head each with its table slices in LDS; lane = query, keys streamed; VALU math,
-// any dtype.  Needs a.workspace (per-head counters) and a.items (chunk prefix) inside the caller's workspace.
-size_t attn_generic_workspace_bytes(int H, int64_t W);
+// any dtype.  Needs a.workspace (work queues, unit list), a.partials and a.max_key_tiles (key blocks of 64).
+int attn_generic_key_blocks(int max_window_voxels);
+size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels);
+float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels);
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
