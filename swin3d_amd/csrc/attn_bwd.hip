@@ -31,6 +31,11 @@ namespace {
 constexpr int kBwdThreads = 256;
 constexpr int kBwdWaves = kBwdThreads / 64;
 constexpr int kChunk = 64;            // owned elements per unit = lanes of a wavefront
+// Work distribution: atomics on one cache line retire one after the other (about 12 ns each on this part), so
+// every head has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues and a
+// wavefront moves to the next queue when the one it draws from is empty.
+constexpr int kQueues = 8;
+constexpr int kCounterStride = 64;    // ints between counters (256 bytes)
 constexpr float kFixP = 16777216.0f;  // 2^24: softmax weights of one query sum to at most 1
 constexpr float kFixL = 8388608.0f;   // 2^23: |dL| / max|dL| <= 1, at most 64 lanes meet in one bin
 
@@ -42,7 +47,7 @@ struct BwdArgs {
     void *dq, *dk, *dv;
     float *dtq, *dtk, *dtv;
     float *delta;     // [N,H] dout_i . o_i
-    int32_t *units;   // [W] inclusive prefix of 64-element chunks per window, then H work counters
+    int32_t *units;   // H * kQueues work counters (kCounterStride apart), the unit count, (window, chunk) per unit
     int32_t H, D, nd, total_rows;
     int64_t N, W, table_len;
     int32_t rows[kMaxAxes];
@@ -129,10 +134,14 @@ __global__ void bwd_prepare_kernel(BwdArgs a)
         a.dtk[t] = 0.0f;
         a.dtv[t] = 0.0f;
     }
-    for (int64_t t = t0; t < a.H; t += stride) a.units[a.W + t] = 0;
+    for (int64_t t = t0; t < a.H * kQueues; t += stride) a.units[t * kCounterStride] = 0;
 }
 
-// inclusive prefix of ceil(n_w / 64) over the windows; one workgroup
+__host__ __device__ inline size_t units_total_index(int H) { return static_cast<size_t>(H) * kQueues * kCounterStride; }
+__host__ __device__ inline size_t units_list_index(int H) { return units_total_index(H) + 64; }
+
+// unit list in window order: one (window, chunk of 64 owned elements) descriptor per unit, and the unit count;
+// one workgroup
 __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
 {
     __shared__ int part[1024];
@@ -150,16 +159,19 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
         __syncthreads();
     }
     int run = part[threadIdx.x] - sum;
+    int2 *list = reinterpret_cast<int2 *>(a.units + units_list_index(a.H));
     for (int w = begin; w < end; ++w) {
-        run += (a.w_sizes[w] + kChunk - 1) / kChunk;
-        a.units[w] = run;
+        const int chunks = (a.w_sizes[w] + kChunk - 1) / kChunk;
+        for (int c = 0; c < chunks; ++c) list[run + c] = make_int2(w, c);
+        run += chunks;
     }
+    if (threadIdx.x == 1023) a.units[units_total_index(a.H)] = part[1023];
 }
 
 // the work counters are re-armed between sweeps
 __global__ void bwd_reset_counters_kernel(BwdArgs a)
 {
-    for (int t = threadIdx.x; t < a.H; t += blockDim.x) a.units[a.W + t] = 0;
+    for (int t = threadIdx.x; t < a.H * kQueues; t += blockDim.x) a.units[t * kCounterStride] = 0;
 }
 
 // MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv (head_dim 8); 1 = dk, dTq; 2 = dv, dTv (head_dim 16:
@@ -221,24 +233,28 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 #pragma unroll
         for (int c = 0; c < D; ++c) acc_a[m][c] = acc_b[m][c] = 0.0f;
 
-    const int *unit_end = a.units;
-    const int total_units = __builtin_amdgcn_readfirstlane(unit_end[a.W - 1]);
-    int *counter = a.units + a.W + h;
+    const int2 *unit_list = reinterpret_cast<const int2 *>(a.units + units_list_index(H));
+    const int total_units = __builtin_amdgcn_readfirstlane(a.units[units_total_index(H)]);
+    int *counters = a.units + h * kQueues * kCounterStride;
 
+    int queue = (blockIdx.x / H) % kQueues;
+    int tried = 0;       // queues found empty so far
+    int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
+    if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
     for (;;) {
-        int unit = 0;
-        if (lane == 0) unit = atomicAdd(counter, 1);
-        unit = __builtin_amdgcn_readfirstlane(unit);
-        if (unit >= total_units) break;
-        int lo = 0, hi = static_cast<int>(a.W) - 1;
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (__builtin_amdgcn_readfirstlane(unit_end[mid]) > unit) hi = mid; else lo = mid + 1;
+        int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        while (unit >= total_units && ++tried < kQueues) {
+            queue = (queue + 1) % kQueues;
+            if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+            unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
         }
-        const int w = lo;
+        if (unit >= total_units) break;
+        if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+        const int2 desc = unit_list[unit];
+        const int w = __builtin_amdgcn_readfirstlane(desc.x);
+        const int chunk = __builtin_amdgcn_readfirstlane(desc.y);
         const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
-        const int chunk = unit - (w > 0 ? __builtin_amdgcn_readfirstlane(unit_end[w - 1]) : 0);
         // group size: a window of at most 32 voxels streams two elements per step
         const int gs = n_w <= 32 ? 32 : 64;
         const int ng = 64 / gs;
@@ -523,9 +539,10 @@ int fill_bwd_axes(BwdArgs &a, const int32_t *table_sizes, int nd, int64_t table_
     return S3D_OK;
 }
 
-size_t bwd_units_bytes(int64_t W, int H)
+size_t bwd_units_bytes(int64_t W, int64_t N, int H)
 {
-    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(H)), 256);
+    const size_t max_units = static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / kChunk;
+    return align_up(sizeof(int32_t) * (units_list_index(H) + 2 * max_units), 256);
 }
 
 }  // namespace
@@ -536,7 +553,7 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_
 {
     using namespace s3d;
     if (H < 1 || N < 0 || W < 0) return 0;
-    return bwd_units_bytes(W, H) + align_up(sizeof(float) * static_cast<size_t>(N) * H, 256);
+    return bwd_units_bytes(W, N, H) + align_up(sizeof(float) * static_cast<size_t>(N) * H, 256);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
@@ -584,7 +601,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
     a.units = static_cast<int32_t *>(workspace);
-    a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, H));
+    a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (N == 0 || W == 0) {
         // nothing to differentiate: the table gradients are zero

@@ -24,7 +24,6 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWavesPerGroup = kThreads / 64;
 constexpr int kChunk = 64;   // queries per unit = lanes of a wavefront
-constexpr int kKeys = 2;    // streamed keys per loop iteration
 // Work distribution.  Atomics on one cache line retire one after the other (about 12 ns each on this part),
 // so a single counter per head bounds a launch of 50 000 units to 0.6 ms whatever the units cost.  Every head
 // has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues; a wavefront
@@ -155,14 +154,15 @@ __host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N
     return ws_units_offset(H) + (sizeof(int2) * ws_max_units(W, N, max_blocks) + 255) / 256 * 256;
 }
 
-// Unit list of the launch, in window order: one descriptor (window, query chunk | key block << 16) per unit,
-// the unit count, and the queue counters at zero; one workgroup.  A unit is 64 queries of a window against
-// one block of at most 64 of its keys: the longest unit bounds the tail of the launch, so windows of more
-// than 64 voxels are split along the keys as well and leave partial results that a second kernel combines.
-// Windows beyond the caller's size bound get no units.
+// Unit list of the launch: one descriptor (window, query chunk | key block << 16) per unit, the unit count,
+// and the queue counters at zero; one workgroup.  A unit is 64 queries of a window against one block of at
+// most 64 of its keys: the longest unit bounds the tail of the launch, so windows of more than 64 voxels are
+// split along the keys as well and leave partial results that a second kernel combines.  Units of windows
+// with more than 32 voxels (33 to 64 steps) come first, then the short ones (at most 16 steps), each class in
+// window order: the launch ends on short units.  Windows beyond the caller's size bound get no units.
 __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
 {
-    __shared__ int wave_total[16];
+    __shared__ int wave_long[16], wave_all[16];
     char *ws = static_cast<char *>(a.workspace);
     int *counters = reinterpret_cast<int *>(ws);
     int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
@@ -174,34 +174,44 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
         const int blocks = key_blocks(n);
         return blocks > a.max_key_tiles ? 0 : blocks * blocks;
     };
-    int sum = 0;
-    for (int w = begin; w < end; ++w) sum += units_of(a.w_sizes[w]);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int incl = sum;
-    for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
+    int sum_long = 0, sum_all = 0;
+    for (int w = begin; w < end; ++w) {
+        const int n = a.w_sizes[w];
+        sum_all += units_of(n);
+        if (n > 32) sum_long += units_of(n);
     }
-    if (lane == 63) wave_total[wave] = incl;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl_long = sum_long, incl_all = sum_all;
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up_long = __shfl_up(incl_long, off), up_all = __shfl_up(incl_all, off);
+        if (lane >= off) { incl_long += up_long; incl_all += up_all; }
+    }
+    if (lane == 63) { wave_long[wave] = incl_long; wave_all[wave] = incl_all; }
     __syncthreads();
     if (threadIdx.x < 16) {
-        int v = wave_total[threadIdx.x];
+        int v_long = wave_long[threadIdx.x], v_all = wave_all[threadIdx.x];
         for (int off = 1; off < 16; off <<= 1) {
-            const int up = __shfl_up(v, off);
-            if (threadIdx.x >= off) v += up;
+            const int up_long = __shfl_up(v_long, off), up_all = __shfl_up(v_all, off);
+            if (threadIdx.x >= off) { v_long += up_long; v_all += up_all; }
         }
-        wave_total[threadIdx.x] = v;
+        wave_long[threadIdx.x] = v_long;
+        wave_all[threadIdx.x] = v_all;
     }
     __syncthreads();
-    int run = incl + (wave > 0 ? wave_total[wave - 1] : 0) - sum;
+    const int total_long = wave_long[15];
+    const int before_long = incl_long + (wave > 0 ? wave_long[wave - 1] : 0) - sum_long;
+    const int before_all = incl_all + (wave > 0 ? wave_all[wave - 1] : 0) - sum_all;
+    int run_long = before_long;
+    int run_short = total_long + (before_all - before_long);
     for (int w = begin; w < end; ++w) {
         const int n = a.w_sizes[w];
         const int blocks = key_blocks(n);
         if (units_of(n) == 0) continue;
+        int &run = n > 32 ? run_long : run_short;
         for (int c = 0; c < blocks; ++c)
             for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
     }
-    if (threadIdx.x == 1023) *total = wave_total[15];
+    if (threadIdx.x == 1023) *total = wave_all[15];
     for (int t = threadIdx.x; t < a.H * kQueues; t += 1024) counters[t * kCounterStride] = 0;
 }
 
@@ -258,6 +268,9 @@ template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() {
 template <typename T, int D, int ND>
 __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sweep_kernel(AttnArgs a)
 {
+    // streamed keys per loop iteration: at head_dim 16 two interleaved chains hide the LDS round trips,
+    // at head_dim 8 the extra registers cost more than they bring
+    constexpr int kKeys = D <= 8 ? 1 : 2;
     extern __shared__ float smem[];
     const int H = a.H;
     const int HD = H * D;
