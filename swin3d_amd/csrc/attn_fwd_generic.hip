@@ -74,6 +74,25 @@ __device__ __forceinline__ float to_float(__half x) { return __half2float(x); }
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
+// 16-byte LDS reads at a 32-bit LDS address (pointer arithmetic on generic pointers is 64-bit, which costs a
+// 64-bit multiply-add per gathered row)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const u32x4_t lds_uint4_t;
+typedef __attribute__((address_space(3))) const f32x4_t lds_float4_t;
+// a * b + c with 24-bit factors: one full-rate instruction (the compiler's choice for a 32-bit multiply-add,
+// v_mad_u64_u32, issues at a quarter of the rate)
+__device__ __forceinline__ uint32_t mad_u24(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t d;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(c));
+    return d;
+}
+__device__ __forceinline__ uint32_t lds_address(const void *p)
+{
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p));   // low half of a flat LDS address
+}
+
 // One (row, head) slice of D channels in registers.  fp32: D floats, products by FMA.  fp16: D/2 packed pairs
 // kept as loaded; dot products with v_dot2_f32_f16 (exact fp16 products, fp32 accumulation), widening only
 // where a sum of rows is needed.
@@ -81,6 +100,14 @@ template <typename T, int D> struct Slice;
 template <int D> struct Slice<float, D> {
     float x[D];
     __device__ __forceinline__ void load(const float *p) { load_row<D>(p, x); }
+    __device__ __forceinline__ void load_lds(uint32_t addr)
+    {
+#pragma unroll
+        for (int c = 0; c < D; c += 4) {
+            const f32x4_t v = *(lds_float4_t *)(addr + 4 * c);
+            x[c] = v[0]; x[c + 1] = v[1]; x[c + 2] = v[2]; x[c + 3] = v[3];
+        }
+    }
     __device__ __forceinline__ float dot(const Slice &o, float acc) const
     {
 #pragma unroll
@@ -103,6 +130,11 @@ template <int D> struct Slice<__half, D> {
     {
 #pragma unroll
         for (int c = 0; c < D; c += 8) *reinterpret_cast<uint4 *>(&x[c / 2]) = *reinterpret_cast<const uint4 *>(p + c);
+    }
+    __device__ __forceinline__ void load_lds(uint32_t addr)
+    {
+#pragma unroll
+        for (int c = 0; c < D; c += 8) *reinterpret_cast<u32x4_t *>(&x[c / 2]) = *(lds_uint4_t *)(addr + 2 * c);
     }
     __device__ __forceinline__ float dot(const Slice &o, float acc) const
     {
@@ -300,13 +332,17 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
     const int2 *units = reinterpret_cast<const int2 *>(ws + ws_units_offset(H));
     const int total_units = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(ws + ws_total_offset(H)));
     int *counters = static_cast<int *>(a.workspace) + h * kQueues * kCounterStride;
+    constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
+    const uint32_t tab_addr = __builtin_amdgcn_readfirstlane(lds_address(tab));
+    const uint32_t row_bytes = kRowBytes;
     float half_rows[ND], upper[ND];
-    int base_off[ND];
+    uint32_t base_off[ND];
 #pragma unroll
     for (int n = 0; n < ND; ++n) {
         half_rows[n] = static_cast<float>(a.rows[n] / 2);
         upper[n] = crse_upper(a.rows[n]);
-        base_off[n] = a.base[n] * kRowStride;
+        // LDS byte address of the axis table's first row
+        base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + a.base[n] * kRowBytes);
     }
 
     int queue = (blockIdx.x / H) % kQueues;
@@ -360,7 +396,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
         for (int it = 0; it < steps; it += kKeys) {
             Slice<T, D> kv[kKeys], v_in[kKeys];
             float logit[kKeys];
-            int off[kKeys][ND];
+            uint32_t off[kKeys][ND];
             bool valid[kKeys];
 #pragma unroll
             for (int u = 0; u < kKeys; ++u) {
@@ -376,7 +412,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
                 for (int n = 0; n < ND; ++n) cj[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
 #pragma unroll
                 for (int n = 0; n < ND; ++n)
-                    off[u][n] = base_off[n] + __umul24(crse_row(ci[n], cj[n], half_rows[n], upper[n]), kRowStride);
+                    off[u][n] = mad_u24(static_cast<uint32_t>(crse_row(ci[n], cj[n], half_rows[n], upper[n])), row_bytes, base_off[n]);
             }
 #pragma unroll
             for (int u = 0; u < kKeys; ++u) {
@@ -384,8 +420,8 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
 #pragma unroll
                 for (int n = 0; n < ND; ++n) {
                     Slice<T, D> tq_r, tk_r;
-                    tq_r.load(tab + off[u][n]);
-                    tk_r.load(tab + off[u][n] + D);
+                    tq_r.load_lds(off[u][n]);
+                    tk_r.load_lds(off[u][n] + D * sizeof(T));
                     if (Slice<T, D>::kChainLogit) logit[u] = kv[u].dot(tk_r, qv.dot(tq_r, logit[u]));
                     else logit[u] += kv[u].dot(tk_r, qv.dot(tq_r, 0.0f));
                 }
@@ -409,7 +445,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
 #pragma unroll
                     for (int n = 0; n < ND; ++n) {
                         Slice<T, D> tv_r;
-                        tv_r.load(tab + off[u][n] + 2 * D);
+                        tv_r.load_lds(off[u][n] + 2 * D * sizeof(T));
                         tv_r.fma_to(acc, p);
                     }
                 }
