@@ -41,7 +41,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (1 = force the generic kernel)")
+    ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (0 = the library picks, 1 = sweep kernel, 2 = MFMA kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-encoder", action="store_true",
                     help="skip the Swin3D-L encoder end-to-end latency")

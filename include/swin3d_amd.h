@@ -83,7 +83,8 @@ const char *s3d_last_error_string(void);
  *                  of 8 that is >= H*D: with 3*H*D and q, k, v pointing H*D apart the kernels read the
  *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
  *                  place, without the reference's reshape / permute / contiguous copy.
- *   flags          0, or S3D_ATTN_FORCE_GENERIC to run the VALU kernel for every case
+ *   flags          0 (the library picks the kernel), S3D_ATTN_FORCE_GENERIC to run the VALU sweep kernel
+ *                  for every case, or S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies
  *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
  *                  (MFMA kernel: a transposed copy of the value table, the work list, and
  *                  N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
@@ -100,8 +101,9 @@ const char *s3d_last_error_string(void);
  * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.
  */
 #define S3D_ATTN_FORCE_GENERIC 1
-/* 1 if s3d_attn_fwd runs these shapes on the MFMA kernel (fp16, every axis table <= 64 rows),
- * 0 if on the generic VALU kernel.  No counterpart in the reference (it has one kernel). */
+#define S3D_ATTN_FORCE_MFMA 2
+/* 1 if s3d_attn_fwd with flags 0 runs these shapes on the MFMA kernel (fp16, head_dim 16, every axis
+ * table <= 64 rows), 0 if on the VALU sweep kernel.  No counterpart in the reference (it has one kernel). */
 int s3d_attn_fwd_uses_mfma(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype);
 size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,
                                     int64_t N, int64_t W, int32_t max_window_voxels);

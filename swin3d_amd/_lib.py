@@ -13,6 +13,7 @@ S3D_DTYPE_F32 = 0
 S3D_DTYPE_F16 = 1
 KNN_KMAX = 64
 S3D_ATTN_FORCE_GENERIC = 1
+S3D_ATTN_FORCE_MFMA = 2
 
 _lib = None
 

@@ -78,7 +78,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
     int64_t total = 0;
     for (int n = 0; n < nd; ++n) total += table_sizes[n];
     if (fill_axes(a, table_sizes, nd, total) != S3D_OK) return 0;
-    return attn_mfma_supported(a, dtype) ? 1 : 0;
+    return attn_mfma_supported(a, dtype) && attn_mfma_preferred(a) ? 1 : 0;
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
@@ -124,7 +124,8 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.out_sum = out_sum;
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype);
+    const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype) &&
+                           (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
     if (max_window_voxels < 1)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: max_window_voxels = %d (an upper bound of w_sizes, >= 1)",
                     max_window_voxels);

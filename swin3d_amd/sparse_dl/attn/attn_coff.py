@@ -98,7 +98,8 @@ def _host_table_sizes(table_sizes):
 
 
 def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
-                             n_coords, return_stats=False, force_generic=False, max_window_voxels=None):
+                             n_coords, return_stats=False, force_generic=False, max_window_voxels=None,
+                             force_mfma=False):
     """softmax-normalised window attention, [N,H,D] in the dtype of q.
 
     q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5); dense, or views with
@@ -109,7 +110,9 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     n2n            [N] window-sorted position -> row of q/k/v
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
-    force_generic  run the VALU kernel even where the MFMA kernel applies (fp16)
+    force_generic  run the VALU sweep kernel for every case
+    force_mfma     run the MFMA kernel wherever it applies (fp16, axis tables of at most 64 rows); by default
+                   it serves head_dim 16 only
     max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
                    (set by build_window_index) or, failing that, read back from the device
     """
@@ -179,7 +182,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
             n, h, d, w_sizes.numel(), max_window_voxels, row_stride, _DTYPE_CODE[q.dtype],
-            _lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0, workspace.data_ptr(),
+            (_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |
+            (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0), workspace.data_ptr(),
             ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
     if return_stats:

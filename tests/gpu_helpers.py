@@ -6,7 +6,7 @@ import torch
 import swin3d_amd
 
 
-def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", force_generic=False):
+def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", force_generic=False, force_mfma=False):
     """-> numpy float64 output [N,H,D] of swin3d_amd.window_attention_forward."""
     dev = torch.device(device)
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
@@ -15,7 +15,7 @@ def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", 
         t(case.q).to(dtype), t(case.k).to(dtype), t(case.v).to(dtype),
         t(case.tq).to(dtype), t(case.tk).to(dtype), t(case.tv).to(dtype),
         t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
-        return_stats=return_stats, force_generic=force_generic)
+        return_stats=return_stats, force_generic=force_generic, force_mfma=force_mfma)
     torch.cuda.synchronize()
     if return_stats:
         return tuple(r.double().cpu().numpy() for r in res)

@@ -17,8 +17,9 @@ def _check(oracle_lib, case, dtype):
     got = run_attention(case, dtype)
     assert_attn_close(got, ref, dtype)
     if dtype == torch.float16:
-        # fp16 runs on the MFMA kernel by default; the generic kernel must agree with the oracle too
+        # fp16: the library picks the sweep or the MFMA kernel by head_dim; both must agree with the oracle
         assert_attn_close(run_attention(case, dtype, force_generic=True), ref, dtype)
+        assert_attn_close(run_attention(case, dtype, force_mfma=True), ref, dtype)
     return got, ref
 
 
@@ -114,9 +115,11 @@ def test_stats_outputs(oracle_lib, hip_lib):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
-def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib):
-    """max_window_voxels below the real maximum: windows beyond the bound are left out (their output
-    rows keep what the buffer held), every other window is complete, nothing is written out of bounds."""
+@pytest.mark.parametrize("kernel", ["sweep", "mfma"])
+def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib, kernel):
+    """max_window_voxels below the real maximum: windows beyond the bound (rounded up to the kernel's key
+    block: 64 voxels for the sweep kernel, 32 for the MFMA kernel) are left out (their output rows keep what
+    the buffer held), every other window is complete, nothing is written out of bounds."""
     import swin3d_amd
     case = make_attn_case(oracle_lib, seed=38, n=1000, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
     to_half_and_back(_sharp16(case))
@@ -129,7 +132,8 @@ def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib):
     i = case.index
     got = swin3d_amd.window_attention_forward(
         h(case.q), h(case.k), h(case.v), h(case.tq), h(case.tk), h(case.tv), t(case.table_sizes),
-        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32)
+        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32,
+        force_generic=kernel == "sweep", force_mfma=kernel == "mfma")
     torch.cuda.synchronize()
     got = got.double().cpu().numpy()
     small = np.repeat(w_sizes <= 32, w_sizes)           # per sorted position
@@ -156,10 +160,10 @@ def test_strided_qkv_views_are_read_in_place(oracle_lib, hip_lib, dtype):
     assert not q.is_contiguous() and q.stride(0) == 3 * h * d
     i = case.index
     f = lambda a: t(a).to(dtype)
-    for force_generic in (False, True):
+    for force_generic, force_mfma in ((False, False), (True, False), (False, True)):
         got = swin3d_amd.window_attention_forward(q, k, v, f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
                                                   t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
-                                                  force_generic=force_generic)
+                                                  force_generic=force_generic, force_mfma=force_mfma)
         torch.cuda.synchronize()
         assert got.is_contiguous() and got.shape == (n, h, d)
         assert_attn_close(got.double().cpu().numpy(), ref, dtype)
