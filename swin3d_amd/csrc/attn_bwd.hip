@@ -34,8 +34,18 @@ constexpr int kChunk = 64;            // owned elements per unit = lanes of a wa
 // Work distribution: atomics on one cache line retire one after the other (about 12 ns each on this part), so
 // every head has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues and a
 // wavefront moves to the next queue when the one it draws from is empty.
+// The chip has eight XCDs with an L2 each: a wavefront starts on the queue of the XCD it runs on, so all heads
+// of a unit are served from the same XCD and the unit's rows reach that L2 once.
 constexpr int kQueues = 8;
 constexpr int kCounterStride = 64;    // ints between counters (256 bytes)
+
+// id of the XCD (accelerator complex die) the wavefront runs on
+__device__ __forceinline__ int xcd_id()
+{
+    int id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(id));
+    return id;
+}
 constexpr float kFixP = 16777216.0f;  // 2^24: softmax weights of one query sum to at most 1
 constexpr float kFixL = 8388608.0f;   // 2^23: |dL| / max|dL| <= 1, at most 64 lanes meet in one bin
 
@@ -192,7 +202,8 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     extern __shared__ float smem[];
     const int H = a.H;
     const int HD = H * D;
-    const int h = blockIdx.x % H;
+    // workgroups go to the XCDs in turn: consecutive runs of eight serve one head, so every XCD gets every head
+    const int h = (blockIdx.x / kQueues) % H;
     // fp32 table slices of the head, rows padded by 16 bytes: with a 32- or 64-byte row stride a wavefront's
     // 16-byte gathers of different rows would fall on 4 or 2 of the eight 4-bank groups
     constexpr int kRowStride = D + 4;
@@ -237,7 +248,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int total_units = __builtin_amdgcn_readfirstlane(a.units[units_total_index(H)]);
     int *counters = a.units + h * kQueues * kCounterStride;
 
-    int queue = (blockIdx.x / H) % kQueues;
+    int queue = xcd_id() % kQueues;
     int tried = 0;       // queues found empty so far
     int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
     if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
@@ -501,9 +512,9 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
     }
-    // a workgroup serves one head for its whole life: a multiple of H workgroups, about two per CU
-    const int per_head = (2 * cus + a.H - 1) / a.H;
-    const int grid = per_head * a.H;
+    // a workgroup serves one head for its whole life: whole sets of (XCDs x heads), about two workgroups per CU
+    const int set = kQueues * a.H;
+    const int grid = (2 * cus / set > 0 ? 2 * cus / set : 1) * set;
     if constexpr (D <= 8) {
         // one key-owned sweep when both sets of table-gradient registers fit two wavefronts per SIMD
         if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;

@@ -28,8 +28,18 @@ constexpr int kChunk = 64;   // queries per unit = lanes of a wavefront
 // so a single counter per head bounds a launch of 50 000 units to 0.6 ms whatever the units cost.  Every head
 // has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues; a wavefront
 // draws from the queue it starts on and moves to the next one when that is empty.
+// The chip has eight XCDs with an L2 each: a wavefront starts on the queue of the XCD it runs on, so all heads
+// of a unit are served from the same XCD and the unit's q, k, v rows and coordinates reach that L2 once.
 constexpr int kQueues = 8;
 constexpr int kCounterStride = 64;   // ints between counters (256 bytes)
+
+// id of the XCD (accelerator complex die) the wavefront runs on
+__device__ __forceinline__ int xcd_id()
+{
+    int id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(id));
+    return id;
+}
 
 template <int D> __device__ __forceinline__ void load_row(const float *p, float *dst)
 {
@@ -306,7 +316,8 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
     extern __shared__ float smem[];
     const int H = a.H;
     const int HD = H * D;
-    const int h = blockIdx.x % H;
+    // workgroups go to the XCDs in turn: consecutive runs of eight serve one head, so every XCD gets every head
+    const int h = (blockIdx.x / kQueues) % H;
     // table slices of the head in the I/O type, interleaved per row
     constexpr int kRowStride = table_row_stride<T, D>();
     T *tab = reinterpret_cast<T *>(smem);
@@ -345,7 +356,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
         base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + a.base[n] * kRowBytes);
     }
 
-    int queue = (blockIdx.x / H) % kQueues;
+    int queue = xcd_id() % kQueues;
     int tried = 0;       // queues found empty so far
     int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
     if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
@@ -503,8 +514,10 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
     // registers and LDS allow
     int per_cu = groups_per_cu<T, D>();
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
-    const int per_head = (per_cu * cus + a.H - 1) / a.H;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_head * a.H)), dim3(kThreads), lds, stream, a);
+    // as many as fit the chip at once in whole sets of (XCDs x heads)
+    const int set = kQueues * a.H;
+    const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     if (a.max_key_tiles > 1) {
         const int64_t threads = a.N * a.H;
