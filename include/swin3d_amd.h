@@ -76,19 +76,23 @@ const char *s3d_last_error_string(void);
  *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
  *   max_window_voxels  an upper bound of every w_sizes entry (e.g. counts[2] of s3d_window_index, or
- *                  window^3).  It sizes the per-key-tile partial results of windows with more than 32
- *                  voxels; a window larger than the bound is skipped (its output rows are not
- *                  written), so the bound must hold for a complete result.
+ *                  window^3), >= 1.  It sizes the partial results of windows that are split along their
+ *                  keys (blocks of 64 voxels in the sweep kernel, 32 in the MFMA kernel); a window with
+ *                  more key blocks than the bound allows is skipped (its output rows are not written),
+ *                  so the bound must hold for a complete result.
  *   qkv_row_stride elements between consecutive voxel rows of q, k and v (0 = H*D, dense).  A multiple
  *                  of 8 that is >= H*D: with 3*H*D and q, k, v pointing H*D apart the kernels read the
  *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
  *                  place, without the reference's reshape / permute / contiguous copy.
  *   flags          0 (the library picks the kernel), S3D_ATTN_FORCE_GENERIC to run the VALU sweep kernel
  *                  for every case, or S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies
- *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes
- *                  (MFMA kernel: a transposed copy of the value table, the work list, and
- *                  N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
- *                  max_window_voxels > 32)
+ *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes: work-queue
+ *                  counters, the unit list, and N * ceil(max_window_voxels / 64) * H * (D + 2) floats of
+ *                  partial results when max_window_voxels > 64 (sweep kernel); a transposed copy of the
+ *                  value table, the work list and N * ceil(max_window_voxels / 32) * H * (D + 2) floats
+ *                  when max_window_voxels > 32 (MFMA kernel)
+ *   w2n must be ascending (the exclusive prefix sum of w_sizes, as the reference builds it:
+ *   Swin3D/modules/swin3d_layers.py:100-103).
  *   D in {8,16}, nd in {3,6,9}, H >= 1.
  *
  * Row index of axis n for the pair (query i, key j), all in fp32:

@@ -1,12 +1,14 @@
-// Sparse-voxel windowed self-attention forward with cRSE tables (gfx950): generic kernel.
+// Sparse-voxel windowed self-attention forward with cRSE tables (gfx950): sweep kernel.
 //
-// Covers every dtype / shape the library accepts with fp32 arithmetic on the vector ALU (the MFMA kernel
-// takes the fp16 cases).  A workgroup serves one head for its whole life and keeps that head's slices of
-// the three relative-signal tables in LDS (loaded once, not once per window).  A wavefront draws units from
-// a per-head queue; a unit is one window and one chunk of 64 of its queries.  Lane = query: q_i, the running
-// maximum, sum and output stay in the lane's registers while the window's keys stream through the
-// wavefront one per step (two per step, in two 32-lane groups, when the window has at most 32 voxels), so
-// there is no cross-lane reduction, no atomic and no O(pairs) index array; the result is deterministic.
+// Covers every dtype / shape the library accepts on the vector ALU (fp32 arithmetic; fp16 inputs enter through
+// packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one head for its
+// whole life and keeps that head's slices of the three relative-signal tables in LDS (loaded once, not once per
+// window).  A wavefront draws units from the head's work queues; a unit is 64 queries of a window against a
+// block of at most 64 of its keys.  Lane = query: q_i, the running maximum, sum and output stay in the lane's
+// registers while the keys stream through the wavefront one per step (two per step, in two 32-lane groups,
+// when the window has at most 32 voxels), so there is no cross-lane reduction, no atomic on data and no
+// O(pairs) index array; the result is deterministic.  Windows of more than 64 voxels leave one partial result
+// per key block, combined by generic_merge_kernel.
 //
 // Math (per window, sorted positions i, j, head h), following the reference kernels
 // Swin3D/src/attn/self_attn_aio_fwd.cu:16-52 and :111-188:
