@@ -133,13 +133,13 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
  *   dout           device [N,H,D] of `dtype`: gradient of the loss w.r.t. `out`
  *   dq, dk, dv     device [N,H,D] of `dtype`, overwritten (every row belongs to exactly one window)
  *   dtable_q/k/v   device FP32 [table_len], overwritten; layout of the tables
- *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, N, W) bytes
+ *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W) bytes
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
  * dq, dk, dv are sums in a fixed order (deterministic); the table gradients are accumulated per
  * wavefront and added to global memory with fp32 atomics (order varies between runs).
  */
-size_t s3d_attn_bwd_workspace_bytes(int32_t H, int64_t N, int64_t W);
+size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W);
 int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
                  const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
                  const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords,

@@ -57,6 +57,7 @@ struct BwdArgs {
     void *dq, *dk, *dv;
     float *dtq, *dtk, *dtv;
     float *delta;     // [N,H] dout_i . o_i
+    float *tgrad;     // per-wavefront table gradients of a sweep: [wavefront][kind][64 * BLK rows][D]
     int32_t *units;   // H * kQueues work counters (kCounterStride apart), the unit count, (window, chunk) per unit
     int32_t H, D, nd, total_rows;
     int64_t N, W, table_len;
@@ -118,12 +119,42 @@ __device__ __forceinline__ float lane_value(float x, int src)
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
 }
 
-__device__ __forceinline__ int crse_row(float ci, float cj, int rows)
+// Row of the axis table hit by a pair; fp32 arithmetic in the reference's operation order (subtract, add
+// half the row count, clamp, truncate).  The reference clamps to [0, rows] and folds the upper edge onto
+// the last row after truncation; clamping to [0, largest float below rows] gives the same row for every
+// input with one median-of-three and no integer minimum.
+__device__ __forceinline__ float crse_upper(int rows)
+{
+    return __int_as_float(__float_as_int(static_cast<float>(rows)) - 1);
+}
+__device__ __forceinline__ int crse_row(float ci, float cj, float half_rows, float upper)
 {
     float rel = ci - cj;
-    rel = rel + static_cast<float>(rows / 2);
-    rel = fminf(fmaxf(rel, 0.0f), static_cast<float>(rows));
-    return min(static_cast<int>(rel), rows - 1);
+    rel = rel + half_rows;
+    return static_cast<int>(__builtin_amdgcn_fmed3f(rel, 0.0f, upper));
+}
+
+// 16-byte LDS reads at a 32-bit LDS address (pointer arithmetic on generic pointers is 64-bit)
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const f32x4_t lds_float4_t;
+__device__ __forceinline__ uint32_t lds_address(const void *p)
+{
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p));   // low half of a flat LDS address
+}
+template <int D> __device__ __forceinline__ void load_row_lds(uint32_t addr, float *dst)
+{
+#pragma unroll
+    for (int c = 0; c < D; c += 4) {
+        const f32x4_t v = *(lds_float4_t *)(addr + 4 * c);
+        dst[c] = v[0]; dst[c + 1] = v[1]; dst[c + 2] = v[2]; dst[c + 3] = v[3];
+    }
+}
+// a * b + c with 24-bit factors: one full-rate instruction (a 32-bit integer multiply issues at a quarter of the rate)
+__device__ __forceinline__ uint32_t mad_u24(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t d;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(c));
+    return d;
 }
 
 // delta[i][h] = dout_i . o_i; the table gradients and the work counters start at zero
@@ -204,14 +235,13 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int HD = H * D;
     // workgroups go to the XCDs in turn: consecutive runs of eight serve one head, so every XCD gets every head
     const int h = (blockIdx.x / kQueues) % H;
-    // fp32 table slices of the head, rows padded by 16 bytes: with a 32- or 64-byte row stride a wavefront's
-    // 16-byte gathers of different rows would fall on 4 or 2 of the eight 4-bank groups
-    constexpr int kRowStride = D + 4;
-    const int cells = a.total_rows * kRowStride;
-    float *tab_q = smem;
-    float *tab_k = tab_q + cells;
-    float *tab_v = tab_k + cells;
-    int *hist_all = reinterpret_cast<int *>(tab_v + cells);
+    // fp32 table slices of the head; a row holds the q-side, k-side and v-side slices back to back (one LDS
+    // address per pair and axis) and is padded by 16 bytes: with a row stride that is a multiple of 32 bytes a
+    // wavefront's 16-byte gathers of different rows would fall on few of the eight 4-bank groups
+    constexpr int kRowStride = 3 * D + 4;
+    constexpr int kRowBytes = kRowStride * 4;
+    float *tab = smem;
+    int *hist_all = reinterpret_cast<int *>(tab + a.total_rows * kRowStride);
 
     {
         const T *gq = static_cast<const T *>(a.table_q);
@@ -220,9 +250,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         for (int t = threadIdx.x; t < a.total_rows * D; t += kBwdThreads) {
             const int r = t / D, c = t - r * D;
             const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
-            tab_q[r * kRowStride + c] = as_float(gq[g]);
-            tab_k[r * kRowStride + c] = as_float(gk[g]);
-            tab_v[r * kRowStride + c] = as_float(gv[g]);
+            tab[r * kRowStride + c] = as_float(gq[g]);
+            tab[r * kRowStride + D + c] = as_float(gk[g]);
+            tab[r * kRowStride + 2 * D + c] = as_float(gv[g]);
         }
         for (int t = threadIdx.x; t < kBwdWaves * kHistWords; t += kBwdThreads) hist_all[t] = 0;
     }
@@ -243,6 +273,17 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     for (int m = 0; m < BLK; ++m)
 #pragma unroll
         for (int c = 0; c < D; ++c) acc_a[m][c] = acc_b[m][c] = 0.0f;
+
+    const uint32_t tab_addr = __builtin_amdgcn_readfirstlane(lds_address(tab));
+    const uint32_t row_bytes = kRowBytes;
+    float half_rows[ND], upper[ND];
+    uint32_t base_off[ND];
+#pragma unroll
+    for (int n = 0; n < ND; ++n) {
+        half_rows[n] = static_cast<float>(a.rows[n] / 2);
+        upper[n] = crse_upper(a.rows[n]);
+        base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + a.base[n] * kRowBytes);
+    }
 
     const int2 *unit_list = reinterpret_cast<const int2 *>(a.units + units_list_index(H));
     const int total_units = __builtin_amdgcn_readfirstlane(a.units[units_total_index(H)]);
@@ -332,11 +373,11 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
             for (int n = 0; n < ND; ++n) {
                 const float ci = KEY_OWNED ? st_c[n] : own_c[n];
                 const float cj = KEY_OWNED ? own_c[n] : st_c[n];
-                r[n] = crse_row(ci, cj, a.rows[n]);
-                const int off = (a.base[n] + r[n]) * kRowStride;
+                r[n] = crse_row(ci, cj, half_rows[n], upper[n]);
+                const uint32_t off = mad_u24(static_cast<uint32_t>(r[n]), row_bytes, base_off[n]);
                 float tq_r[D], tk_r[D];
-                load_row<D>(tab_q + off, tq_r);
-                load_row<D>(tab_k + off, tk_r);
+                load_row_lds<D>(off, tq_r);
+                load_row_lds<D>(off + 4 * D, tk_r);
 #pragma unroll
                 for (int c = 0; c < D; ++c) {
                     bq[c] += tq_r[c];
@@ -344,7 +385,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                 }
                 if constexpr (kNeedDl) {
                     float tv_r[D];
-                    load_row<D>(tab_v + off, tv_r);
+                    load_row_lds<D>(off + 8 * D, tv_r);
 #pragma unroll
                     for (int c = 0; c < D; ++c) bv[c] += tv_r[c];
                 }
@@ -449,25 +490,45 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         }
     }
 
-    // lane l of block m = flat table row 64 m + l: add this wavefront's table gradients to the global tables
-    float *dst_a = KEY_OWNED ? a.dtq : a.dtk;
+    // lane l of block m = flat table row 64 m + l: the wavefront leaves its table gradients in a slot of its own
+    // (no atomics: thousands of wavefronts adding to the same few thousand addresses cost 15 % of the backward);
+    // bwd_reduce_tables_kernel sums the slots of a head
+    float *slot = a.tgrad + (static_cast<size_t>(blockIdx.x) * kBwdWaves + wave) * (2 * kFlat * D);
 #pragma unroll
     for (int m = 0; m < BLK; ++m) {
         const int row = m * 64 + lane;
-        if (row < a.total_rows) {
-            const int64_t g = static_cast<int64_t>(row) * HD + h * D;
-#pragma unroll
-            for (int c = 0; c < D; ++c) {
-                if constexpr (kAccA) atomicAdd(dst_a + g + c, acc_a[m][c]);
-                if constexpr (kAccB) atomicAdd(a.dtv + g + c, acc_b[m][c]);
-            }
-        }
+        if constexpr (kAccA) store_row<D>(slot + static_cast<size_t>(row) * D, acc_a[m]);
+        if constexpr (kAccB) store_row<D>(slot + static_cast<size_t>(kFlat + row) * D, acc_b[m]);
     }
+}
+
+// Sums the per-wavefront table gradients of a sweep over the wavefronts of each head: one thread per
+// (kind, flat row, head, channel).  dst_a / dst_b: the gradient tables of kind 0 / 1 (null = not produced).
+__global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float *dst_a, float *dst_b, int flat_rows,
+                                                                 int groups)
+{
+    const int H = a.H, D = a.D;
+    const int per_kind = a.total_rows * H * D;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= 2 * per_kind) return;
+    const int kind = t / per_kind;
+    float *dst = kind == 0 ? dst_a : dst_b;
+    if (!dst) return;
+    const int e = t - kind * per_kind;
+    const int c = e % D, h = (e / D) % H, row = e / (D * H);
+    const size_t slot_floats = 2 * static_cast<size_t>(flat_rows) * D;
+    const size_t in_slot = (static_cast<size_t>(kind) * flat_rows + row) * D + c;
+    // workgroup b serves head (b / kQueues) % H
+    float sum = 0.0f;
+    for (int b = h * kQueues; b < groups; b += H * kQueues)
+        for (int x = 0; x < kQueues * kBwdWaves; ++x)
+            sum += a.tgrad[(static_cast<size_t>(b) * kBwdWaves + x) * slot_floats + in_slot];
+    dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
 }
 
 size_t bwd_lds_bytes(const BwdArgs &a, int kinds, int blk)
 {
-    return sizeof(float) * 3 * static_cast<size_t>(a.total_rows) * (a.D + 4) +
+    return sizeof(float) * static_cast<size_t>(a.total_rows) * (3 * a.D + 4) +
            sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(blk) * 64;
 }
 
@@ -486,16 +547,41 @@ int launch_sweep_blk(const BwdArgs &a, int grid, hipStream_t stream)
     hipLaunchKernelGGL(bwd_reset_counters_kernel, dim3(1), dim3(64), 0, stream, a);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
+    float *dst_a = need_dl ? (KEY_OWNED ? a.dtq : a.dtk) : nullptr;
+    float *dst_b = (KEY_OWNED && MODE != 1) ? a.dtv : nullptr;
+    const int threads = 2 * a.total_rows * a.H * a.D;
+    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
+                       a, dst_a, dst_b, BLK * 64, grid);
+    S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }
 
-// the usual tables (quant 4: 32-row colour / normal axes) fit 2/3 of ND blocks; any table fits ND blocks
+// table-gradient registers for as many 64-row blocks as the head's flat table has: 5 for window 5 at four steps
+// per cell with all nine axes (312 rows), 6 for window 7 (360 rows); every block costs 2 * D registers and a
+// share of the per-step histogram flush
 template <typename T, int D, int ND, bool KEY_OWNED, int MODE>
 int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
 {
+    const int blocks = (a.total_rows + 63) / 64;
     constexpr int kSmall = 2 * ND / 3;
-    if (a.total_rows <= 64 * kSmall) return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, kSmall>(a, grid, stream);
+    if constexpr (ND == 9) {
+        if (blocks <= 5) return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, 5>(a, grid, stream);
+    }
+    if (blocks <= kSmall) return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, kSmall>(a, grid, stream);
     return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, ND>(a, grid, stream);
+}
+
+// workgroups of a sweep: whole sets of (XCDs x heads), about two per CU (a workgroup serves one head for its
+// whole life)
+int bwd_grid(int H)
+{
+    int device = 0, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
+    }
+    const int set = kQueues * H;
+    return (2 * cus / set > 0 ? 2 * cus / set : 1) * set;
 }
 
 template <typename T, int D, int ND>
@@ -507,14 +593,7 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
     S3D_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(bwd_units_kernel, dim3(1), dim3(1024), 0, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
-    int device = 0, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
-    }
-    // a workgroup serves one head for its whole life: whole sets of (XCDs x heads), about two workgroups per CU
-    const int set = kQueues * a.H;
-    const int grid = (2 * cus / set > 0 ? 2 * cus / set : 1) * set;
+    const int grid = bwd_grid(a.H);
     if constexpr (D <= 8) {
         // one key-owned sweep when both sets of table-gradient registers fit two wavefronts per SIMD
         if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
@@ -556,15 +635,24 @@ size_t bwd_units_bytes(int64_t W, int64_t N, int H)
     return align_up(sizeof(int32_t) * (units_list_index(H) + 2 * max_units), 256);
 }
 
+size_t bwd_delta_bytes(int64_t N, int H) { return align_up(sizeof(float) * static_cast<size_t>(N) * H, 256); }
+
+// one slot per wavefront of a sweep: two kinds x (64 rows per axis at most) x D floats
+size_t bwd_tgrad_bytes(int H, int D, int nd)
+{
+    return align_up(sizeof(float) * static_cast<size_t>(bwd_grid(H)) * kBwdWaves * 2 * (64 * nd) * D, 256);
+}
+
 }  // namespace
 }  // namespace s3d
 
-extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_bytes(int32_t H, int64_t N,
+extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D,
+                                                                                      int32_t nd, int64_t N,
                                                                                       int64_t W)
 {
     using namespace s3d;
-    if (H < 1 || N < 0 || W < 0) return 0;
-    return bwd_units_bytes(W, N, H) + align_up(sizeof(float) * static_cast<size_t>(N) * H, 256);
+    if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || N < 0 || W < 0) return 0;
+    return bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
@@ -597,7 +685,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     if (int rc = fill_bwd_axes(a, table_sizes, nd, table_len)) return rc;
     if (!dtable_q || !dtable_k || !dtable_v)
         return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null table-gradient pointer");
-    const size_t need = s3d_attn_bwd_workspace_bytes(H, N, W);
+    const size_t need = s3d_attn_bwd_workspace_bytes(H, D, nd, N, W);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_bwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
@@ -613,6 +701,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
     a.units = static_cast<int32_t *>(workspace);
     a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H));
+    a.tgrad = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (N == 0 || W == 0) {
         // nothing to differentiate: the table gradients are zero

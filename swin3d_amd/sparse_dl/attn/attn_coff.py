@@ -240,7 +240,7 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
     out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, n, w_sizes.numel())
+        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, n, w_sizes.numel())
         workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
         status = lib.s3d_attn_bwd(

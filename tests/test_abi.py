@@ -70,7 +70,7 @@ def test_more_argument_errors_without_a_device(hip_lib):
     c_big = (ctypes.c_int32 * 9)(*big)
     st = hip_lib.s3d_attn_bwd(*([None] * 6), c_big, 9, sum(big), *([None] * 14), 10, 6, 8, 1, 1, None, 0, None)
     assert st < 0 and b"table rows per head" in hip_lib.s3d_last_error_string()
-    assert hip_lib.s3d_attn_bwd_workspace_bytes(6, 1000, 40) >= 4 * (40 + 6) + 4 * 6000
+    assert hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, 1000, 40) >= 4 * (40 + 6) + 4 * 6000
     st = hip_lib.s3d_knn_interpolate(None, None, 0, 10, None, 10, 8, 0, None, None)
     assert st < 0 and b"K=0" in hip_lib.s3d_last_error_string()
     st = hip_lib.s3d_knn_interpolate(None, None, 3, 10, None, 10, 8, 7, None, None)
