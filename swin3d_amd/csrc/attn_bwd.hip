@@ -22,30 +22,16 @@
 //
 // Windows of at most 32 voxels put two streamed elements in one wavefront step (two 32-lane groups).
 #include "attn_kernels.h"
-
-#include <hip/hip_fp16.h>
+#include "sweep_common.h"
 
 namespace s3d {
 namespace {
 
+using namespace sweep;
+
 constexpr int kBwdThreads = 256;
 constexpr int kBwdWaves = kBwdThreads / 64;
 constexpr int kChunk = 64;            // owned elements per unit = lanes of a wavefront
-// Work distribution: atomics on one cache line retire one after the other (about 12 ns each on this part), so
-// every head has kQueues counters, each on a cache line of its own; unit u belongs to queue u % kQueues and a
-// wavefront moves to the next queue when the one it draws from is empty.
-// The chip has eight XCDs with an L2 each: a wavefront starts on the queue of the XCD it runs on, so all heads
-// of a unit are served from the same XCD and the unit's rows reach that L2 once.
-constexpr int kQueues = 8;
-constexpr int kCounterStride = 64;    // ints between counters (256 bytes)
-
-// id of the XCD (accelerator complex die) the wavefront runs on
-__device__ __forceinline__ int xcd_id()
-{
-    int id;
-    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID, 0, 4)" : "=s"(id));
-    return id;
-}
 constexpr float kFixP = 16777216.0f;  // 2^24: softmax weights of one query sum to at most 1
 constexpr float kFixL = 8388608.0f;   // 2^23: |dL| / max|dL| <= 1, at most 64 lanes meet in one bin
 
@@ -72,89 +58,10 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
 }
 
-template <int D> __device__ __forceinline__ void load_row(const float *p, float *dst)
-{
-#pragma unroll
-    for (int c = 0; c < D; c += 4) {
-        const float4 x = *reinterpret_cast<const float4 *>(p + c);
-        dst[c] = x.x; dst[c + 1] = x.y; dst[c + 2] = x.z; dst[c + 3] = x.w;
-    }
-}
-template <int D> __device__ __forceinline__ void load_row(const __half *p, float *dst)
-{
-#pragma unroll
-    for (int c = 0; c < D; c += 8) {
-        const uint4 x = *reinterpret_cast<const uint4 *>(p + c);
-        const __half2 *hh = reinterpret_cast<const __half2 *>(&x);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float2 f = __half22float2(hh[e]);
-            dst[c + 2 * e] = f.x;
-            dst[c + 2 * e + 1] = f.y;
-        }
-    }
-}
-template <int D> __device__ __forceinline__ void store_row(float *p, const float *src)
-{
-#pragma unroll
-    for (int c = 0; c < D; c += 4) *reinterpret_cast<float4 *>(p + c) = make_float4(src[c], src[c + 1], src[c + 2], src[c + 3]);
-}
-template <int D> __device__ __forceinline__ void store_row(__half *p, const float *src)
-{
-#pragma unroll
-    for (int c = 0; c < D; c += 8) {
-        uint4 x;
-        __half2 *hh = reinterpret_cast<__half2 *>(&x);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) hh[e] = __floats2half2_rn(src[c + 2 * e], src[c + 2 * e + 1]);
-        *reinterpret_cast<uint4 *>(p + c) = x;
-    }
-}
-__device__ __forceinline__ float as_float(float x) { return x; }
-__device__ __forceinline__ float as_float(__half x) { return __half2float(x); }
-
 // value of x in lane `src` (src uniform): a scalar read instead of an LDS permute
 __device__ __forceinline__ float lane_value(float x, int src)
 {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src));
-}
-
-// Row of the axis table hit by a pair; fp32 arithmetic in the reference's operation order (subtract, add
-// half the row count, clamp, truncate).  The reference clamps to [0, rows] and folds the upper edge onto
-// the last row after truncation; clamping to [0, largest float below rows] gives the same row for every
-// input with one median-of-three and no integer minimum.
-__device__ __forceinline__ float crse_upper(int rows)
-{
-    return __int_as_float(__float_as_int(static_cast<float>(rows)) - 1);
-}
-__device__ __forceinline__ int crse_row(float ci, float cj, float half_rows, float upper)
-{
-    float rel = ci - cj;
-    rel = rel + half_rows;
-    return static_cast<int>(__builtin_amdgcn_fmed3f(rel, 0.0f, upper));
-}
-
-// 16-byte LDS reads at a 32-bit LDS address (pointer arithmetic on generic pointers is 64-bit)
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) const f32x4_t lds_float4_t;
-__device__ __forceinline__ uint32_t lds_address(const void *p)
-{
-    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p));   // low half of a flat LDS address
-}
-template <int D> __device__ __forceinline__ void load_row_lds(uint32_t addr, float *dst)
-{
-#pragma unroll
-    for (int c = 0; c < D; c += 4) {
-        const f32x4_t v = *(lds_float4_t *)(addr + 4 * c);
-        dst[c] = v[0]; dst[c + 1] = v[1]; dst[c + 2] = v[2]; dst[c + 3] = v[3];
-    }
-}
-// a * b + c with 24-bit factors: one full-rate instruction (a 32-bit integer multiply issues at a quarter of the rate)
-__device__ __forceinline__ uint32_t mad_u24(uint32_t a, uint32_t b, uint32_t c)
-{
-    uint32_t d;
-    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(c));
-    return d;
 }
 
 // delta[i][h] = dout_i . o_i; the table gradients and the work counters start at zero
@@ -167,7 +74,7 @@ __global__ void bwd_prepare_kernel(BwdArgs a)
     const T *o = static_cast<const T *>(a.out);
     for (int64_t t = t0; t < a.N * a.H; t += stride) {
         float s = 0.0f;
-        for (int c = 0; c < a.D; ++c) s += as_float(go[t * a.D + c]) * as_float(o[t * a.D + c]);
+        for (int c = 0; c < a.D; ++c) s += to_float(go[t * a.D + c]) * to_float(o[t * a.D + c]);
         a.delta[t] = s;
     }
     for (int64_t t = t0; t < a.table_len; t += stride) {
@@ -235,13 +142,13 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int HD = H * D;
     // workgroups go to the XCDs in turn: consecutive runs of eight serve one head, so every XCD gets every head
     const int h = (blockIdx.x / kQueues) % H;
-    // fp32 table slices of the head; a row holds the q-side, k-side and v-side slices back to back (one LDS
-    // address per pair and axis) and is padded by 16 bytes: with a row stride that is a multiple of 32 bytes a
-    // wavefront's 16-byte gathers of different rows would fall on few of the eight 4-bank groups
-    constexpr int kRowStride = 3 * D + 4;
-    constexpr int kRowBytes = kRowStride * 4;
-    float *tab = smem;
-    int *hist_all = reinterpret_cast<int *>(tab + a.total_rows * kRowStride);
+    // table slices of the head in the I/O type; a row holds the q-side, k-side and v-side slices back to back (one
+    // LDS address per pair and axis)
+    constexpr int kRowStride = table_row_stride<T, D>();
+    constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
+    T *tab = reinterpret_cast<T *>(smem);
+    int *hist_all = reinterpret_cast<int *>(reinterpret_cast<char *>(smem) +
+                                            (static_cast<size_t>(a.total_rows) * kRowBytes + 15) / 16 * 16);
 
     {
         const T *gq = static_cast<const T *>(a.table_q);
@@ -250,9 +157,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         for (int t = threadIdx.x; t < a.total_rows * D; t += kBwdThreads) {
             const int r = t / D, c = t - r * D;
             const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
-            tab[r * kRowStride + c] = as_float(gq[g]);
-            tab[r * kRowStride + D + c] = as_float(gk[g]);
-            tab[r * kRowStride + 2 * D + c] = as_float(gv[g]);
+            tab[r * kRowStride + c] = gq[g];
+            tab[r * kRowStride + D + c] = gk[g];
+            tab[r * kRowStride + 2 * D + c] = gv[g];
         }
         for (int t = threadIdx.x; t < kBwdWaves * kHistWords; t += kBwdThreads) hist_all[t] = 0;
     }
@@ -274,6 +181,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 #pragma unroll
         for (int c = 0; c < D; ++c) acc_a[m][c] = acc_b[m][c] = 0.0f;
 
+    // 1.0 the optimiser cannot see through: x * one + sum keeps an fp16 row widened inside one mixed-precision FMA
+    float one = 1.0f;
+    asm volatile("" : "+v"(one));
     const uint32_t tab_addr = __builtin_amdgcn_readfirstlane(lds_address(tab));
     const uint32_t row_bytes = kRowBytes;
     float half_rows[ND], upper[ND];
@@ -316,14 +226,15 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         const int own_pos = s0 + min(own, n_w - 1);
         const int own_row = a.n2n[own_pos];
 
-        // owned side
-        float own_x[D], own_y[D], own_c[ND], own_m = 0.0f, own_inv = 0.0f, own_delta = 0.0f;
+        // owned side, in the I/O type (fp16: packed pairs)
+        Slice<T, D> own_x, own_y;
+        float own_c[ND], own_m = 0.0f, own_inv = 0.0f, own_delta = 0.0f;
         if constexpr (KEY_OWNED) {
-            load_row<D>(gk + static_cast<int64_t>(own_row) * HD + h * D, own_x);   // k_j
-            if constexpr (kNeedDl) load_row<D>(gv + static_cast<int64_t>(own_row) * HD + h * D, own_y);   // v_j
+            own_x.load(gk + static_cast<int64_t>(own_row) * HD + h * D);   // k_j
+            if constexpr (kNeedDl) own_y.load(gv + static_cast<int64_t>(own_row) * HD + h * D);   // v_j
         } else {
-            load_row<D>(gq + static_cast<int64_t>(own_row) * HD + h * D, own_x);   // q_i
-            load_row<D>(ggo + static_cast<int64_t>(own_row) * HD + h * D, own_y);  // dout_i
+            own_x.load(gq + static_cast<int64_t>(own_row) * HD + h * D);   // q_i
+            own_y.load(ggo + static_cast<int64_t>(own_row) * HD + h * D);  // dout_i
             own_m = a.out_max[static_cast<int64_t>(own_row) * H + h];
             own_inv = 1.0f / a.out_sum[static_cast<int64_t>(own_row) * H + h];
             own_delta = a.delta[static_cast<int64_t>(own_row) * H + h];
@@ -343,77 +254,78 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
             const int st_row = st_row_next;
             if (it + 1 < steps) st_row_next = a.n2n[s0 + min(st + ng, n_w - 1)];
             // streamed side (the same for all lanes of a group)
-            float st_x[D], st_y[D], st_c[ND], st_m = 0.0f, st_inv = 0.0f, st_delta = 0.0f;
+            Slice<T, D> st_x, st_y;
+            float st_c[ND], st_m = 0.0f, st_inv = 0.0f, st_delta = 0.0f;
             if constexpr (KEY_OWNED) {
-                load_row<D>(gq + static_cast<int64_t>(st_row) * HD + h * D, st_x);    // q_i
-                load_row<D>(ggo + static_cast<int64_t>(st_row) * HD + h * D, st_y);   // dout_i
+                st_x.load(gq + static_cast<int64_t>(st_row) * HD + h * D);    // q_i
+                st_y.load(ggo + static_cast<int64_t>(st_row) * HD + h * D);   // dout_i
                 st_m = a.out_max[static_cast<int64_t>(st_row) * H + h];
                 st_inv = 1.0f / a.out_sum[static_cast<int64_t>(st_row) * H + h];
                 st_delta = a.delta[static_cast<int64_t>(st_row) * H + h];
             } else {
-                load_row<D>(gk + static_cast<int64_t>(st_row) * HD + h * D, st_x);    // k_j
-                load_row<D>(gv + static_cast<int64_t>(st_row) * HD + h * D, st_y);    // v_j
+                st_x.load(gk + static_cast<int64_t>(st_row) * HD + h * D);    // k_j
+                st_y.load(gv + static_cast<int64_t>(st_row) * HD + h * D);    // v_j
             }
 #pragma unroll
             for (int n = 0; n < ND; ++n) st_c[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
 
-            const float *qv = KEY_OWNED ? st_x : own_x;
-            const float *kv = KEY_OWNED ? own_x : st_x;
-            const float *vv = KEY_OWNED ? own_y : st_y;
-            const float *gov = KEY_OWNED ? st_y : own_y;
+            const Slice<T, D> &qv = KEY_OWNED ? st_x : own_x;
+            const Slice<T, D> &kv = KEY_OWNED ? own_x : st_x;
+            const Slice<T, D> &vv = KEY_OWNED ? own_y : st_y;
+            const Slice<T, D> &gov = KEY_OWNED ? st_y : own_y;
             const float m_i = KEY_OWNED ? st_m : own_m;
             const float inv_i = KEY_OWNED ? st_inv : own_inv;
             const float delta_i = KEY_OWNED ? st_delta : own_delta;
 
+            // L = q.k + q.Tq + k.Tk and dP = dout.(v + Tv) as dot products against the gathered rows; the one
+            // row sum that enters an owned gradient as a vector is kept: Tk (dk_j) or Tq (dq_i)
+            constexpr bool kChain = Slice<T, D>::kChainLogit;
             int r[ND];
-            float bq[D], bk[D], bv[D];
+            float tsum[D];
 #pragma unroll
-            for (int c = 0; c < D; ++c) bq[c] = bk[c] = bv[c] = 0.0f;
+            for (int c = 0; c < D; ++c) tsum[c] = 0.0f;
+            float logit = qv.dot(kv, 0.0f);
+            float dp = 0.0f;
+            if constexpr (kNeedDl) dp = gov.dot(vv, 0.0f);
 #pragma unroll
             for (int n = 0; n < ND; ++n) {
                 const float ci = KEY_OWNED ? st_c[n] : own_c[n];
                 const float cj = KEY_OWNED ? own_c[n] : st_c[n];
                 r[n] = crse_row(ci, cj, half_rows[n], upper[n]);
                 const uint32_t off = mad_u24(static_cast<uint32_t>(r[n]), row_bytes, base_off[n]);
-                float tq_r[D], tk_r[D];
-                load_row_lds<D>(off, tq_r);
-                load_row_lds<D>(off + 4 * D, tk_r);
-#pragma unroll
-                for (int c = 0; c < D; ++c) {
-                    bq[c] += tq_r[c];
-                    bk[c] += tk_r[c];
+                Slice<T, D> tq_r, tk_r;
+                tq_r.load_lds(off);
+                tk_r.load_lds(off + D * sizeof(T));
+                if constexpr (KEY_OWNED) {
+                    if (kChain) logit = qv.dot(tq_r, logit); else logit += qv.dot(tq_r, 0.0f);
+                    tk_r.fma_to(tsum, one);
+                } else {
+                    tq_r.fma_to(tsum, one);
+                    if (kChain) logit = kv.dot(tk_r, logit); else logit += kv.dot(tk_r, 0.0f);
                 }
                 if constexpr (kNeedDl) {
-                    float tv_r[D];
-                    load_row_lds<D>(off + 8 * D, tv_r);
-#pragma unroll
-                    for (int c = 0; c < D; ++c) bv[c] += tv_r[c];
+                    Slice<T, D> tv_r;
+                    tv_r.load_lds(off + 2 * D * sizeof(T));
+                    if (kChain) dp = gov.dot(tv_r, dp); else dp += gov.dot(tv_r, 0.0f);
                 }
             }
-            float logit = 0.0f;
-#pragma unroll
-            for (int c = 0; c < D; ++c) logit += qv[c] * kv[c] + qv[c] * bq[c] + kv[c] * bk[c];
+            if (kChain) logit = (KEY_OWNED ? kv : qv).dot_f32(tsum, logit);
+            else logit += (KEY_OWNED ? kv : qv).dot_f32(tsum, 0.0f);
             const bool valid = own_valid && st_valid;
             const float p = valid ? __expf(logit - m_i) * inv_i : 0.0f;
             float dl = 0.0f;
-            if constexpr (kNeedDl) {
-                float dp = 0.0f;
-#pragma unroll
-                for (int c = 0; c < D; ++c) dp += gov[c] * (vv[c] + bv[c]);
-                dl = p * (dp - delta_i);
-            }
+            if constexpr (kNeedDl) dl = p * (dp - delta_i);
             if constexpr (KEY_OWNED) {
                 if constexpr (MODE != 2) {
+                    qv.fma_to(res_x, dl);                                           // dk_j += dl (q_i + Tk)
 #pragma unroll
-                    for (int c = 0; c < D; ++c) res_x[c] += dl * (qv[c] + bk[c]);   // dk_j
+                    for (int c = 0; c < D; ++c) res_x[c] += dl * tsum[c];
                 }
-                if constexpr (MODE != 1) {
-#pragma unroll
-                    for (int c = 0; c < D; ++c) res_y[c] += p * gov[c];             // dv_j
-                }
+                if constexpr (MODE != 1) gov.fma_to(res_y, p);                      // dv_j += p dout_i
             } else {
+                kv.fma_to(res_x, dl);                                               // dq_i += dl (k_j + Tq)
 #pragma unroll
-                for (int c = 0; c < D; ++c) res_x[c] += dl * (kv[c] + bq[c]);       // dq_i
+                for (int c = 0; c < D; ++c) res_x[c] += dl * tsum[c];
             }
 
             // table gradients: histogram of the step over table rows, then a rank-1 update (lane = row)
@@ -441,29 +353,23 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                 const int src = __builtin_amdgcn_readfirstlane(g * gs);   // a lane of group g: its streamed registers are the group's
                 if constexpr (kAccA) {
                     const float sc = lane_value(amax, src) * (1.0f / kFixL);
-                    float sx[D];
-#pragma unroll
-                    for (int c = 0; c < D; ++c) sx[c] = lane_value(st_x[c], src);   // q_i (key-owned) or k_j
+                    const Slice<T, D> sx = st_x.lane(src);   // q_i (key-owned) or k_j
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
                         int *cell = hist_a + g * kFlat + m * 64 + lane;
                         const float gsum = static_cast<float>(*cell) * sc;
                         *cell = 0;
-#pragma unroll
-                        for (int c = 0; c < D; ++c) acc_a[m][c] += gsum * sx[c];
+                        sx.fma_to(acc_a[m], gsum);
                     }
                 }
                 if constexpr (kAccB) {
-                    float sy[D];
-#pragma unroll
-                    for (int c = 0; c < D; ++c) sy[c] = lane_value(st_y[c], src);   // dout_i
+                    const Slice<T, D> sy = st_y.lane(src);   // dout_i
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
                         int *cell = hist_b + g * kFlat + m * 64 + lane;
                         const float psum = static_cast<float>(*cell) * (1.0f / kFixP);
                         *cell = 0;
-#pragma unroll
-                        for (int c = 0; c < D; ++c) acc_b[m][c] += psum * sy[c];
+                        sy.fma_to(acc_b[m], psum);
                     }
                 }
             }
@@ -526,9 +432,10 @@ __global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float
     dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
 }
 
+template <typename T, int D>
 size_t bwd_lds_bytes(const BwdArgs &a, int kinds, int blk)
 {
-    return sizeof(float) * static_cast<size_t>(a.total_rows) * (3 * a.D + 4) +
+    return align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride<T, D>(), 16) +
            sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(blk) * 64;
 }
 
@@ -538,7 +445,7 @@ int launch_sweep_blk(const BwdArgs &a, int grid, hipStream_t stream)
     constexpr bool need_dl = !KEY_OWNED || MODE != 2;
     constexpr int kinds = (need_dl ? 1 : 0) + ((KEY_OWNED && MODE != 1) ? 1 : 0);
     auto kernel = attn_bwd_sweep_kernel<T, D, ND, KEY_OWNED, MODE, BLK>;
-    const size_t lds = bwd_lds_bytes(a, kinds, BLK);
+    const size_t lds = bwd_lds_bytes<T, D>(a, kinds, BLK);
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: the tables of one head (%d rows x %d) do not fit LDS",
                     a.total_rows, a.D);
