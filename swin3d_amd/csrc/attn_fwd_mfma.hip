@@ -32,6 +32,7 @@
 // one step ahead of its use (next head's q/k/v fragments, next axis' table fragments) and the
 // transposed value table of all heads sits in LDS, shared by the wavefronts of the workgroup.
 #include "attn_kernels.h"
+#include "sweep_common.h"
 
 namespace s3d {
 namespace {
@@ -45,6 +46,12 @@ constexpr int kWaves = 8;             // wavefronts per workgroup (they share th
 constexpr int kTile = 32;             // queries / keys per tile
 constexpr float kFix = 16777216.0f;   // 2^24 fixed point of the histogram
 constexpr int kItemsPerWave = 2;      // heads are grouped so that a wavefront draws about this many items
+
+// index (in ints) of the first work counter inside the item list: after the [W + 3] header, on a 256-byte boundary
+__host__ __device__ inline size_t queue_counters_index(int64_t W)
+{
+    return (static_cast<size_t>(W > 0 ? W : 1) + 3 + 63) / 64 * 64;
+}
 
 // LDS operations of one wavefront execute in order; this only stops the compiler from moving
 // LDS accesses across the point where lanes exchange data (global loads stay free to move).
@@ -155,7 +162,11 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
     const int total_items = __builtin_amdgcn_readfirstlane(item_end[a.W - 1]) * groups;
     // work items are handed out through a device counter (zeroed by attn_prepare_kernel), so a
     // wavefront that drew long items simply draws fewer of them
-    int *next_item = static_cast<int *>(a.items) + a.W;
+    // eight queues, each counter on a cache line of its own (atomics on one line retire one at a time); item i
+    // belongs to queue i % 8 and a wavefront starts on the queue of the XCD it runs on
+    int *counters = static_cast<int *>(a.items) + queue_counters_index(a.W);
+    int queue = sweep::xcd_id() % sweep::kQueues;
+    int tried = 0;
 
     const int cc = min(il, D - 1);               // channel this lane feeds to the value MFMAs
     const bool c_valid = il < D;
@@ -170,9 +181,13 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
 
     for (;;) {
         int item = 0;
-        if (lane == 0) item = atomicAdd(next_item, 1);
-        item = __builtin_amdgcn_readfirstlane(item);
-        if (item >= total_items) break;
+        if (lane == 0) item = atomicAdd(counters + queue * sweep::kCounterStride, 1);
+        item = __builtin_amdgcn_readfirstlane(item) * sweep::kQueues + queue;
+        if (item >= total_items) {
+            if (++tried == sweep::kQueues) break;
+            queue = (queue + 1) % sweep::kQueues;
+            continue;
+        }
         // item = (tile pair, head group); consecutive items share the tile pair
         const int pair = item / groups;
         const int h_begin = (item - pair * groups) * group_heads;
@@ -554,6 +569,8 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(AttnArgs a)
         run += tiles * tiles;
         item_end[w] = run;
     }
+    // the work counters of the attention kernel
+    if (threadIdx.x < sweep::kQueues) item_end[queue_counters_index(a.W) + threadIdx.x * sweep::kCounterStride] = 0;
     if (threadIdx.x == 1023) {
         // heads are split into groups when the tile pairs alone are too few to keep every wavefront
         // of the persistent grid busy with several items (deep stages: few, large windows, many heads)
@@ -561,7 +578,7 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(AttnArgs a)
         int groups = pairs > 0 ? (a.target_items + pairs - 1) / pairs : 1;
         groups = max(1, min(groups, a.H));
         const int group_heads = (a.H + groups - 1) / groups;
-        item_end[W] = 0;   // the work counter of the attention kernel
+        item_end[W] = 0;
         item_end[W + 1] = (a.H + group_heads - 1) / group_heads;
         item_end[W + 2] = group_heads;
     }
@@ -643,7 +660,7 @@ size_t attn_mfma_table_bytes(int H, int D, int padded_rows)
 
 size_t attn_mfma_items_bytes(int64_t W)
 {
-    return align_up(sizeof(int32_t) * (static_cast<size_t>(W > 0 ? W : 1) + 3), 256);
+    return sizeof(int32_t) * (queue_counters_index(W) + static_cast<size_t>(sweep::kQueues) * sweep::kCounterStride);
 }
 
 int attn_mfma_key_tiles(int max_window_voxels)
