@@ -38,9 +38,14 @@ __host__ __device__ inline size_t ws_max_units(int64_t W, int64_t N, int max_blo
 {
     return (static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / kChunk) * max_blocks;
 }
-__host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
+// list of the windows that are split along their keys (their count sits next to the unit count)
+__host__ __device__ inline size_t ws_split_offset(int H, int64_t W, int64_t N, int max_blocks)
 {
     return ws_units_offset(H) + (sizeof(int2) * ws_max_units(W, N, max_blocks) + 255) / 256 * 256;
+}
+__host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
+{
+    return ws_split_offset(H, W, N, max_blocks) + (sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1) + 255) / 256 * 256;
 }
 
 // Unit list of the launch: one descriptor (window, query chunk | key block << 16) per unit, the unit count,
@@ -52,10 +57,13 @@ __host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N
 __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
 {
     __shared__ int wave_long[16], wave_all[16];
+    __shared__ int split_count;
+    if (threadIdx.x == 0) split_count = 0;
     char *ws = static_cast<char *>(a.workspace);
     int *counters = reinterpret_cast<int *>(ws);
     int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
     int2 *units = reinterpret_cast<int2 *>(ws + ws_units_offset(a.H));
+    int *split = reinterpret_cast<int *>(ws + ws_split_offset(a.H, a.W, a.N, a.max_key_tiles));
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
     const int begin = threadIdx.x * per, end = min(begin + per, W);
@@ -99,48 +107,55 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
         int &run = n > 32 ? run_long : run_short;
         for (int c = 0; c < blocks; ++c)
             for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
+        if (blocks > 1) split[atomicAdd(&split_count, 1)] = w;   // any order: the merge treats windows independently
     }
-    if (threadIdx.x == 1023) *total = wave_all[15];
+    __syncthreads();
+    if (threadIdx.x == 1023) {
+        total[0] = wave_all[15];
+        total[1] = split_count;
+    }
     for (int t = threadIdx.x; t < a.H * kQueues; t += 1024) counters[t * kCounterStride] = 0;
 }
 
 // Windows of more than 64 voxels: combine the per-key-block partial results (unnormalised output, running
-// maximum, sum) of every (voxel, head).  One thread per (sorted position, head), position fastest.
+// maximum, sum) of every (voxel, head).  Workgroups take the split windows of the launch in turn; one thread
+// per (voxel of the window, head), voxel fastest.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
 {
     const int H = a.H;
-    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (t >= a.N * H) return;
-    const int h = static_cast<int>(t / a.N), pos = static_cast<int>(t - static_cast<int64_t>(h) * a.N);
-    int lo = 0, hi = static_cast<int>(a.W) - 1;   // last window that starts at or before pos
-    while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (a.w2n[mid] <= pos) lo = mid; else hi = mid - 1;
-    }
-    const int blocks = key_blocks(a.w_sizes[lo]);
-    if (blocks <= 1 || blocks > a.max_key_tiles) return;
-    const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
+    const char *ws = static_cast<const char *>(a.workspace);
+    const int count = reinterpret_cast<const int *>(ws + ws_total_offset(H))[1];
+    const int *split = reinterpret_cast<const int *>(ws + ws_split_offset(H, a.W, a.N, a.max_key_tiles));
     const int64_t block_stride = static_cast<int64_t>(H) * a.N * (D + 2);
-    float m = -INFINITY;
-    for (int kb = 0; kb < blocks; ++kb) m = fmaxf(m, part[kb * block_stride + D]);
-    float l = 0.0f, o[D];
+    for (int e = blockIdx.x; e < count; e += gridDim.x) {
+        const int w = split[e];
+        const int n_w = a.w_sizes[w], s0 = a.w2n[w];
+        const int blocks = key_blocks(n_w);
+        for (int t = threadIdx.x; t < n_w * H; t += blockDim.x) {
+            const int h = t / n_w, pos = s0 + (t - h * n_w);
+            const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
+            float m = -INFINITY;
+            for (int kb = 0; kb < blocks; ++kb) m = fmaxf(m, part[kb * block_stride + D]);
+            float l = 0.0f, o[D];
 #pragma unroll
-    for (int c = 0; c < D; ++c) o[c] = 0.0f;
-    for (int kb = 0; kb < blocks; ++kb) {
-        const float *pk = part + kb * block_stride;
-        const float wgt = __expf(pk[D] - m);
-        l += pk[D + 1] * wgt;
+            for (int c = 0; c < D; ++c) o[c] = 0.0f;
+            for (int kb = 0; kb < blocks; ++kb) {
+                const float *pk = part + kb * block_stride;
+                const float wgt = __expf(pk[D] - m);
+                l += pk[D + 1] * wgt;
 #pragma unroll
-        for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
+                for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
+            }
+            const int row = a.n2n[pos];
+            const float inv = 1.0f / l;
+#pragma unroll
+            for (int c = 0; c < D; ++c) o[c] *= inv;
+            store_row<D>(static_cast<T *>(a.out) + (static_cast<int64_t>(row) * H + h) * D, o);
+            if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
+            if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
+        }
     }
-    const int row = a.n2n[pos];
-    const float inv = 1.0f / l;
-#pragma unroll
-    for (int c = 0; c < D; ++c) o[c] *= inv;
-    store_row<D>(static_cast<T *>(a.out) + (static_cast<int64_t>(row) * H + h) * D, o);
-    if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
-    if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
 }
 
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
@@ -359,8 +374,8 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     if (a.max_key_tiles > 1) {
-        const int64_t threads = a.N * a.H;
-        hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256),
+        const int64_t want = a.W < 1024 ? a.W : 1024;
+        hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>(want > 0 ? want : 1)), dim3(256),
                            0, stream, a);
         S3D_HIP_CHECK(hipGetLastError());
     }
