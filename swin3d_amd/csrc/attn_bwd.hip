@@ -24,6 +24,8 @@
 #include "attn_kernels.h"
 #include "sweep_common.h"
 
+#include <type_traits>
+
 namespace s3d {
 namespace {
 
@@ -56,6 +58,25 @@ __device__ __forceinline__ void wave_lds_fence()
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+}
+
+// max of a non-negative value over the lanes of each group (32-lane halves when two_groups, else the wavefront),
+// returned in every lane: DPP moves inside the 16-lane rows and across them, two scalar reads; no LDS permutes
+__device__ __forceinline__ float group_max_nonneg(float v, bool two_groups, int grp)
+{
+    auto step = [](float x, auto ctrl, auto row_mask) {
+        const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value, decltype(row_mask)::value,
+                                                      0xf, true);
+        return fmaxf(x, __int_as_float(moved));
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{}, std::integral_constant<int, 0xf>{});    // quad_perm [1,0,3,2]
+    v = step(v, std::integral_constant<int, 0x4E>{}, std::integral_constant<int, 0xf>{});    // quad_perm [2,3,0,1]
+    v = step(v, std::integral_constant<int, 0x141>{}, std::integral_constant<int, 0xf>{});   // row_half_mirror
+    v = step(v, std::integral_constant<int, 0x140>{}, std::integral_constant<int, 0xf>{});   // row_mirror
+    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{});   // row_bcast15 into rows 1, 3
+    const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 31));
+    const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+    return two_groups ? (grp ? hi : lo) : fmaxf(lo, hi);
 }
 
 // value of x in lane `src` (src uniform): a scalar read instead of an LDS permute
@@ -169,6 +190,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const int lane = threadIdx.x & 63;
     int *hist_a = hist_all + wave * kHistWords;                 // dL histogram
     int *hist_b = hist_a + (kAccA ? 2 * kFlat : 0);             // P histogram
+    unsigned long long *hist_ab = reinterpret_cast<unsigned long long *>(hist_a);   // both, [group][flat row]
 
     const T *gq = static_cast<const T *>(a.q);
     const T *gk = static_cast<const T *>(a.k);
@@ -330,19 +352,27 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 
             // table gradients: histogram of the step over table rows, then a rank-1 update (lane = row)
             float amax = 0.0f;
+            int qd = 0, qp = 0;
             if constexpr (kAccA) {
-                amax = fabsf(dl);
+                amax = group_max_nonneg(fabsf(dl), ng == 2, grp);
+                qd = __float2int_rn(dl * (amax > 0.0f ? kFixL / amax : 0.0f));
+            }
+            if constexpr (kAccB) qp = __float2int_rn(p * kFixP);
+            if constexpr (kAccA && kAccB) {
+                // both histograms hit the same rows: one 64-bit cell per row, dL in the upper half and P (never
+                // negative, at most 64 * 2^24 per cell: no carry) in the lower, one atomic per pair and axis
+                const unsigned long long both =
+                    (static_cast<unsigned long long>(static_cast<unsigned>(qd)) << 32) + static_cast<unsigned>(qp);
+                if (valid && both != 0) {
 #pragma unroll
-                for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-                if (gs == 64) amax = fmaxf(amax, __shfl_xor(amax, 32));
-                const int qd = __float2int_rn(dl * (amax > 0.0f ? kFixL / amax : 0.0f));
+                    for (int n = 0; n < ND; ++n) atomicAdd(hist_ab + grp * kFlat + a.base[n] + r[n], both);
+                }
+            } else if constexpr (kAccA) {
                 if (valid && qd != 0) {
 #pragma unroll
                     for (int n = 0; n < ND; ++n) atomicAdd(hist_a + grp * kFlat + a.base[n] + r[n], qd);
                 }
-            }
-            if constexpr (kAccB) {
-                const int qp = __float2int_rn(p * kFixP);
+            } else {
                 if (valid && qp != 0) {
 #pragma unroll
                     for (int n = 0; n < ND; ++n) atomicAdd(hist_b + grp * kFlat + a.base[n] + r[n], qp);
@@ -351,7 +381,21 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
             wave_lds_fence();
             for (int g = 0; g < ng; ++g) {
                 const int src = __builtin_amdgcn_readfirstlane(g * gs);   // a lane of group g: its streamed registers are the group's
-                if constexpr (kAccA) {
+                if constexpr (kAccA && kAccB) {
+                    const float sc = lane_value(amax, src) * (1.0f / kFixL);
+                    const Slice<T, D> sx = st_x.lane(src);   // q_i
+                    const Slice<T, D> sy = st_y.lane(src);   // dout_i
+#pragma unroll
+                    for (int m = 0; m < BLK; ++m) {
+                        unsigned long long *cell = hist_ab + g * kFlat + m * 64 + lane;
+                        const unsigned long long both = *cell;
+                        *cell = 0;
+                        const float gsum = static_cast<float>(static_cast<int>(both >> 32)) * sc;
+                        const float psum = static_cast<float>(static_cast<unsigned>(both)) * (1.0f / kFixP);
+                        sx.fma_to(acc_a[m], gsum);
+                        sy.fma_to(acc_b[m], psum);
+                    }
+                } else if constexpr (kAccA) {
                     const float sc = lane_value(amax, src) * (1.0f / kFixL);
                     const Slice<T, D> sx = st_x.lane(src);   // q_i (key-owned) or k_j
 #pragma unroll
@@ -361,8 +405,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                         *cell = 0;
                         sx.fma_to(acc_a[m], gsum);
                     }
-                }
-                if constexpr (kAccB) {
+                } else {
                     const Slice<T, D> sy = st_y.lane(src);   // dout_i
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
