@@ -161,8 +161,16 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
 template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() { return sizeof(T) == 4 && D > 8 ? 3 : 4; }
 
-template <typename T, int D, int ND>
-__global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sweep_kernel(AttnArgs a)
+// elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
+template <typename T, int D, int HP> __host__ __device__ constexpr int table_row_stride_heads()
+{
+    return HP * 3 * D + ((HP * 3 * D * static_cast<int>(sizeof(T)) / 4) % 8 == 0 ? 16 / static_cast<int>(sizeof(T)) : 0);
+}
+
+// HP: heads a wavefront carries through a unit (adjacent heads HP * g .. HP * g + HP - 1).  The cRSE rows and
+// LDS addresses of a pair do not depend on the head, so two heads share that part of the work.
+template <typename T, int D, int ND, int HP>
+__global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) void attn_fwd_sweep_kernel(AttnArgs a)
 {
     // streamed keys per loop iteration: at head_dim 16 two interleaved chains hide the LDS round trips,
     // at head_dim 8 the extra registers cost more than they bring
@@ -170,21 +178,24 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
     extern __shared__ float smem[];
     const int H = a.H;
     const int HD = H * D;
-    // workgroups go to the XCDs in turn: consecutive runs of eight serve one head, so every XCD gets every head
-    const int h = (blockIdx.x / kQueues) % H;
-    // table slices of the head in the I/O type, interleaved per row
-    constexpr int kRowStride = table_row_stride<T, D>();
+    // workgroups go to the XCDs in turn: consecutive runs of eight serve one head group, so every XCD gets every head
+    const int hg = (blockIdx.x / kQueues) % (H / HP);
+    const int h = hg * HP;   // first head of the group
+    // table slices of the heads in the I/O type, interleaved per row: [head][q-side | k-side | v-side]
+    constexpr int kRowStride = table_row_stride_heads<T, D, HP>();
     T *tab = reinterpret_cast<T *>(smem);
     {
         const T *gq = static_cast<const T *>(a.table_q);
         const T *gk = static_cast<const T *>(a.table_k);
         const T *gv = static_cast<const T *>(a.table_v);
-        for (int t = threadIdx.x; t < a.total_rows * D; t += kThreads) {
-            const int r = t / D, c = t - r * D;
-            const int64_t g = static_cast<int64_t>(r) * HD + h * D + c;
-            tab[r * kRowStride + c] = gq[g];
-            tab[r * kRowStride + D + c] = gk[g];
-            tab[r * kRowStride + 2 * D + c] = gv[g];
+        for (int t = threadIdx.x; t < a.total_rows * HP * D; t += kThreads) {
+            const int r = t / (HP * D), hc = t - r * (HP * D);
+            const int hh = hc / D, c = hc - hh * D;
+            const int64_t g = static_cast<int64_t>(r) * HD + (h + hh) * D + c;
+            T *row = tab + r * kRowStride + hh * 3 * D;
+            row[c] = gq[g];
+            row[D + c] = gk[g];
+            row[2 * D + c] = gv[g];
         }
     }
     __syncthreads();   // the only workgroup barrier
@@ -196,8 +207,9 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
     const char *ws = static_cast<const char *>(a.workspace);
     const int2 *units = reinterpret_cast<const int2 *>(ws + ws_units_offset(H));
     const int total_units = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(ws + ws_total_offset(H)));
-    int *counters = static_cast<int *>(a.workspace) + h * kQueues * kCounterStride;
+    int *counters = static_cast<int *>(a.workspace) + hg * kQueues * kCounterStride;
     constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
+    constexpr uint32_t kHeadBytes = 3 * D * sizeof(T);   // one head's slices inside a row
     const uint32_t tab_addr = __builtin_amdgcn_readfirstlane(lds_address(tab));
     const uint32_t row_bytes = kRowBytes;
     float half_rows[ND], upper[ND];
@@ -242,14 +254,18 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
         const int own_pos = s0 + min(own, n_w - 1);
         const int own_row = a.n2n[own_pos];
 
-        Slice<T, D> qv;
-        float ci[ND], acc[D];
-        qv.load(gq + static_cast<int64_t>(own_row) * a.row_stride + h * D);
+        Slice<T, D> qv[HP];
+        float ci[ND], acc[HP][D], m[HP], l[HP];
+#pragma unroll
+        for (int hh = 0; hh < HP; ++hh) {
+            qv[hh].load(gq + static_cast<int64_t>(own_row) * a.row_stride + (h + hh) * D);
+#pragma unroll
+            for (int c = 0; c < D; ++c) acc[hh][c] = 0.0f;
+            m[hh] = -INFINITY;
+            l[hh] = 0.0f;
+        }
 #pragma unroll
         for (int n = 0; n < ND; ++n) ci[n] = a.n_coords[static_cast<int64_t>(own_pos) * ND + n];
-#pragma unroll
-        for (int c = 0; c < D; ++c) acc[c] = 0.0f;
-        float m = -INFINITY, l = 0.0f;
 
         // kKeys streamed keys per iteration: their loads and dependent chains interleave, which hides the
         // LDS and cache round trips a single chain would wait out one after the other
@@ -259,8 +275,8 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
 #pragma unroll
         for (int u = 0; u < kKeys; ++u) row_next[u] = a.n2n[k0 + min(u * ng + grp, n_k - 1)];
         for (int it = 0; it < steps; it += kKeys) {
-            Slice<T, D> kv[kKeys], v_in[kKeys];
-            float logit[kKeys];
+            Slice<T, D> kv[kKeys][HP], v_in[kKeys][HP];
+            float logit[kKeys][HP];
             uint32_t off[kKeys][ND];
             bool valid[kKeys];
 #pragma unroll
@@ -270,8 +286,11 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
                 const int st_pos = k0 + min(st, n_k - 1);
                 const int st_row = row_next[u];
                 row_next[u] = a.n2n[k0 + min(st + kKeys * ng, n_k - 1)];
-                kv[u].load(gk + static_cast<int64_t>(st_row) * a.row_stride + h * D);
-                v_in[u].load(gv + static_cast<int64_t>(st_row) * a.row_stride + h * D);
+#pragma unroll
+                for (int hh = 0; hh < HP; ++hh) {
+                    kv[u][hh].load(gk + static_cast<int64_t>(st_row) * a.row_stride + (h + hh) * D);
+                    v_in[u][hh].load(gv + static_cast<int64_t>(st_row) * a.row_stride + (h + hh) * D);
+                }
                 float cj[ND];
 #pragma unroll
                 for (int n = 0; n < ND; ++n) cj[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
@@ -281,80 +300,90 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D>())) void attn_fwd_sw
             }
 #pragma unroll
             for (int u = 0; u < kKeys; ++u) {
-                logit[u] = qv.dot(kv[u], 0.0f);
+#pragma unroll
+                for (int hh = 0; hh < HP; ++hh) logit[u][hh] = qv[hh].dot(kv[u][hh], 0.0f);
 #pragma unroll
                 for (int n = 0; n < ND; ++n) {
-                    Slice<T, D> tq_r, tk_r;
-                    tq_r.load_lds(off[u][n]);
-                    tk_r.load_lds(off[u][n] + D * sizeof(T));
-                    if (Slice<T, D>::kChainLogit) logit[u] = kv[u].dot(tk_r, qv.dot(tq_r, logit[u]));
-                    else logit[u] += kv[u].dot(tk_r, qv.dot(tq_r, 0.0f));
+#pragma unroll
+                    for (int hh = 0; hh < HP; ++hh) {
+                        Slice<T, D> tq_r, tk_r;
+                        tq_r.load_lds(off[u][n] + hh * kHeadBytes);
+                        tk_r.load_lds(off[u][n] + hh * kHeadBytes + D * sizeof(T));
+                        if (Slice<T, D>::kChainLogit) logit[u][hh] = kv[u][hh].dot(tk_r, qv[hh].dot(tq_r, logit[u][hh]));
+                        else logit[u][hh] += kv[u][hh].dot(tk_r, qv[hh].dot(tq_r, 0.0f));
+                    }
                 }
             }
             if (valid[0]) {   // slot 0 is the lowest key of the iteration
-                float m_new = fmaxf(m, logit[0]);
 #pragma unroll
-                for (int u = 1; u < kKeys; ++u) {
-                    logit[u] = valid[u] ? logit[u] : -INFINITY;
-                    m_new = fmaxf(m_new, logit[u]);
-                }
-                const float scale = __expf(m - m_new);   // exp(-inf) = 0 on the first key
-                l *= scale;
+                for (int hh = 0; hh < HP; ++hh) {
+                    float m_new = fmaxf(m[hh], logit[0][hh]);
 #pragma unroll
-                for (int c = 0; c < D; ++c) acc[c] *= scale;
-#pragma unroll
-                for (int u = 0; u < kKeys; ++u) {
-                    const float p = __expf(logit[u] - m_new);
-                    l += p;
-                    v_in[u].fma_to(acc, p);
-#pragma unroll
-                    for (int n = 0; n < ND; ++n) {
-                        Slice<T, D> tv_r;
-                        tv_r.load_lds(off[u][n] + 2 * D * sizeof(T));
-                        tv_r.fma_to(acc, p);
+                    for (int u = 1; u < kKeys; ++u) {
+                        logit[u][hh] = valid[u] ? logit[u][hh] : -INFINITY;
+                        m_new = fmaxf(m_new, logit[u][hh]);
                     }
+                    const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
+                    l[hh] *= scale;
+#pragma unroll
+                    for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+#pragma unroll
+                    for (int u = 0; u < kKeys; ++u) {
+                        const float p = __expf(logit[u][hh] - m_new);
+                        l[hh] += p;
+                        v_in[u][hh].fma_to(acc[hh], p);
+#pragma unroll
+                        for (int n = 0; n < ND; ++n) {
+                            Slice<T, D> tv_r;
+                            tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
+                            tv_r.fma_to(acc[hh], p);
+                        }
+                    }
+                    m[hh] = m_new;
                 }
-                m = m_new;
             }
         }
-        if (ng == 2) {
-            // the two groups saw alternate keys of the same queries: merge their softmax states
-            const float m_o = __shfl_xor(m, 32), l_o = __shfl_xor(l, 32);
-            const float m_all = fmaxf(m, m_o);
-            const float w_me = (m == -INFINITY) ? 0.0f : __expf(m - m_all);
-            const float w_ot = (m_o == -INFINITY) ? 0.0f : __expf(m_o - m_all);
-            l = l * w_me + l_o * w_ot;
 #pragma unroll
-            for (int c = 0; c < D; ++c) acc[c] = acc[c] * w_me + __shfl_xor(acc[c], 32) * w_ot;
-            m = m_all;
-        }
-        if (own_valid && grp == 0) {
-            if (blocks == 1) {
-                const float inv = 1.0f / l;
+        for (int hh = 0; hh < HP; ++hh) {
+            if (ng == 2) {
+                // the two groups saw alternate keys of the same queries: merge their softmax states
+                const float m_o = __shfl_xor(m[hh], 32), l_o = __shfl_xor(l[hh], 32);
+                const float m_all = fmaxf(m[hh], m_o);
+                const float w_me = (m[hh] == -INFINITY) ? 0.0f : __expf(m[hh] - m_all);
+                const float w_ot = (m_o == -INFINITY) ? 0.0f : __expf(m_o - m_all);
+                l[hh] = l[hh] * w_me + l_o * w_ot;
 #pragma unroll
-                for (int c = 0; c < D; ++c) acc[c] *= inv;
-                store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + h * D, acc);
-                if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h] = m;
-                if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h] = l;
-            } else {
-                float *part = a.partials + ((static_cast<int64_t>(kb) * H + h) * a.N + own_pos) * (D + 2);
+                for (int c = 0; c < D; ++c) acc[hh][c] = acc[hh][c] * w_me + __shfl_xor(acc[hh][c], 32) * w_ot;
+                m[hh] = m_all;
+            }
+            if (own_valid && grp == 0) {
+                if (blocks == 1) {
+                    const float inv = 1.0f / l[hh];
 #pragma unroll
-                for (int c = 0; c < D; ++c) part[c] = acc[c];
-                part[D] = m;
-                part[D + 1] = l;
+                    for (int c = 0; c < D; ++c) acc[hh][c] *= inv;
+                    store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + (h + hh) * D, acc[hh]);
+                    if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h + hh] = m[hh];
+                    if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h + hh] = l[hh];
+                } else {
+                    float *part = a.partials + ((static_cast<int64_t>(kb) * H + h + hh) * a.N + own_pos) * (D + 2);
+#pragma unroll
+                    for (int c = 0; c < D; ++c) part[c] = acc[hh][c];
+                    part[D] = m[hh];
+                    part[D + 1] = l[hh];
+                }
             }
         }
     }
 }
 
-template <typename T, int D, int ND>
-int launch_sweep(const AttnArgs &a, hipStream_t stream)
+template <typename T, int D, int ND, int HP>
+int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
 {
-    const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride<T, D>(), 16);
+    const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride_heads<T, D, HP>(), 16);
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
-    auto kernel = attn_fwd_sweep_kernel<T, D, ND>;
+    auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP>;
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     hipLaunchKernelGGL(generic_units_kernel, dim3(1), dim3(1024), 0, stream, a);
@@ -364,12 +393,11 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
         int v = 0;
         if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
     }
-    // a workgroup serves one head for its whole life: a multiple of H workgroups, as many per CU as
-    // registers and LDS allow
-    int per_cu = groups_per_cu<T, D>();
+    // a workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow,
+    // in whole sets of (XCDs x head groups)
+    int per_cu = HP == 1 ? groups_per_cu<T, D>() : 3;
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
-    // as many as fit the chip at once in whole sets of (XCDs x heads)
-    const int set = kQueues * a.H;
+    const int set = kQueues * (a.H / HP);
     const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
@@ -380,6 +408,16 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
         S3D_HIP_CHECK(hipGetLastError());
     }
     return S3D_OK;
+}
+
+template <typename T, int D, int ND>
+int launch_sweep(const AttnArgs &a, hipStream_t stream)
+{
+    // two heads per wavefront where the registers allow it (head_dim 8, fp16) and the heads pair up
+    if constexpr (D <= 8 && sizeof(T) == 2) {
+        if (a.H % 2 == 0) return launch_sweep_heads<T, D, ND, 2>(a, stream);
+    }
+    return launch_sweep_heads<T, D, ND, 1>(a, stream);
 }
 
 template <typename T>
