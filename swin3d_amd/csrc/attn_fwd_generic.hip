@@ -71,11 +71,19 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
         const int blocks = key_blocks(n);
         return blocks > a.max_key_tiles ? 0 : blocks * blocks;
     };
+    // window sizes are fetched eight at a time with independent loads (a dependent load per window would make
+    // this one-workgroup kernel a chain of memory round trips)
+    constexpr int kBatch = 8;
     int sum_long = 0, sum_all = 0;
-    for (int w = begin; w < end; ++w) {
-        const int n = a.w_sizes[w];
-        sum_all += units_of(n);
-        if (n > 32) sum_long += units_of(n);
+    for (int first = begin; first < end; first += kBatch) {
+        int n[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) n[i] = first + i < end ? a.w_sizes[first + i] : 0;
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            sum_all += units_of(n[i]);
+            if (n[i] > 32) sum_long += units_of(n[i]);
+        }
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int incl_long = sum_long, incl_all = sum_all;
@@ -100,14 +108,20 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
     const int before_all = incl_all + (wave > 0 ? wave_all[wave - 1] : 0) - sum_all;
     int run_long = before_long;
     int run_short = total_long + (before_all - before_long);
-    for (int w = begin; w < end; ++w) {
-        const int n = a.w_sizes[w];
-        const int blocks = key_blocks(n);
-        if (units_of(n) == 0) continue;
-        int &run = n > 32 ? run_long : run_short;
-        for (int c = 0; c < blocks; ++c)
-            for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
-        if (blocks > 1) split[atomicAdd(&split_count, 1)] = w;   // any order: the merge treats windows independently
+    for (int first = begin; first < end; first += kBatch) {
+        int sizes[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) sizes[i] = first + i < end ? a.w_sizes[first + i] : 0;
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const int n = sizes[i], w = first + i;
+            const int blocks = key_blocks(n);
+            if (units_of(n) == 0) continue;
+            int &run = n > 32 ? run_long : run_short;
+            for (int c = 0; c < blocks; ++c)
+                for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
+            if (blocks > 1) split[atomicAdd(&split_count, 1)] = w;   // any order: the merge treats windows independently
+        }
     }
     __syncthreads();
     if (threadIdx.x == 1023) {
