@@ -202,14 +202,17 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
         const T *gq = static_cast<const T *>(a.table_q);
         const T *gk = static_cast<const T *>(a.table_k);
         const T *gv = static_cast<const T *>(a.table_v);
-        for (int t = threadIdx.x; t < a.total_rows * HP * D; t += kThreads) {
-            const int r = t / (HP * D), hc = t - r * (HP * D);
-            const int hh = hc / D, c = hc - hh * D;
+        // 16-byte pieces: a (row, head) slice of a table is D * sizeof(T) / 16 of them
+        constexpr int kPieces = D * static_cast<int>(sizeof(T)) / 16;
+        constexpr int kPerPiece = 16 / static_cast<int>(sizeof(T));
+        for (int t = threadIdx.x; t < a.total_rows * HP * kPieces; t += kThreads) {
+            const int r = t / (HP * kPieces), hp = t - r * (HP * kPieces);
+            const int hh = hp / kPieces, c = (hp - hh * kPieces) * kPerPiece;
             const int64_t g = static_cast<int64_t>(r) * HD + (h + hh) * D + c;
-            T *row = tab + r * kRowStride + hh * 3 * D;
-            row[c] = gq[g];
-            row[D + c] = gk[g];
-            row[2 * D + c] = gv[g];
+            T *row = tab + r * kRowStride + hh * 3 * D + c;
+            *reinterpret_cast<uint4 *>(row) = *reinterpret_cast<const uint4 *>(gq + g);
+            *reinterpret_cast<uint4 *>(row + D) = *reinterpret_cast<const uint4 *>(gk + g);
+            *reinterpret_cast<uint4 *>(row + 2 * D) = *reinterpret_cast<const uint4 *>(gv + g);
         }
     }
     __syncthreads();   // the only workgroup barrier
