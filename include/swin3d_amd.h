@@ -220,6 +220,27 @@ int s3d_knn(int32_t K, const float *src_xyz, int64_t Ns, const float *query_xyz,
 int s3d_knn_interpolate(const int32_t *idx, const float *dist2, int32_t K, int64_t Nq, const void *src_feat,
                         int64_t Ns, int32_t C, int32_t dtype, void *out, void *stream);
 
+/*
+ * Residual add fused with LayerNorm, for the Swin block on either side of the attention operator.
+ *
+ * The reference block (Swin3D/modules/swin3d_layers.py:617-623) computes
+ *   feats = short_cut + attn(norm1(feats));  feats = feats + mlp(norm2(feats))
+ * with torch kernels (add, LayerNorm in fp32, and under autocast a cast in front of the next GEMM).  This call
+ * does, per row of C channels,
+ *   s = x + residual            (residual null: s = x)
+ *   x_out = s                   (skipped when residual or x_out is null; x_out may be x)
+ *   y = (s - mean(s)) / sqrt(var(s) + eps) * gamma + beta      (biased variance, as torch.nn.LayerNorm)
+ *
+ *   x              device [N,C] fp32 (the residual stream)
+ *   residual       device [N,C] of residual_dtype (S3D_DTYPE_F32 / S3D_DTYPE_F16), or null
+ *   gamma, beta    device [C] fp32
+ *   y              device [N,C] of y_dtype
+ * C a multiple of 4 and at most 1024; arithmetic in fp32.
+ */
+int s3d_add_layernorm(const float *x, const void *residual, int32_t residual_dtype, const float *gamma,
+                      const float *beta, float eps, float *x_out, void *y, int32_t y_dtype, int64_t N, int32_t C,
+                      void *stream);
+
 #ifdef __cplusplus
 }
 #endif

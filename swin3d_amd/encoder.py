@@ -27,6 +27,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
+from .fused_norm import add_layernorm
 from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
 from .sparse_dl.knn import KNN, KNNInterpolate, knn_query
 from .window_index import get_index01
@@ -209,8 +210,25 @@ class SwinBlock(nn.Module):
         self.mlp = nn.Sequential(nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
 
     def forward(self, feats, attn_args):
+        if self._fused_path(feats):
+            feats, pending = self.forward_fused(feats, None, attn_args)
+            return feats + pending
         feats = feats + self.attn(self.norm1(feats), attn_args)      # fp32 + fp16 promotes to fp32
         return feats + self.mlp(self.norm2(feats))
+
+    def forward_fused(self, feats, pending, attn_args):
+        """Inference under fp16 autocast: (feats, pending) stands for the residual stream feats + pending, where
+        pending is the previous block's MLP output (or None).  The residual adds and LayerNorms run as fused
+        kernels that write the normalised rows in fp16, the dtype the following GEMM reads; the block's own MLP
+        output is handed on as the new pending term instead of being added here."""
+        feats, normed = add_layernorm(feats, pending, self.norm1)
+        feats, normed = add_layernorm(feats, self.attn(normed, attn_args), self.norm2, inplace=pending is not None)
+        return feats, self.mlp(normed)
+
+    def _fused_path(self, feats):
+        return (not torch.is_grad_enabled() and feats.is_cuda and feats.dtype == torch.float32
+                and torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.float16
+                and feats.shape[1] % 4 == 0 and feats.shape[1] <= 1024)
 
 
 class Stage(nn.Module):
@@ -233,8 +251,14 @@ class Stage(nn.Module):
         args = [get_index01(voxels.coords, voxels.stride, self.window_size, local, extra, shift=s)
                 for s in (0, self.window_size // 2)]
         feats = voxels.feats
-        for i, block in enumerate(self.blocks):
-            feats = block(feats, args[i % 2])
+        if len(self.blocks) > 0 and self.blocks[0]._fused_path(feats):
+            pending = None
+            for i, block in enumerate(self.blocks):
+                feats, pending = block.forward_fused(feats, pending, args[i % 2])
+            feats = feats + pending
+        else:
+            for i, block in enumerate(self.blocks):
+                feats = block(feats, args[i % 2])
         voxels = voxels.with_feats(feats)
         if self.downsample is None:
             return voxels, voxels, signals

@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -76,6 +76,11 @@ def test_more_argument_errors_without_a_device(hip_lib):
     st = hip_lib.s3d_knn_interpolate(None, None, 3, 10, None, 10, 8, 7, None, None)
     assert st < 0 and b"dtype" in hip_lib.s3d_last_error_string()
     assert hip_lib.s3d_knn_interpolate(None, None, 3, 0, None, 10, 8, 0, None, None) == 0   # nothing to do
+    st = hip_lib.s3d_add_layernorm(None, None, 0, None, None, 1e-5, None, None, 1, 10, 66, None)
+    assert st < 0 and b"multiple of 4" in hip_lib.s3d_last_error_string()
+    st = hip_lib.s3d_add_layernorm(None, None, 0, None, None, 1e-5, None, None, 5, 10, 64, None)
+    assert st < 0 and b"y_dtype" in hip_lib.s3d_last_error_string()
+    assert hip_lib.s3d_add_layernorm(None, None, 0, None, None, 1e-5, None, None, 1, 0, 64, None) == 0
 
 
 def test_kernel_choice_is_reported(hip_lib):
