@@ -133,6 +133,14 @@ class StemConv(nn.Module):
         return voxels.with_feats(F.relu(self.norm(out.float())))
 
 
+def _fused_norm_applies(feats):
+    """Inference under fp16 autocast on an fp32 residual stream: the fused add + LayerNorm kernel can stand in for
+    torch's LayerNorm (it has no autograd)."""
+    return (not torch.is_grad_enabled() and feats.is_cuda and feats.dtype == torch.float32
+            and torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.float16
+            and feats.shape[1] % 4 == 0 and feats.shape[1] <= 1024)
+
+
 class GridKNNDownsample(nn.Module):
     """Coarse voxel = stride-2 cell; its feature = max over the K=16 nearest fine points of
     Linear(LayerNorm(feature)); its coordinate signals = those of the picked representative."""
@@ -151,9 +159,15 @@ class GridKNNDownsample(nn.Module):
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()
         idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(voxels.coords[:, 0]),
                            segment_offsets(coarse[:, 0]))
-        m, c = coarse.shape[0], voxels.feats.shape[1]
-        grouped = voxels.feats[idx.view(-1).long().clamp_(min=0)].view(m, self.k, c)
-        feats = self.linear(self.norm(grouped)).amax(dim=1)
+        # LayerNorm and Linear act on single rows, so they commute with the gather: project the Ns fine rows once
+        # instead of the K * Nq gathered copies (the reference statement, swin3d_layers.py:292-312, gathers first)
+        if _fused_norm_applies(voxels.feats):
+            _, normed = add_layernorm(voxels.feats, None, self.norm)
+        else:
+            normed = self.norm(voxels.feats)
+        projected = self.linear(normed)
+        grouped = projected[idx.view(-1).long().clamp_(min=0)].view(coarse.shape[0], self.k, projected.shape[1])
+        feats = grouped.amax(dim=1)
         return SparseVoxels(coarse, feats.float(), voxels.stride * self.factor), coarse_signals
 
 
@@ -226,9 +240,7 @@ class SwinBlock(nn.Module):
         return feats, self.mlp(normed)
 
     def _fused_path(self, feats):
-        return (not torch.is_grad_enabled() and feats.is_cuda and feats.dtype == torch.float32
-                and torch.is_autocast_enabled() and torch.get_autocast_dtype("cuda") == torch.float16
-                and feats.shape[1] % 4 == 0 and feats.shape[1] <= 1024)
+        return _fused_norm_applies(feats)
 
 
 class Stage(nn.Module):
