@@ -82,6 +82,39 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
     _check(oracle_lib, case, dtype)
 
 
+def boundary_size_case(oracle_lib, heads, dim, seed=41):
+    """One window per size in 1, 16, 31..33, 63..65, 127..129, 192, 193 voxels (window 7): the sizes at which the
+    kernels change their lane mapping (two 32-lane groups up to 32 voxels) and split a window into chunks of 64
+    queries and blocks of 64 (sweep kernel) or 32 (MFMA kernel) keys."""
+    ws, quant = 7, 4
+    sizes = [1, 16, 31, 32, 33, 63, 64, 65, 127, 128, 129, 192, 193]
+    rng = np.random.default_rng(seed)
+    cells = np.stack(np.meshgrid(np.arange(7), np.arange(7), np.arange(7), indexing="ij"), -1).reshape(-1, 3)
+    rows = []
+    for wi, n in enumerate(sizes):
+        pick = cells[rng.permutation(343)[:n]]
+        rows.append(np.concatenate([np.zeros((n, 1), np.int64), pick + np.array([7 * wi, 0, 0])], 1))
+    coords = np.concatenate(rows).astype(np.int32)
+    coords = coords[rng.permutation(coords.shape[0])]
+    n = coords.shape[0]
+    frac = rng.random((n, 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (n, 6)).astype(np.float32)
+    case = make_attn_case(oracle_lib, seed=seed, n=n, ws=ws, quant=quant, heads=heads, dim=dim, extent=(12, 12, 6))
+    case.coords = coords
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
+    assert sorted(case.index["w_sizes"].tolist()) == sizes
+    return case
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("heads,dim", [(2, 8), (3, 8), (2, 16)])
+def test_window_sizes_at_the_kernel_boundaries(oracle_lib, hip_lib, dtype, heads, dim):
+    case = boundary_size_case(oracle_lib, heads, dim)
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
 def test_single_voxel_windows_and_one_head(oracle_lib, hip_lib):
     coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
     case = make_attn_case(oracle_lib, seed=34, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")

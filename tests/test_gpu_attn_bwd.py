@@ -94,6 +94,19 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("heads,dim", [(2, 8), (2, 16)])
+def test_window_sizes_at_the_kernel_boundaries(oracle_lib, hip_lib, dtype, heads, dim):
+    """Windows of exactly 1, 16, 31..33, 63..65, 127..129, 192 and 193 voxels: where the sweeps change their lane
+    mapping and start splitting a window into chunks of 64 owned elements."""
+    from test_gpu_attn import boundary_size_case
+    case = boundary_size_case(oracle_lib, heads, dim, seed=71)
+    if dtype == torch.float16:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+    _check(oracle_lib, case, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("ws,quant,heads,dim,cRSE", [
     (3, 4, 4, 8, "XYZ_RGB_NORM"),     # small tables
     (4, 8, 3, 8, "XYZ_RGB_NORM"),     # quant 8: 576 table rows per head, nine 64-row register blocks
