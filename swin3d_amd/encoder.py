@@ -189,27 +189,49 @@ class WindowAttention(nn.Module):
                 setattr(self, f"{kind}_{name}_table", table)
         self.qkv = nn.Linear(dim, dim * 3)
         self.proj = nn.Linear(dim, dim)
+        self._cache = None   # inference-time copies of the scaled projection and the flat tables
 
     def _flat_table(self, kind):
         names = ("xyz", "rgb", "norm")[: crse_num_axes(self.cRSE) // 3]
         return torch.cat([getattr(self, f"{kind}_{n}_table").reshape(-1) for n in names])
 
-    def forward(self, feats, attn_args):
-        n = feats.shape[0]
-        _, _, m2w, w_sizes, w2n, n2n, w2m, n_coords = attn_args
-        # q scale folded into the projection (a C x C multiply instead of an N x C one); q, k, v stay
-        # slices of the [N, 3C] projection output, which the attention kernels read in place
+    def _prepared(self):
+        """(qkv weight with the q scale folded in, its bias, the three flat tables).  Without autograd (inference)
+        they are built once per parameter version, in the autocast dtype when autocast is on, instead of on every
+        call: the scaling, three concatenations and the casts are a dozen small kernels per block otherwise."""
+        caching = not torch.is_grad_enabled()
+        dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else self.qkv.weight.dtype
+        names = ("xyz", "rgb", "norm")[: crse_num_axes(self.cRSE) // 3]
+        params = [self.qkv.weight, self.qkv.bias] + [getattr(self, f"{k}_{n}_table") for k in ("query", "key", "value")
+                                                     for n in names]
+        key = (dtype,) + tuple((p.data_ptr(), p._version) for p in params if p is not None)
+        if caching and self._cache is not None and self._cache[0] == key:
+            return self._cache[1]
+        # q scale folded into the projection (a C x C multiply instead of an N x C one)
         scale = torch.ones(3 * self.dim, dtype=self.qkv.weight.dtype, device=self.qkv.weight.device)
         scale[: self.dim] = self.scale
+        weight = self.qkv.weight * scale.unsqueeze(1)
         bias = None if self.qkv.bias is None else self.qkv.bias * scale
-        qkv = F.linear(feats, self.qkv.weight * scale.unsqueeze(1), bias).view(n, 3, self.num_heads, self.head_dim)
+        tables = [self._flat_table(kind) for kind in ("query", "key", "value")]
+        if caching:
+            weight, tables = weight.to(dtype), [t.to(dtype) for t in tables]
+            bias = None if bias is None else bias.to(dtype)
+            self._cache = (key, (weight, bias, tables))
+        return weight, bias, tables
+
+    def forward(self, feats, attn_args):
+        n = feats.shape[0]
+        _, _, m2w, w_sizes, w2n, n2n, w2m, n_coords = attn_args[:8]
+        weight, bias, tables = self._prepared()
+        # q, k, v stay slices of the [N, 3C] projection output, which the attention kernels read in place
+        qkv = F.linear(feats, weight, bias).view(n, 3, self.num_heads, self.head_dim)
         query, key, value = qkv[:, 0], qkv[:, 1], qkv[:, 2]
-        n_crse = scale_crse_coords(n_coords, self.quant_size, self.cRSE)
+        # the scaled signals of the index set, when the caller prepared them once for all blocks that share it
+        n_crse = attn_args[8] if len(attn_args) > 8 else scale_crse_coords(n_coords, self.quant_size, self.cRSE)
         precision = (PrecisionMode.HALF_NONE, PrecisionMode.HALF_FORWARD, PrecisionMode.HALF_ALL)[self.fp16_mode]
         out = SelfAttnAIOFunction.apply(
-            query, key, value, self._flat_table("query"), self._flat_table("key"), self._flat_table("value"),
-            self.table_sizes, [m2w, w_sizes, w2m, w2n, n2n, n_crse], PosEmb.SEPARATE, TableDims.D0,
-            IndexMode.INDIRECT, precision)
+            query, key, value, *tables, self.table_sizes, [m2w, w_sizes, w2m, w2n, n2n, n_crse], PosEmb.SEPARATE,
+            TableDims.D0, IndexMode.INDIRECT, precision)
         out = out.reshape(n, self.dim)
         return self.proj(out if torch.is_autocast_enabled() else out.to(feats.dtype))
 
@@ -262,6 +284,10 @@ class Stage(nn.Module):
         extra = signals[:, 4:].float()
         args = [get_index01(voxels.coords, voxels.stride, self.window_size, local, extra, shift=s)
                 for s in (0, self.window_size // 2)]
+        if len(self.blocks) > 0:
+            # the quantiser scaling of the signals is the same for every block of the stage: once per index set
+            attn = self.blocks[0].attn
+            args = [tuple(a) + (scale_crse_coords(a[7], attn.quant_size, attn.cRSE),) for a in args]
         feats = voxels.feats
         if len(self.blocks) > 0 and self.blocks[0]._fused_path(feats):
             pending = None
