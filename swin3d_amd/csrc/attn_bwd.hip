@@ -122,7 +122,7 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
     part[threadIdx.x] = sum;
     __syncthreads();
     for (int off = 1; off < 1024; off <<= 1) {
-        const int add = threadIdx.x >= off ? part[threadIdx.x - off] : 0;
+        const int add = static_cast<int>(threadIdx.x) >= off ? part[threadIdx.x - off] : 0;
         __syncthreads();
         part[threadIdx.x] += add;
         __syncthreads();

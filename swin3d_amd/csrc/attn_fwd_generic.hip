@@ -25,7 +25,6 @@ namespace {
 using namespace sweep;
 
 constexpr int kThreads = 256;
-constexpr int kWavesPerGroup = kThreads / 64;
 constexpr int kChunk = 64;   // queries per unit = lanes of a wavefront
 // key blocks a window of n voxels is split into (units stream at most kChunk keys), and their even size
 __host__ __device__ inline int key_blocks(int n) { return (n + kChunk - 1) / kChunk; }
@@ -97,7 +96,7 @@ __global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
         int v_long = wave_long[threadIdx.x], v_all = wave_all[threadIdx.x];
         for (int off = 1; off < 16; off <<= 1) {
             const int up_long = __shfl_up(v_long, off), up_all = __shfl_up(v_all, off);
-            if (threadIdx.x >= off) { v_long += up_long; v_all += up_all; }
+            if (static_cast<int>(threadIdx.x) >= off) { v_long += up_long; v_all += up_all; }
         }
         wave_long[threadIdx.x] = v_long;
         wave_all[threadIdx.x] = v_all;
