@@ -25,109 +25,181 @@ namespace {
 using namespace sweep;
 
 constexpr int kThreads = 256;
-constexpr int kChunk = 64;   // queries per unit = lanes of a wavefront
+constexpr int kChunk = 64;   // slots per unit at most = lanes of a wavefront
+constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
 // key blocks a window of n voxels is split into (units stream at most kChunk keys), and their even size
 __host__ __device__ inline int key_blocks(int n) { return (n + kChunk - 1) / kChunk; }
 __host__ __device__ inline int key_block_size(int n) { const int b = key_blocks(n); return (n + b - 1) / b; }
 
-// byte offsets inside the workspace: the queue counters, the unit count, the unit descriptors, the partial results
+// byte offsets inside the workspace: the queue counters, the totals (units, split windows, slots), the first
+// entry of every unit, the sorted window entries, the placement notes and per-workgroup bin totals of the list
+// builder, the list of split windows, the partial results
+__host__ __device__ inline size_t ws_round(size_t bytes) { return (bytes + 255) / 256 * 256; }
 __host__ __device__ inline size_t ws_total_offset(int H) { return sizeof(int32_t) * static_cast<size_t>(H) * kQueues * kCounterStride; }
 __host__ __device__ inline size_t ws_units_offset(int H) { return ws_total_offset(H) + 256; }
-__host__ __device__ inline size_t ws_max_units(int64_t W, int64_t N, int max_blocks)
+// a voxel of a window with b key blocks takes b slots; a unit is at least 16 slots
+__host__ __device__ inline size_t ws_max_units(int64_t N, int max_blocks)
 {
-    return (static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / kChunk) * max_blocks;
+    return static_cast<size_t>(N > 0 ? N : 0) * max_blocks / (kChunk / 4) + 4;
 }
-// list of the windows that are split along their keys (their count sits next to the unit count)
+__host__ __device__ inline size_t ws_entries_offset(int H, int64_t N, int max_blocks)
+{
+    return ws_units_offset(H) + ws_round(sizeof(int32_t) * ws_max_units(N, max_blocks));
+}
+__host__ __device__ inline size_t ws_place_offset(int H, int64_t W, int64_t N, int max_blocks)
+{
+    return ws_entries_offset(H, N, max_blocks) + ws_round(sizeof(int4) * (static_cast<size_t>(W > 0 ? W : 0) + kChunk));
+}
+__host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N, int max_blocks)
+{
+    return ws_place_offset(H, W, N, max_blocks) + ws_round(sizeof(int2) * static_cast<size_t>(W > 0 ? W : 1));
+}
 __host__ __device__ inline size_t ws_split_offset(int H, int64_t W, int64_t N, int max_blocks)
 {
-    return ws_units_offset(H) + (sizeof(int2) * ws_max_units(W, N, max_blocks) + 255) / 256 * 256;
+    return ws_bins_offset(H, W, N, max_blocks) + ws_round(sizeof(unsigned long long) * kListGroups * (kChunk + 1));
 }
 __host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
 {
-    return ws_split_offset(H, W, N, max_blocks) + (sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1) + 255) / 256 * 256;
+    return ws_split_offset(H, W, N, max_blocks) + ws_round(sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1));
 }
 
-// Unit list of the launch: one descriptor (window, query chunk | key block << 16) per unit, the unit count,
-// and the queue counters at zero; one workgroup.  A unit is 64 queries of a window against one block of at
-// most 64 of its keys: the longest unit bounds the tail of the launch, so windows of more than 64 voxels are
-// split along the keys as well and leave partial results that a second kernel combines.  Units of windows
-// with more than 32 voxels (33 to 64 steps) come first, then the short ones (at most 16 steps), each class in
-// window order: the launch ends on short units.  Windows beyond the caller's size bound get no units.
-__global__ __launch_bounds__(1024) void generic_units_kernel(AttnArgs a)
+// How the slots of a launch (sorted by steps, longest first) are cut into units.  A unit is one pass of a
+// wavefront: 64 slots, or 32 slots whose lanes l and l + 32 share a query and take alternate keys (half the
+// steps), or 16 slots in four such groups (a quarter).  The launch ends when the last wavefront ends, so the
+// last slots go into the finer units: about two 16-slot units and one 32-slot unit per wavefront of a head
+// group (`waves`), everything before them into 64-slot units.
+struct UnitPlan {
+    int units[3];   // units of 64, 32 and 16 slots, in this order along the slots
+    __host__ __device__ int first_slot(int g) const { return g == 0 ? 0 : g == 1 ? units[0] * kChunk : units[0] * kChunk + units[1] * (kChunk / 2); }
+    __host__ __device__ int first_unit(int g) const { return g == 0 ? 0 : g == 1 ? units[0] : units[0] + units[1]; }
+};
+__host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 {
-    __shared__ int wave_long[16], wave_all[16];
-    __shared__ int split_count;
-    if (threadIdx.x == 0) split_count = 0;
+    const int fine = 32 * (waves > 0 ? waves : 1);   // slots of each finer kind
+    const int in_c = total_slots < fine ? total_slots : fine;
+    const int in_b = total_slots - in_c < fine ? total_slots - in_c : fine;
+    UnitPlan plan;
+    plan.units[0] = (total_slots - in_c - in_b + kChunk - 1) / kChunk;
+    const int left_b = total_slots - plan.units[0] * kChunk;            // may be negative by rounding
+    const int take_b = left_b < 0 ? 0 : (left_b < in_b ? left_b : in_b);
+    plan.units[1] = (take_b + kChunk / 2 - 1) / (kChunk / 2);
+    const int left_c = total_slots - plan.units[0] * kChunk - plan.units[1] * (kChunk / 2);
+    plan.units[2] = left_c <= 0 ? 0 : (left_c + kChunk / 4 - 1) / (kChunk / 4);
+    return plan;
+}
+
+// Work list of the launch, built by two small kernels.  A voxel of a window that is split into b key blocks
+// (b = 1 up to 64 voxels) takes b slots, one per key block, and a slot streams the block's keys: at most 64
+// steps.  The windows are sorted by that step count, longest first (a counting sort over the 64 possible
+// counts), their slots laid out back to back in that order - [window][key block][voxel] - and cut into units,
+// so a wavefront's lanes carry queries of several windows when the windows are small, every lane of a unit
+// runs (almost) the same number of steps, and the launch ends on its shortest units.
+//
+// generic_count_kernel: every workgroup takes a run of windows; a window takes a place in the workgroup's bin
+// of its step count - its rank there and the slots before it (one 64-bit LDS atomic returns both, so the two
+// orders agree; the order inside a bin does not affect results) - and the workgroup leaves its bin totals.
+__global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
+{
+    __shared__ unsigned long long bin[kChunk + 1];   // per step count: windows << 32 | slots
+    if (threadIdx.x <= kChunk) bin[threadIdx.x] = 0;
+    __syncthreads();
+    char *ws = static_cast<char *>(a.workspace);
+    int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
+    int2 *place = reinterpret_cast<int2 *>(ws + ws_place_offset(a.H, a.W, a.N, a.max_key_tiles));
+    unsigned long long *group_bins =
+        reinterpret_cast<unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N, a.max_key_tiles));
+    const int W = static_cast<int>(a.W);
+    const int per = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
+    for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
+        const int n = a.w_sizes[w];
+        const int blocks = key_blocks(n);
+        int2 got = make_int2(-1, 0);
+        if (n > 0 && blocks <= a.max_key_tiles) {
+            const unsigned long long before =
+                atomicAdd(&bin[key_block_size(n)], (1ull << 32) | static_cast<unsigned>(n * blocks));
+            got = make_int2(static_cast<int>(before >> 32), static_cast<int>(before & 0xffffffffu));
+        }
+        place[w] = got;
+    }
+    __syncthreads();
+    if (threadIdx.x <= kChunk) group_bins[blockIdx.x * (kChunk + 1) + threadIdx.x] = bin[threadIdx.x];
+    if (blockIdx.x == 0 && threadIdx.x == 0) total[1] = 0;   // split windows, counted by the second kernel
+}
+
+// generic_place_kernel (same grid): bins in descending step order, workgroups in order inside a bin.  Writes one
+// entry (first slot, voxels, first sorted position, steps) per window in sorted order, the entry that holds
+// the first slot of every unit, the list of split windows for the merge, the totals, and the queue counters
+// at zero.  Windows beyond the caller's size bound get no slots.
+__global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
+{
+    __shared__ int bin_entry[kChunk + 1], bin_slot[kChunk + 1];
+    __shared__ int sums[2];
     char *ws = static_cast<char *>(a.workspace);
     int *counters = reinterpret_cast<int *>(ws);
     int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
-    int2 *units = reinterpret_cast<int2 *>(ws + ws_units_offset(a.H));
+    int *unit_first = reinterpret_cast<int *>(ws + ws_units_offset(a.H));
+    int4 *entries = reinterpret_cast<int4 *>(ws + ws_entries_offset(a.H, a.N, a.max_key_tiles));
+    const int2 *place = reinterpret_cast<const int2 *>(ws + ws_place_offset(a.H, a.W, a.N, a.max_key_tiles));
+    const unsigned long long *group_bins =
+        reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N, a.max_key_tiles));
     int *split = reinterpret_cast<int *>(ws + ws_split_offset(a.H, a.W, a.N, a.max_key_tiles));
+    // lane l of the first wavefront holds the bin of 64 - l steps: the launch's total, and what the
+    // workgroups before this one put there
+    if (threadIdx.x < kChunk) {
+        const int lane = threadIdx.x, steps = kChunk - lane;
+        unsigned long long all = 0, before = 0;
+#pragma unroll 8
+        for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
+            const unsigned long long v = group_bins[g * (kChunk + 1) + steps];
+            all += v;
+            before += g < static_cast<int>(blockIdx.x) ? v : 0;
+        }
+        const int cnt = static_cast<int>(all >> 32), slots = static_cast<int>(all & 0xffffffffu);
+        int incl_c = cnt, incl_s = slots;
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up_c = __shfl_up(incl_c, off), up_s = __shfl_up(incl_s, off);
+            if (lane >= off) { incl_c += up_c; incl_s += up_s; }
+        }
+        bin_entry[steps] = incl_c - cnt + static_cast<int>(before >> 32);
+        bin_slot[steps] = incl_s - slots + static_cast<int>(before & 0xffffffffu);
+        if (lane == kChunk - 1) { sums[0] = incl_c; sums[1] = incl_s; }
+    }
+    __syncthreads();
+    const int total_entries = sums[0], total_slots = sums[1];
+    const UnitPlan plan = plan_units(total_slots, a.target_items);
     const int W = static_cast<int>(a.W);
-    const int per = (W + 1023) / 1024;
-    const int begin = threadIdx.x * per, end = min(begin + per, W);
-    auto units_of = [&](int n) {
-        const int blocks = key_blocks(n);
-        return blocks > a.max_key_tiles ? 0 : blocks * blocks;
-    };
-    // window sizes are fetched eight at a time with independent loads (a dependent load per window would make
-    // this one-workgroup kernel a chain of memory round trips)
-    constexpr int kBatch = 8;
-    int sum_long = 0, sum_all = 0;
-    for (int first = begin; first < end; first += kBatch) {
-        int n[kBatch];
+    const int per = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
+    for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
+        const int2 got = place[w];
+        if (got.x < 0) continue;
+        const int n = a.w_sizes[w];
+        const int blocks = key_blocks(n), steps = key_block_size(n);
+        const int e = bin_entry[steps] + got.x;
+        const int s = bin_slot[steps] + got.y;
+        entries[e] = make_int4(s, n, a.w2n[w], steps);
+        // the units whose first slot is one of this window's
+        const int s_end = s + n * blocks;
 #pragma unroll
-        for (int i = 0; i < kBatch; ++i) n[i] = first + i < end ? a.w_sizes[first + i] : 0;
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            sum_all += units_of(n[i]);
-            if (n[i] > 32) sum_long += units_of(n[i]);
+        for (int g = 0; g < 3; ++g) {
+            const int size = kChunk >> g, from = plan.first_slot(g), count = plan.units[g];
+            int v = s <= from ? 0 : (s - from + size - 1) / size;
+            for (; v < count && from + v * size < s_end; ++v) unit_first[plan.first_unit(g) + v] = e;
         }
+        if (blocks > 1) split[atomicAdd(total + 1, 1)] = w;   // any order: the merge treats windows independently
     }
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int incl_long = sum_long, incl_all = sum_all;
-    for (int off = 1; off < 64; off <<= 1) {
-        const int up_long = __shfl_up(incl_long, off), up_all = __shfl_up(incl_all, off);
-        if (lane >= off) { incl_long += up_long; incl_all += up_all; }
-    }
-    if (lane == 63) { wave_long[wave] = incl_long; wave_all[wave] = incl_all; }
-    __syncthreads();
-    if (threadIdx.x < 16) {
-        int v_long = wave_long[threadIdx.x], v_all = wave_all[threadIdx.x];
-        for (int off = 1; off < 16; off <<= 1) {
-            const int up_long = __shfl_up(v_long, off), up_all = __shfl_up(v_all, off);
-            if (static_cast<int>(threadIdx.x) >= off) { v_long += up_long; v_all += up_all; }
+    if (blockIdx.x == 0) {
+        // a wavefront reads 64 entries from a unit's first one: pad the list with entries no slot belongs to
+        if (threadIdx.x < kChunk) entries[total_entries + threadIdx.x] = make_int4(total_slots, 1, 0, 1);
+        if (threadIdx.x == 0) {
+            total[0] = plan.units[0] + plan.units[1] + plan.units[2];
+            total[2] = total_slots;
+            total[3] = plan.units[0];
+            total[4] = plan.units[1];
         }
-        wave_long[threadIdx.x] = v_long;
-        wave_all[threadIdx.x] = v_all;
+        for (int t = threadIdx.x; t < a.H * kQueues; t += kListThreads) counters[t * kCounterStride] = 0;
     }
-    __syncthreads();
-    const int total_long = wave_long[15];
-    const int before_long = incl_long + (wave > 0 ? wave_long[wave - 1] : 0) - sum_long;
-    const int before_all = incl_all + (wave > 0 ? wave_all[wave - 1] : 0) - sum_all;
-    int run_long = before_long;
-    int run_short = total_long + (before_all - before_long);
-    for (int first = begin; first < end; first += kBatch) {
-        int sizes[kBatch];
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) sizes[i] = first + i < end ? a.w_sizes[first + i] : 0;
-#pragma unroll
-        for (int i = 0; i < kBatch; ++i) {
-            const int n = sizes[i], w = first + i;
-            const int blocks = key_blocks(n);
-            if (units_of(n) == 0) continue;
-            int &run = n > 32 ? run_long : run_short;
-            for (int c = 0; c < blocks; ++c)
-                for (int kb = 0; kb < blocks; ++kb) units[run++] = make_int2(w, c | (kb << 16));
-            if (blocks > 1) split[atomicAdd(&split_count, 1)] = w;   // any order: the merge treats windows independently
-        }
-    }
-    __syncthreads();
-    if (threadIdx.x == 1023) {
-        total[0] = wave_all[15];
-        total[1] = split_count;
-    }
-    for (int t = threadIdx.x; t < a.H * kQueues; t += 1024) counters[t * kCounterStride] = 0;
 }
 
 // Windows of more than 64 voxels: combine the per-key-block partial results (unnormalised output, running
@@ -221,8 +293,14 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
     const T *gk = static_cast<const T *>(a.k);
     const T *gv = static_cast<const T *>(a.v);
     const char *ws = static_cast<const char *>(a.workspace);
-    const int2 *units = reinterpret_cast<const int2 *>(ws + ws_units_offset(H));
-    const int total_units = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int *>(ws + ws_total_offset(H)));
+    const int *unit_first = reinterpret_cast<const int *>(ws + ws_units_offset(H));
+    const int4 *entries = reinterpret_cast<const int4 *>(ws + ws_entries_offset(H, a.N, a.max_key_tiles));
+    const int total_units = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[0]);
+    const int total_slots = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[2]);
+    UnitPlan plan;
+    plan.units[0] = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[3]);
+    plan.units[1] = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[4]);
+    plan.units[2] = 0;
     int *counters = static_cast<int *>(a.workspace) + hg * kQueues * kCounterStride;
     constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
     constexpr uint32_t kHeadBytes = 3 * D * sizeof(T);   // one head's slices inside a row
@@ -240,7 +318,7 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
 
     int queue = xcd_id() % kQueues;
     int tried = 0;       // queues found empty so far
-    int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
+    int drawn = 0;       // ticket of the next unit
     if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
     for (;;) {
         int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
@@ -250,25 +328,34 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
             unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
         }
         if (unit >= total_units) break;
-        if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
-        const int2 desc = units[unit];
-        const int w = __builtin_amdgcn_readfirstlane(desc.x);
-        const int chunk = __builtin_amdgcn_readfirstlane(desc.y) & 0xffff;
-        const int kb = __builtin_amdgcn_readfirstlane(desc.y) >> 16;
-        const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
-        const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
-        // the unit's keys: block kb of the window's even split into blocks of at most 64
+        // the lane's slot: a query of a window and one block of at most 64 of the window's keys.  The unit's 64
+        // slots lie in at most 64 consecutive entries from the unit's first one; each lane reads one entry and
+        // finds its own (the last entry that starts at or before its slot) by a search across the lanes.
+        const int first = __builtin_amdgcn_readfirstlane(unit_first[unit]);
+        const int4 seen = entries[first + lane];
+        // the unit's kind: 2^gshift groups of lanes that share queries and take alternate keys
+        const int gshift = unit < plan.first_unit(1) ? 0 : unit < plan.first_unit(2) ? 1 : 2;
+        const int gs = kChunk >> gshift;
+        const int grp = lane >> (6 - gshift);
+        const int slot_raw = plan.first_slot(gshift) + (unit - plan.first_unit(gshift)) * gs + (lane & (gs - 1));
+        const bool own_valid = slot_raw < total_slots;
+        const int slot = min(slot_raw, total_slots - 1);   // lanes past the end repeat the last slot
+        int at = 0;
+#pragma unroll
+        for (int half = 32; half > 0; half >>= 1)
+            if (__shfl(seen.x, at + half) <= slot) at += half;
+        const int n_w = __shfl(seen.y, at), s0 = __shfl(seen.z, at), block_size = __shfl(seen.w, at);
+        const int in_window = slot - __shfl(seen.x, at);               // [key block][voxel]
+        // entries are sorted by steps, longest first
+        const int max_steps = (__builtin_amdgcn_readfirstlane(seen.w) + (1 << gshift) - 1) >> gshift;
         const int blocks = key_blocks(n_w);
-        const int k_begin = kb * key_block_size(n_w);
-        const int n_k = min(key_block_size(n_w), n_w - k_begin);
-        // a window of at most 32 voxels streams two keys per step (lanes l and l + 32 own the same query)
-        const int gs = n_w <= 32 ? 32 : 64;
-        const int ng = 64 / gs;
-        const int grp = lane / gs;
-        const int own = chunk * kChunk + (lane - grp * gs);
-        const bool own_valid = own < n_w;
-        const int own_pos = s0 + min(own, n_w - 1);
+        const int kb = blocks == 1 ? 0 : in_window / n_w;
+        const int own_pos = s0 + (in_window - kb * n_w);
         const int own_row = a.n2n[own_pos];
+        // the slot's keys: block kb of the window's even split into blocks of at most 64
+        const int k_begin = kb * block_size;
+        const int n_k = min(block_size, n_w - k_begin);
+        const int k0 = s0 + k_begin;
 
         Slice<T, D> qv[HP];
         float ci[ND], acc[HP][D], m[HP], l[HP];
@@ -285,23 +372,24 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
 
         // kKeys streamed keys per iteration: their loads and dependent chains interleave, which hides the
         // LDS and cache round trips a single chain would wait out one after the other
-        const int steps = (n_k + ng - 1) / ng;
-        const int k0 = s0 + k_begin;
         int row_next[kKeys];
 #pragma unroll
-        for (int u = 0; u < kKeys; ++u) row_next[u] = a.n2n[k0 + min(u * ng + grp, n_k - 1)];
-        for (int it = 0; it < steps; it += kKeys) {
+        for (int u = 0; u < kKeys; ++u) row_next[u] = a.n2n[k0 + min((u << gshift) + grp, n_k - 1)];
+        for (int it = 0; it < max_steps; it += kKeys) {
+            // the next unit's ticket is drawn during the last iteration: the atomic's round trip overlaps that
+            // work, and a unit is not held back (out of reach of idle wavefronts) for longer than one step
+            if (it + kKeys >= max_steps && lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
             Slice<T, D> kv[kKeys][HP], v_in[kKeys][HP];
             float logit[kKeys][HP];
             uint32_t off[kKeys][ND];
             bool valid[kKeys];
 #pragma unroll
             for (int u = 0; u < kKeys; ++u) {
-                const int st = (it + u) * ng + grp;
+                const int st = ((it + u) << gshift) + grp;
                 valid[u] = st < n_k;
                 const int st_pos = k0 + min(st, n_k - 1);
                 const int st_row = row_next[u];
-                row_next[u] = a.n2n[k0 + min(st + kKeys * ng, n_k - 1)];
+                row_next[u] = a.n2n[k0 + min(st + (kKeys << gshift), n_k - 1)];
 #pragma unroll
                 for (int hh = 0; hh < HP; ++hh) {
                     kv[u][hh].load(gk + static_cast<int64_t>(st_row) * a.row_stride + (h + hh) * D);
@@ -330,7 +418,7 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
                     }
                 }
             }
-            if (valid[0]) {   // slot 0 is the lowest key of the iteration
+            if (valid[0]) {   // the lowest key of the iteration; lanes whose block has ended sit the step out
 #pragma unroll
                 for (int hh = 0; hh < HP; ++hh) {
                     float m_new = fmaxf(m[hh], logit[0][hh]);
@@ -361,15 +449,15 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
         }
 #pragma unroll
         for (int hh = 0; hh < HP; ++hh) {
-            if (ng == 2) {
-                // the two groups saw alternate keys of the same queries: merge their softmax states
-                const float m_o = __shfl_xor(m[hh], 32), l_o = __shfl_xor(l[hh], 32);
+            // groups saw alternate keys of the same queries: merge their softmax states
+            for (int other = 32; other >= gs; other >>= 1) {
+                const float m_o = __shfl_xor(m[hh], other), l_o = __shfl_xor(l[hh], other);
                 const float m_all = fmaxf(m[hh], m_o);
                 const float w_me = (m[hh] == -INFINITY) ? 0.0f : __expf(m[hh] - m_all);
                 const float w_ot = (m_o == -INFINITY) ? 0.0f : __expf(m_o - m_all);
                 l[hh] = l[hh] * w_me + l_o * w_ot;
 #pragma unroll
-                for (int c = 0; c < D; ++c) acc[hh][c] = acc[hh][c] * w_me + __shfl_xor(acc[hh][c], 32) * w_ot;
+                for (int c = 0; c < D; ++c) acc[hh][c] = acc[hh][c] * w_me + __shfl_xor(acc[hh][c], other) * w_ot;
                 m[hh] = m_all;
             }
             if (own_valid && grp == 0) {
@@ -399,11 +487,12 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
+    if (a.N * a.max_key_tiles > INT32_MAX - kChunk)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %lld voxels x %d key blocks exceed the 32-bit slot count",
+                    (long long)a.N, a.max_key_tiles);
     auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP>;
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    hipLaunchKernelGGL(generic_units_kernel, dim3(1), dim3(1024), 0, stream, a);
-    S3D_HIP_CHECK(hipGetLastError());
     int device = 0, cus = 256;
     if (hipGetDevice(&device) == hipSuccess) {
         int v = 0;
@@ -415,10 +504,17 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
     const int set = kQueues * (a.H / HP);
     const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, a);
+    AttnArgs b = a;
+    b.target_items = sets * kQueues * (kThreads / 64);   // wavefronts that serve one head group
+    const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
+    const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
+    hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+    hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
     S3D_HIP_CHECK(hipGetLastError());
     if (a.max_key_tiles > 1) {
-        const int64_t want = a.W < 1024 ? a.W : 1024;
+        const int64_t want = a.W < 256 ? a.W : 256;
         hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>(want > 0 ? want : 1)), dim3(256),
                            0, stream, a);
         S3D_HIP_CHECK(hipGetLastError());
