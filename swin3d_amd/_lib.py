@@ -25,7 +25,7 @@ _i64 = ctypes.c_int64
 SIGNATURES = {
     "s3d_version": (ctypes.c_int, []),
     "s3d_last_error_string": (ctypes.c_char_p, []),
-    "s3d_attn_fwd_uses_mfma": (ctypes.c_int, [_vp, _i32, _i32, _i32, _i32]),
+    "s3d_attn_fwd_uses_mfma": (ctypes.c_int, [_vp, _i32, _i32, _i32, _i32, _i64, _i64]),
     "s3d_attn_fwd_workspace_bytes": (ctypes.c_size_t, [_vp, _i32, _i32, _i32, _i64, _i64, _i32]),
     "s3d_attn_fwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
                      [_i64, _i32, _i32, _i64, _i32, _i64, _i32, _i32, _vp, ctypes.c_size_t, _vp]),

@@ -67,14 +67,16 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
-    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype)
+    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype, int64_t N, int64_t W)
 {
     using namespace s3d;
-    if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1) return 0;
+    if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1 || N < 0 || W < 0) return 0;
     AttnArgs a{};
     a.H = H;
     a.D = D;
     a.nd = nd;
+    a.N = N;
+    a.W = W;
     int64_t total = 0;
     for (int n = 0; n < nd; ++n) total += table_sizes[n];
     if (fill_axes(a, table_sizes, nd, total) != S3D_OK) return 0;

@@ -1,14 +1,14 @@
 // Sparse-voxel windowed self-attention forward with cRSE tables (gfx950): sweep kernel.
 //
 // Covers every dtype / shape the library accepts on the vector ALU (fp32 arithmetic; fp16 inputs enter through
-// packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one head for its
-// whole life and keeps that head's slices of the three relative-signal tables in LDS (loaded once, not once per
-// window).  A wavefront draws units from the head's work queues; a unit is 64 queries of a window against a
-// block of at most 64 of its keys.  Lane = query: q_i, the running maximum, sum and output stay in the lane's
-// registers while the keys stream through the wavefront one per step (two per step, in two 32-lane groups,
-// when the window has at most 32 voxels), so there is no cross-lane reduction, no atomic on data and no
-// O(pairs) index array; the result is deterministic.  Windows of more than 64 voxels leave one partial result
-// per key block, combined by generic_merge_kernel.
+// packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one head (or two)
+// for its whole life and keeps the slices of the three relative-signal tables in LDS (loaded once, not once
+// per window).  Lane = slot = one query against a block of at most 64 keys of its window: q_i, the running
+// maximum, sum and output stay in the lane's registers while the lane streams its own window's keys, one per
+// step, so there is no cross-lane reduction, no atomic on data and no O(pairs) index array; the result is
+// deterministic.  The slots of all windows, sorted by step count, are packed into units of 64 (the lanes of a
+// wavefront carry queries of several small windows); wavefronts draw units from the head's work queues.
+// Windows of more than 64 voxels leave one partial result per key block, combined by generic_merge_kernel.
 //
 // Math (per window, sorted positions i, j, head h), following the reference kernels
 // Swin3D/src/attn/self_attn_aio_fwd.cu:16-52 and :111-188:
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
 }
 
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
-template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() { return sizeof(T) == 4 && D > 8 ? 3 : 4; }
+template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() { return D > 8 ? 3 : 4; }
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
 template <typename T, int D, int HP> __host__ __device__ constexpr int table_row_stride_heads()

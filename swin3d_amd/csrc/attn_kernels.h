@@ -38,9 +38,11 @@ int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
-// the shapes where it is the faster of the two kernels: head_dim 16 (at head_dim 8 the sweep kernel's packed
-// fp16 dot products win)
-inline bool attn_mfma_preferred(const AttnArgs &a) { return a.D > 8; }
+// the shapes where it is the faster of the two kernels: head_dim 16 with well-filled windows (128 voxels on
+// average; measured at window 7: 343-voxel windows 0.88 ms against 1.11 ms, 205 voxels 0.43 against 0.47,
+// 104 voxels even, a room scan with 57 voxels on average 0.43 against 0.37).  At head_dim 8 the sweep kernel's
+// packed fp16 dot products win everywhere.
+inline bool attn_mfma_preferred(const AttnArgs &a) { return a.D > 8 && a.N >= 128 * a.W; }
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
 size_t attn_mfma_items_bytes(int64_t W);
 int attn_mfma_key_tiles(int max_window_voxels);
