@@ -61,8 +61,16 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
         padded += (rows + 15) / 16 * 16;
     }
     if (max_window_voxels < 1 || N < 0 || W < 0) return 0;
-    const size_t mfma = attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
     const size_t generic = attn_generic_workspace_bytes(H, D, W, N, max_window_voxels);
+    // the MFMA kernel's share only for shapes it can run (fp16 is not known here)
+    AttnArgs a{};
+    a.H = H;
+    a.D = D;
+    a.nd = nd;
+    int64_t total = 0;
+    for (int n = 0; n < nd; ++n) total += table_sizes[n];
+    if (fill_axes(a, table_sizes, nd, total) != S3D_OK || !attn_mfma_supported(a, S3D_DTYPE_F16)) return generic;
+    const size_t mfma = attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
     return mfma > generic ? mfma : generic;
 }
 
@@ -146,6 +154,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
     a.partials = attn_generic_partials(workspace, H, W, N, max_window_voxels);
-    a.max_key_tiles = attn_generic_key_blocks(max_window_voxels);
+    a.block_shift = attn_generic_block_shift(H, N, W, max_window_voxels);
+    a.max_key_tiles = attn_generic_key_blocks(H, N, W, max_window_voxels);
     return launch_attn_generic(a, dtype, s);
 }

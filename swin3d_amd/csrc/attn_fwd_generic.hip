@@ -27,9 +27,23 @@ using namespace sweep;
 constexpr int kThreads = 256;
 constexpr int kChunk = 64;   // slots per unit at most = lanes of a wavefront
 constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
-// key blocks a window of n voxels is split into (units stream at most kChunk keys), and their even size
-__host__ __device__ inline int key_blocks(int n) { return (n + kChunk - 1) / kChunk; }
-__host__ __device__ inline int key_block_size(int n) { const int b = key_blocks(n); return (n + b - 1) / b; }
+constexpr int kMaxBlockSteps = 256;   // the longest key block a launch may choose
+// key blocks a window of n voxels is split into when a slot streams at most 2^shift keys, and their even size
+__host__ __device__ inline int key_blocks(int n, int shift) { return (n + (1 << shift) - 1) >> shift; }
+__host__ __device__ inline int key_block_size(int n, int shift) { const int b = key_blocks(n, shift); return (n + b - 1) / b; }
+// The key block length of a launch, 64 << shift.  A window longer than that is split and passes partial results
+// through memory (72 bytes per voxel, head and block at head_dim 16, written and read back), so longer blocks
+// are better as long as the longest slot stays short against what a wavefront does in the whole launch:
+// N^2 / W pairs at least, H heads, over the lanes of about 3072 resident wavefronts.  64 unless half of that
+// covers a longer block.
+__host__ inline int block_shift_for(int H, int64_t N, int64_t W, int max_window_voxels)
+{
+    if (N <= 0 || W <= 0) return 6;
+    const double steps_per_wave = static_cast<double>(N) * static_cast<double>(N) / static_cast<double>(W) * H / (64.0 * 3072.0);
+    int shift = 6;
+    while ((1 << shift) < kMaxBlockSteps && (1 << shift) < max_window_voxels && 2.0 * (2 << shift) <= steps_per_wave) ++shift;
+    return shift;
+}
 
 // byte offsets inside the workspace: the queue counters, the totals (units, split windows, slots), the first
 // entry of every unit, the sorted window entries, the placement notes and per-workgroup bin totals of the list
@@ -56,7 +70,7 @@ __host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N, in
 }
 __host__ __device__ inline size_t ws_split_offset(int H, int64_t W, int64_t N, int max_blocks)
 {
-    return ws_bins_offset(H, W, N, max_blocks) + ws_round(sizeof(unsigned long long) * kListGroups * (kChunk + 1));
+    return ws_bins_offset(H, W, N, max_blocks) + ws_round(sizeof(unsigned long long) * kListGroups * (kMaxBlockSteps + 1));
 }
 __host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
 {
@@ -100,8 +114,8 @@ __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 // orders agree; the order inside a bin does not affect results) - and the workgroup leaves its bin totals.
 __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
 {
-    __shared__ unsigned long long bin[kChunk + 1];   // per step count: windows << 32 | slots
-    if (threadIdx.x <= kChunk) bin[threadIdx.x] = 0;
+    __shared__ unsigned long long bin[kMaxBlockSteps + 1];   // per step count: windows << 32 | slots
+    for (int t = threadIdx.x; t <= kMaxBlockSteps; t += kListThreads) bin[t] = 0;
     __syncthreads();
     char *ws = static_cast<char *>(a.workspace);
     int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
@@ -113,17 +127,18 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
     const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
     for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
         const int n = a.w_sizes[w];
-        const int blocks = key_blocks(n);
+        const int blocks = key_blocks(n, a.block_shift);
         int2 got = make_int2(-1, 0);
         if (n > 0 && blocks <= a.max_key_tiles) {
             const unsigned long long before =
-                atomicAdd(&bin[key_block_size(n)], (1ull << 32) | static_cast<unsigned>(n * blocks));
+                atomicAdd(&bin[key_block_size(n, a.block_shift)], (1ull << 32) | static_cast<unsigned>(n * blocks));
             got = make_int2(static_cast<int>(before >> 32), static_cast<int>(before & 0xffffffffu));
         }
         place[w] = got;
     }
     __syncthreads();
-    if (threadIdx.x <= kChunk) group_bins[blockIdx.x * (kChunk + 1) + threadIdx.x] = bin[threadIdx.x];
+    for (int t = threadIdx.x; t <= kMaxBlockSteps; t += kListThreads)
+        group_bins[blockIdx.x * (kMaxBlockSteps + 1) + t] = bin[t];
     if (blockIdx.x == 0 && threadIdx.x == 0) total[1] = 0;   // split windows, counted by the second kernel
 }
 
@@ -133,7 +148,8 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
 // at zero.  Windows beyond the caller's size bound get no slots.
 __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
 {
-    __shared__ int bin_entry[kChunk + 1], bin_slot[kChunk + 1];
+    __shared__ int bin_entry[kMaxBlockSteps + 1], bin_slot[kMaxBlockSteps + 1];
+    __shared__ int wave_c[kListThreads / 64], wave_s[kListThreads / 64];
     __shared__ int sums[2];
     char *ws = static_cast<char *>(a.workspace);
     int *counters = reinterpret_cast<int *>(ws);
@@ -144,16 +160,20 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
     const unsigned long long *group_bins =
         reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N, a.max_key_tiles));
     int *split = reinterpret_cast<int *>(ws + ws_split_offset(a.H, a.W, a.N, a.max_key_tiles));
-    // lane l of the first wavefront holds the bin of 64 - l steps: the launch's total, and what the
-    // workgroups before this one put there
-    if (threadIdx.x < kChunk) {
-        const int lane = threadIdx.x, steps = kChunk - lane;
+    static_assert(kListThreads == kMaxBlockSteps, "one thread per bin");
+    // thread t holds the bin of (longest block) - t steps: the launch's total, and what the workgroups before
+    // this one put there; an exclusive scan over the threads gives the bins their places
+    {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int steps = (1 << a.block_shift) - static_cast<int>(threadIdx.x);
         unsigned long long all = 0, before = 0;
+        if (steps >= 1) {
 #pragma unroll 8
-        for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
-            const unsigned long long v = group_bins[g * (kChunk + 1) + steps];
-            all += v;
-            before += g < static_cast<int>(blockIdx.x) ? v : 0;
+            for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
+                const unsigned long long v = group_bins[g * (kMaxBlockSteps + 1) + steps];
+                all += v;
+                before += g < static_cast<int>(blockIdx.x) ? v : 0;
+            }
         }
         const int cnt = static_cast<int>(all >> 32), slots = static_cast<int>(all & 0xffffffffu);
         int incl_c = cnt, incl_s = slots;
@@ -161,9 +181,15 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
             const int up_c = __shfl_up(incl_c, off), up_s = __shfl_up(incl_s, off);
             if (lane >= off) { incl_c += up_c; incl_s += up_s; }
         }
-        bin_entry[steps] = incl_c - cnt + static_cast<int>(before >> 32);
-        bin_slot[steps] = incl_s - slots + static_cast<int>(before & 0xffffffffu);
-        if (lane == kChunk - 1) { sums[0] = incl_c; sums[1] = incl_s; }
+        if (lane == 63) { wave_c[wave] = incl_c; wave_s[wave] = incl_s; }
+        __syncthreads();
+        int base_c = 0, base_s = 0;
+        for (int v = 0; v < wave; ++v) { base_c += wave_c[v]; base_s += wave_s[v]; }
+        if (steps >= 1) {
+            bin_entry[steps] = base_c + incl_c - cnt + static_cast<int>(before >> 32);
+            bin_slot[steps] = base_s + incl_s - slots + static_cast<int>(before & 0xffffffffu);
+        }
+        if (threadIdx.x == kListThreads - 1) { sums[0] = base_c + incl_c; sums[1] = base_s + incl_s; }
     }
     __syncthreads();
     const int total_entries = sums[0], total_slots = sums[1];
@@ -175,7 +201,7 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
         const int2 got = place[w];
         if (got.x < 0) continue;
         const int n = a.w_sizes[w];
-        const int blocks = key_blocks(n), steps = key_block_size(n);
+        const int blocks = key_blocks(n, a.block_shift), steps = key_block_size(n, a.block_shift);
         const int e = bin_entry[steps] + got.x;
         const int s = bin_slot[steps] + got.y;
         entries[e] = make_int4(s, n, a.w2n[w], steps);
@@ -216,7 +242,7 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
     for (int e = blockIdx.x; e < count; e += gridDim.x) {
         const int w = split[e];
         const int n_w = a.w_sizes[w], s0 = a.w2n[w];
-        const int blocks = key_blocks(n_w);
+        const int blocks = key_blocks(n_w, a.block_shift);
         for (int t = threadIdx.x; t < n_w * H; t += blockDim.x) {
             const int h = t / n_w, pos = s0 + (t - h * n_w);
             const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
@@ -348,7 +374,7 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
         const int in_window = slot - __shfl(seen.x, at);               // [key block][voxel]
         // entries are sorted by steps, longest first
         const int max_steps = (__builtin_amdgcn_readfirstlane(seen.w) + (1 << gshift) - 1) >> gshift;
-        const int blocks = key_blocks(n_w);
+        const int blocks = key_blocks(n_w, a.block_shift);
         const int kb = blocks == 1 ? 0 : in_window / n_w;
         const int own_pos = s0 + (in_window - kb * n_w);
         const int own_row = a.n2n[own_pos];
@@ -514,7 +540,7 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
     S3D_HIP_CHECK(hipGetLastError());
     if (a.max_key_tiles > 1) {
-        const int64_t want = a.W < 256 ? a.W : 256;
+        const int64_t want = a.W < 1024 ? a.W : 1024;
         hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>(want > 0 ? want : 1)), dim3(256),
                            0, stream, a);
         S3D_HIP_CHECK(hipGetLastError());
@@ -546,13 +572,21 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream)
 
 }  // namespace
 
-int attn_generic_key_blocks(int max_window_voxels) { return key_blocks(max_window_voxels > 0 ? max_window_voxels : 1); }
+int attn_generic_block_shift(int H, int64_t N, int64_t W, int max_window_voxels)
+{
+    return block_shift_for(H, N, W, max_window_voxels);
+}
+
+int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels)
+{
+    return key_blocks(max_window_voxels > 0 ? max_window_voxels : 1, block_shift_for(H, N, W, max_window_voxels));
+}
 
 size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels)
 {
     // queue counters, the unit count, the unit descriptors, and one partial record per (key block, head,
     // voxel) when some window may be split along its keys
-    const int blocks = attn_generic_key_blocks(max_window_voxels);
+    const int blocks = attn_generic_key_blocks(H, N, W, max_window_voxels);
     const size_t partials = blocks <= 1 ? 0 : sizeof(float) * static_cast<size_t>(N) * blocks * H * (D + 2);
     return ws_partials_offset(H, W, N, blocks) + align_up(partials, 256);
 }
@@ -560,7 +594,7 @@ size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_
 float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels)
 {
     return reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                     ws_partials_offset(H, W, N, attn_generic_key_blocks(max_window_voxels)));
+                                     ws_partials_offset(H, W, N, attn_generic_key_blocks(H, N, W, max_window_voxels)));
 }
 
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream)

@@ -20,6 +20,7 @@ struct AttnArgs {
     void *items;                           // int32 [W+1] work-item prefix + counter (MFMA path)
     float *partials;                       // per-key-tile partial results of multi-tile windows
     int32_t max_key_tiles;                 // key tiles of the largest window (stride of `partials`)
+    int32_t block_shift;                   // sweep kernel: a slot streams at most 2^block_shift keys
     int32_t target_items;                  // work items the launch wants at least (heads are split to reach it)
     int32_t H, D, nd, total_rows;
     int64_t N, W;
@@ -31,18 +32,19 @@ struct AttnArgs {
 
 // Persistent workgroups, one head each with its table slices in LDS; lane = query, keys streamed; VALU math,
 // any dtype.  Needs a.workspace (work queues, unit list), a.partials and a.max_key_tiles (key blocks of 64).
-int attn_generic_key_blocks(int max_window_voxels);
+int attn_generic_block_shift(int H, int64_t N, int64_t W, int max_window_voxels);
+int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels);
 size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels);
 float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels);
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
-// the shapes where it is the faster of the two kernels: head_dim 16 with well-filled windows (128 voxels on
-// average; measured at window 7: 343-voxel windows 0.88 ms against 1.11 ms, 205 voxels 0.43 against 0.47,
-// 104 voxels even, a room scan with 57 voxels on average 0.43 against 0.37).  At head_dim 8 the sweep kernel's
-// packed fp16 dot products win everywhere.
-inline bool attn_mfma_preferred(const AttnArgs &a) { return a.D > 8 && a.N >= 128 * a.W; }
+// the shapes where it is the faster of the two kernels: head_dim 16 with nearly full windows (256 voxels on
+// average; measured at window 7: 343-voxel windows 0.88 ms against 0.99 ms, 205 voxels 0.435 against 0.424,
+// 104 voxels 0.165 against 0.145, a room scan with 57 voxels on average 0.43 against 0.35).  At head_dim 8 the
+// sweep kernel's packed fp16 dot products win everywhere.
+inline bool attn_mfma_preferred(const AttnArgs &a) { return a.D > 8 && a.N >= 256 * a.W; }
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
 size_t attn_mfma_items_bytes(int64_t W);
 int attn_mfma_key_tiles(int max_window_voxels);

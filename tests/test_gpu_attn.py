@@ -82,6 +82,40 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
     _check(oracle_lib, case, dtype)
 
 
+@pytest.mark.parametrize("heads,block", [(6, 128), (12, 256)])
+def test_long_key_blocks_in_large_dense_launches(oracle_lib, hip_lib, heads, block):
+    """A 56x56x28 grid at 62 % fill, window 7: 256 windows of about 210 voxels.  With this much work per
+    wavefront the sweep kernel streams key blocks of 128 (6 heads) or 256 keys (12 heads) instead of 64, so these
+    windows are split in two or not at all; checked through the partial-result part of the workspace size
+    (quant 5 gives 70-row axis tables, which only the sweep kernel takes, so the size is that kernel's)."""
+    import ctypes
+    ws, quant, dim = 7, 5, 16
+    rng = np.random.default_rng(52)
+    g = np.stack(np.meshgrid(np.arange(56), np.arange(56), np.arange(28), indexing="ij"), -1).reshape(-1, 3)
+    g = g[rng.random(g.shape[0]) < 0.62]
+    g = g[rng.permutation(g.shape[0])]
+    n = g.shape[0]
+    coords = np.concatenate([np.zeros((n, 1), np.int64), g], 1).astype(np.int32)
+    frac = rng.random((n, 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (n, 6)).astype(np.float32)
+    case = make_attn_case(oracle_lib, seed=52, n=64, ws=ws, quant=quant, heads=heads, dim=dim, extent=(12, 12, 6))
+    case.coords = coords
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
+    case.q, case.k, case.v, (case.tq, case.tk, case.tv) = synth.layer_inputs(
+        n, heads * dim, heads, int(sum(case.table_sizes)), seed=52, recipe="sharp")
+    w_sizes = case.index["w_sizes"]
+    assert w_sizes.shape[0] == 256 and 128 < int(w_sizes.max()) <= 256
+    sizes = [int(x) for x in case.table_sizes]
+    c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
+    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, n, 256) == 0
+    ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), heads, dim, n, 256, int(w_sizes.max()))
+    record = n * heads * (dim + 2) * 4           # one partial record per voxel and head
+    blocks = -(-int(w_sizes.max()) // block)     # 2 at 128 keys per block, 1 (no partial results) at 256
+    assert (blocks - 1) * record <= ws_bytes < blocks * record + (8 << 20)
+    _sharp16(case)
+    _check(oracle_lib, case, torch.float16)
+
+
 def boundary_size_case(oracle_lib, heads, dim, seed=41):
     """One window per size in 1, 16, 31..33, 63..65, 127..129, 192, 193 voxels (window 7): the sizes at which the
     kernels change their lane mapping (two 32-lane groups up to 32 voxels) and split a window into chunks of 64
