@@ -197,11 +197,25 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     const T *gv = static_cast<const T *>(a.v);
     const T *ggo = static_cast<const T *>(a.dout);
 
+    // table-gradient accumulators.  VALU updates (head_dim 8): acc[m][c] of lane l is (flat row 64 m + l, channel
+    // c).  MFMA updates (head_dim 16, where one wavefront per SIMD leaves room for accumulation registers and the
+    // update as matrix instructions measured 3-5 % faster; at head_dim 8 it measured 4 % slower): acc[m] holds
+    // D / 4 four-element results in the layout of the 4x4x1 MFMA (16 blocks of 4 rows x 4 channels), element i of
+    // quad c4 in lane l is (flat row 64 m + 4 (l / 4) + i, channel 4 c4 + l % 4)
+    constexpr bool kMfmaUpdate = D > 8;
     float acc_a[BLK][D], acc_b[BLK][D];
 #pragma unroll
     for (int m = 0; m < BLK; ++m)
 #pragma unroll
         for (int c = 0; c < D; ++c) acc_a[m][c] = acc_b[m][c] = 0.0f;
+    auto mfma_update = [](float (&acc)[D], float row_sum, const float (&b)[D / 4]) {
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            f32x4_t r = {acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]};
+            r = __builtin_amdgcn_mfma_f32_4x4x1f32(row_sum, b[c], r, 0, 0, 0);
+            acc[4 * c] = r[0]; acc[4 * c + 1] = r[1]; acc[4 * c + 2] = r[2]; acc[4 * c + 3] = r[3];
+        }
+    };
 
     // 1.0 the optimiser cannot see through: x * one + sum keeps an fp16 row widened inside one mixed-precision FMA
     float one = 1.0f;
@@ -379,12 +393,20 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                 }
             }
             wave_lds_fence();
+            // rank-1 updates acc[row][c] += hist[row] * x[c]; as 4x4x1 MFMAs the A operand of lane l is the sum of
+            // flat row 64 m + l (A of block l / 4, row l % 4), the B operand channel 4 c4 + l % 4 of the
+            // streamed element (the same 1 x 4 row for all 16 blocks)
             for (int g = 0; g < ng; ++g) {
                 const int src = __builtin_amdgcn_readfirstlane(g * gs);   // a lane of group g: its streamed registers are the group's
                 if constexpr (kAccA && kAccB) {
                     const float sc = lane_value(amax, src) * (1.0f / kFixL);
                     const Slice<T, D> sx = st_x.lane(src);   // q_i
                     const Slice<T, D> sy = st_y.lane(src);   // dout_i
+                    float bx[D / 4], by[D / 4];
+                    if constexpr (kMfmaUpdate) {
+                        sx.quad_channels(lane, bx);
+                        sy.quad_channels(lane, by);
+                    }
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
                         unsigned long long *cell = hist_ab + g * kFlat + m * 64 + lane;
@@ -392,27 +414,38 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
                         *cell = 0;
                         const float gsum = static_cast<float>(static_cast<int>(both >> 32)) * sc;
                         const float psum = static_cast<float>(static_cast<unsigned>(both)) * (1.0f / kFixP);
-                        sx.fma_to(acc_a[m], gsum);
-                        sy.fma_to(acc_b[m], psum);
+                        if constexpr (kMfmaUpdate) {
+                            mfma_update(acc_a[m], gsum, bx);
+                            mfma_update(acc_b[m], psum, by);
+                        } else {
+                            sx.fma_to(acc_a[m], gsum);
+                            sy.fma_to(acc_b[m], psum);
+                        }
                     }
                 } else if constexpr (kAccA) {
                     const float sc = lane_value(amax, src) * (1.0f / kFixL);
                     const Slice<T, D> sx = st_x.lane(src);   // q_i (key-owned) or k_j
+                    float bx[D / 4];
+                    if constexpr (kMfmaUpdate) sx.quad_channels(lane, bx);
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
                         int *cell = hist_a + g * kFlat + m * 64 + lane;
                         const float gsum = static_cast<float>(*cell) * sc;
                         *cell = 0;
-                        sx.fma_to(acc_a[m], gsum);
+                        if constexpr (kMfmaUpdate) mfma_update(acc_a[m], gsum, bx);
+                        else sx.fma_to(acc_a[m], gsum);
                     }
                 } else {
                     const Slice<T, D> sy = st_y.lane(src);   // dout_i
+                    float by[D / 4];
+                    if constexpr (kMfmaUpdate) sy.quad_channels(lane, by);
 #pragma unroll
                     for (int m = 0; m < BLK; ++m) {
                         int *cell = hist_b + g * kFlat + m * 64 + lane;
                         const float psum = static_cast<float>(*cell) * (1.0f / kFixP);
                         *cell = 0;
-                        sy.fma_to(acc_b[m], psum);
+                        if constexpr (kMfmaUpdate) mfma_update(acc_b[m], psum, by);
+                        else sy.fma_to(acc_b[m], psum);
                     }
                 }
             }
@@ -445,9 +478,21 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     float *slot = a.tgrad + (static_cast<size_t>(blockIdx.x) * kBwdWaves + wave) * (2 * kFlat * D);
 #pragma unroll
     for (int m = 0; m < BLK; ++m) {
-        const int row = m * 64 + lane;
-        if constexpr (kAccA) store_row<D>(slot + static_cast<size_t>(row) * D, acc_a[m]);
-        if constexpr (kAccB) store_row<D>(slot + static_cast<size_t>(kFlat + row) * D, acc_b[m]);
+        if constexpr (kMfmaUpdate) {
+#pragma unroll
+            for (int c = 0; c < D / 4; ++c) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const size_t at = static_cast<size_t>(m * 64 + (lane & ~3) + i) * D + 4 * c + (lane & 3);
+                    if constexpr (kAccA) slot[at] = acc_a[m][4 * c + i];
+                    if constexpr (kAccB) slot[static_cast<size_t>(kFlat) * D + at] = acc_b[m][4 * c + i];
+                }
+            }
+        } else {
+            const int row = m * 64 + lane;
+            if constexpr (kAccA) store_row<D>(slot + static_cast<size_t>(row) * D, acc_a[m]);
+            if constexpr (kAccB) store_row<D>(slot + static_cast<size_t>(kFlat + row) * D, acc_b[m]);
+        }
     }
 }
 

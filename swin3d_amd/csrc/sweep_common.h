@@ -131,6 +131,16 @@ template <int D> struct Slice<float, D> {
         for (int c = 0; c < D; ++c) r.x[c] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x[c]), src));
         return r;
     }
+    // out[c4] = channel 4 c4 + lane % 4 (the B operand of a 4x4x1 MFMA whose 1 x 4 row is this slice's quad c4)
+    __device__ __forceinline__ void quad_channels(int lane, float *out) const
+    {
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            const float lo = (lane & 1) ? x[4 * c + 1] : x[4 * c];
+            const float hi = (lane & 1) ? x[4 * c + 3] : x[4 * c + 2];
+            out[c] = (lane & 2) ? hi : lo;
+        }
+    }
     // fp32 logits: one short partial sum per table row keeps the rounding of the (2*D*ND + D)-term sum at the
     // level of a tree sum
     static constexpr bool kChainLogit = false;
@@ -180,6 +190,16 @@ template <int D> struct Slice<__half, D> {
         for (int e = 0; e < D / 2; ++e)
             r.x[e] = __builtin_bit_cast(half2_t, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x[e]), src));
         return r;
+    }
+    // out[c4] = channel 4 c4 + lane % 4 (the B operand of a 4x4x1 MFMA whose 1 x 4 row is this slice's quad c4)
+    __device__ __forceinline__ void quad_channels(int lane, float *out) const
+    {
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            const uint32_t pair = (lane & 2) ? __builtin_bit_cast(uint32_t, x[2 * c + 1]) : __builtin_bit_cast(uint32_t, x[2 * c]);
+            const uint32_t bits = pair >> ((lane & 1) * 16);
+            out[c] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+        }
     }
     // fp16 I/O: the whole logit is one chain of dot-product accumulations
     static constexpr bool kChainLogit = true;
