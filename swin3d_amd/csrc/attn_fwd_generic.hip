@@ -27,6 +27,7 @@ using namespace sweep;
 constexpr int kThreads = 256;
 constexpr int kChunk = 64;   // slots per unit at most = lanes of a wavefront
 constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
+constexpr float kSlack = 10.0f;   // how far a logit may exceed the softmax reference exponent before it moves
 constexpr int kMaxBlockSteps = 256;   // the longest key block a launch may choose
 // key blocks a window of n voxels is split into when a slot streams at most 2^shift keys, and their even size
 __host__ __device__ inline int key_blocks(int n, int shift) { return (n + (1 << shift) - 1) >> shift; }
@@ -270,7 +271,10 @@ __global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
 }
 
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
-template <typename T, int D> __host__ __device__ constexpr int groups_per_cu() { return D > 8 ? 3 : 4; }
+template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
+{
+    return D > 8 || HP == 2 ? 3 : 4;
+}
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
 template <typename T, int D, int HP> __host__ __device__ constexpr int table_row_stride_heads()
@@ -281,11 +285,13 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int table_row
 // HP: heads a wavefront carries through a unit (adjacent heads HP * g .. HP * g + HP - 1).  The cRSE rows and
 // LDS addresses of a pair do not depend on the head, so two heads share that part of the work.
 template <typename T, int D, int ND, int HP>
-__global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) void attn_fwd_sweep_kernel(AttnArgs a)
+__global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fwd_sweep_kernel(AttnArgs a)
 {
     // streamed keys per loop iteration: at head_dim 16 two interleaved chains hide the LDS round trips,
     // at head_dim 8 the extra registers cost more than they bring
     constexpr int kKeys = D <= 8 ? 1 : 2;
+    // lazy softmax reference (see the loop): -4 % for fp16; fp32 measured no gain (head_dim 8) or a loss (16)
+    constexpr bool kLazy = sizeof(T) == 2;
     extern __shared__ float smem[];
     const int H = a.H;
     const int HD = H * D;
@@ -384,13 +390,13 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
         const int k0 = s0 + k_begin;
 
         Slice<T, D> qv[HP];
-        float ci[ND], acc[HP][D], m[HP], l[HP];
+        float ci[ND], acc[HP][D], m[HP], top[HP], l[HP];
 #pragma unroll
         for (int hh = 0; hh < HP; ++hh) {
             qv[hh].load(gq + static_cast<int64_t>(own_row) * a.row_stride + (h + hh) * D);
 #pragma unroll
             for (int c = 0; c < D; ++c) acc[hh][c] = 0.0f;
-            m[hh] = -INFINITY;
+            m[hh] = top[hh] = -INFINITY;
             l[hh] = 0.0f;
         }
 #pragma unroll
@@ -444,33 +450,95 @@ __global__ __launch_bounds__(kThreads, (HP == 1 ? groups_per_cu<T, D>() : 3)) vo
                     }
                 }
             }
-            if (valid[0]) {   // the lowest key of the iteration; lanes whose block has ended sit the step out
+            if constexpr (!kLazy) {
+                // online softmax: the running maximum moves with every key that raises it
+                if (valid[0]) {   // the lowest key of the iteration; lanes whose block has ended sit the step out
+#pragma unroll
+                    for (int hh = 0; hh < HP; ++hh) {
+                        float m_new = fmaxf(m[hh], logit[0][hh]);
+#pragma unroll
+                        for (int u = 1; u < kKeys; ++u) {
+                            logit[u][hh] = valid[u] ? logit[u][hh] : -INFINITY;
+                            m_new = fmaxf(m_new, logit[u][hh]);
+                        }
+                        const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
+                        l[hh] *= scale;
+#pragma unroll
+                        for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+#pragma unroll
+                        for (int u = 0; u < kKeys; ++u) {
+                            const float p = __expf(logit[u][hh] - m_new);
+                            l[hh] += p;
+                            v_in[u][hh].fma_to(acc[hh], p);
+#pragma unroll
+                            for (int n = 0; n < ND; ++n) {
+                                Slice<T, D> tv_r;
+                                tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
+                                tv_r.fma_to(acc[hh], p);
+                            }
+                        }
+                        m[hh] = m_new;
+                    }
+                }
+            } else {
+                // Online softmax against a reference exponent m that follows the running maximum lazily: it moves
+                // (and the sums are rescaled) only when some lane's logit exceeds it by more than kSlack, which
+                // after the first keys of a unit is rare, so most steps skip the rescaling of l and the D outputs;
+                // weights stay below e^kSlack.  `top` is the true running maximum.
+                float hi[HP];
+                bool moved = false;
 #pragma unroll
                 for (int hh = 0; hh < HP; ++hh) {
-                    float m_new = fmaxf(m[hh], logit[0][hh]);
+                    hi[hh] = logit[0][hh];
 #pragma unroll
                     for (int u = 1; u < kKeys; ++u) {
                         logit[u][hh] = valid[u] ? logit[u][hh] : -INFINITY;
-                        m_new = fmaxf(m_new, logit[u][hh]);
+                        hi[hh] = fmaxf(hi[hh], logit[u][hh]);
                     }
-                    const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
-                    l[hh] *= scale;
+                    moved = moved || hi[hh] > m[hh] + kSlack;
+                }
+                if (__builtin_amdgcn_ballot_w64(valid[0] && moved) != 0) {   // uniform: all lanes move their reference
+                    if (valid[0]) {
 #pragma unroll
-                    for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+                        for (int hh = 0; hh < HP; ++hh) {
+                            const float m_new = fmaxf(m[hh], hi[hh]);
+                            const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
+                            l[hh] *= scale;
 #pragma unroll
-                    for (int u = 0; u < kKeys; ++u) {
-                        const float p = __expf(logit[u][hh] - m_new);
-                        l[hh] += p;
-                        v_in[u][hh].fma_to(acc[hh], p);
-#pragma unroll
-                        for (int n = 0; n < ND; ++n) {
-                            Slice<T, D> tv_r;
-                            tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
-                            tv_r.fma_to(acc[hh], p);
+                            for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+                            m[hh] = m_new;
                         }
                     }
-                    m[hh] = m_new;
                 }
+                if (valid[0]) {   // the lowest key of the iteration; lanes whose block has ended sit the step out
+#pragma unroll
+                    for (int hh = 0; hh < HP; ++hh) {
+                        top[hh] = fmaxf(top[hh], hi[hh]);
+#pragma unroll
+                        for (int u = 0; u < kKeys; ++u) {
+                            const float p = __expf(logit[u][hh] - m[hh]);
+                            l[hh] += p;
+                            v_in[u][hh].fma_to(acc[hh], p);
+#pragma unroll
+                            for (int n = 0; n < ND; ++n) {
+                                Slice<T, D> tv_r;
+                                tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
+                                tv_r.fma_to(acc[hh], p);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // from the reference exponent to the true maximum (lanes that saw no key: both are -inf, nothing to scale)
+        if constexpr (kLazy) {
+#pragma unroll
+            for (int hh = 0; hh < HP; ++hh) {
+                const float scale = top[hh] == -INFINITY ? 1.0f : __expf(m[hh] - top[hh]);
+                l[hh] *= scale;
+#pragma unroll
+                for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+                m[hh] = top[hh];
             }
         }
 #pragma unroll
@@ -526,7 +594,7 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     }
     // a workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow,
     // in whole sets of (XCDs x head groups)
-    int per_cu = HP == 1 ? groups_per_cu<T, D>() : 3;
+    int per_cu = groups_per_cu<T, D, HP>();
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
     const int set = kQueues * (a.H / HP);
     const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
