@@ -113,28 +113,64 @@ __host__ __device__ inline size_t units_list_index(int H) { return units_total_i
 // one workgroup
 __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
 {
-    __shared__ int part[1024];
+    // units are listed longest first, in classes of window size (a unit streams the whole window: n steps, or
+    // n / 2 up to 32 voxels), windows in order inside a class: the launch then ends on its shortest units
+    constexpr int kClasses = 6;
+    auto class_of = [](int n) { return n > 256 ? 0 : n > 128 ? 1 : n > 64 ? 2 : n > 32 ? 3 : n > 16 ? 4 : 5; };
+    __shared__ int wave_sum[16][kClasses];
+    __shared__ int class_start[kClasses + 1];
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
-    const int begin = threadIdx.x * per, end = min(begin + per, W);
-    int sum = 0;
-    for (int w = begin; w < end; ++w) sum += (a.w_sizes[w] + kChunk - 1) / kChunk;
-    part[threadIdx.x] = sum;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const int add = static_cast<int>(threadIdx.x) >= off ? part[threadIdx.x - off] : 0;
-        __syncthreads();
-        part[threadIdx.x] += add;
-        __syncthreads();
+    const int begin = min(static_cast<int>(threadIdx.x) * per, W), end = min(begin + per, W);
+    int mine[kClasses];
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) mine[c] = 0;
+    for (int w = begin; w < end; ++w) {
+        const int n = a.w_sizes[w];
+        const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
+#pragma unroll
+        for (int c = 0; c < kClasses; ++c) mine[c] += c == cls ? chunks : 0;
     }
-    int run = part[threadIdx.x] - sum;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl[kClasses];
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) {
+        incl[c] = mine[c];
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl[c], off);
+            if (lane >= off) incl[c] += up;
+        }
+        if (lane == 63) wave_sum[wave][c] = incl[c];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int c = 0; c < kClasses; ++c) {
+            class_start[c] = run;
+            for (int v = 0; v < 16; ++v) {
+                const int t = wave_sum[v][c];
+                wave_sum[v][c] = run;   // units of this class in the wavefronts before v
+                run += t;
+            }
+        }
+        class_start[kClasses] = run;
+    }
+    __syncthreads();
+    int run[kClasses];
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) run[c] = wave_sum[wave][c] + incl[c] - mine[c];
     int2 *list = reinterpret_cast<int2 *>(a.units + units_list_index(a.H));
     for (int w = begin; w < end; ++w) {
-        const int chunks = (a.w_sizes[w] + kChunk - 1) / kChunk;
-        for (int c = 0; c < chunks; ++c) list[run + c] = make_int2(w, c);
-        run += chunks;
+        const int n = a.w_sizes[w];
+        const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
+        int at = 0;
+#pragma unroll
+        for (int c = 0; c < kClasses; ++c) {
+            if (c == cls) { at = run[c]; run[c] += chunks; }
+        }
+        for (int c = 0; c < chunks; ++c) list[at + c] = make_int2(w, c);
     }
-    if (threadIdx.x == 1023) a.units[units_total_index(a.H)] = part[1023];
+    if (threadIdx.x == 0) a.units[units_total_index(a.H)] = class_start[kClasses];
 }
 
 // the work counters are re-armed between sweeps
@@ -237,7 +273,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 
     int queue = xcd_id() % kQueues;
     int tried = 0;       // queues found empty so far
-    int drawn = 0;       // ticket of the next unit, drawn one unit ahead so that the atomic's round trip overlaps work
+    int drawn = 0;       // ticket of the next unit
     if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
     for (;;) {
         int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
@@ -247,7 +283,6 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
             unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
         }
         if (unit >= total_units) break;
-        if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
         const int2 desc = unit_list[unit];
         const int w = __builtin_amdgcn_readfirstlane(desc.x);
         const int chunk = __builtin_amdgcn_readfirstlane(desc.y);
@@ -284,6 +319,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         const int steps = (n_w + ng - 1) / ng;
         int st_row_next = a.n2n[s0 + min(grp, n_w - 1)];
         for (int it = 0; it < steps; ++it) {
+            // the next unit's ticket is drawn during the last step: the atomic's round trip overlaps that work, and
+            // a unit is not held back, out of reach of idle wavefronts, for the length of a unit
+            if (it + 1 == steps && lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
             const int st = it * ng + grp;
             const bool st_valid = st < n_w;
             const int st_pos = s0 + min(st, n_w - 1);
@@ -567,7 +605,9 @@ int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
 }
 
 // workgroups of a sweep: whole sets of (XCDs x heads), about two per CU (a workgroup serves one head for its
-// whole life)
+// whole life).  At head_dim 16 only one fits a CU at a time; the others start as the first heads run out of
+// units and go to the heads that still have some, which measured 5 % faster than a grid of one per CU (whole
+// sets leave 16 of 256 CUs without a workgroup at six heads).
 int bwd_grid(int H)
 {
     int device = 0, cus = 256;
