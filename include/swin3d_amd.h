@@ -107,8 +107,8 @@ const char *s3d_last_error_string(void);
 #define S3D_ATTN_FORCE_GENERIC 1
 #define S3D_ATTN_FORCE_MFMA 2
 /* 1 if s3d_attn_fwd with flags 0 runs these shapes on the MFMA kernel (fp16, head_dim 16, every axis
- * table <= 64 rows, and windows of at least 256 voxels on average: N >= 256 W), 0 if on the VALU sweep
- * kernel.  No counterpart in the reference (it has one kernel). */
+ * table <= 64 rows, and windows of at least 256 voxels on average, N >= 256 W, or 60 with 16 heads or more),
+ * 0 if on the VALU sweep kernel.  No counterpart in the reference (it has one kernel). */
 int s3d_attn_fwd_uses_mfma(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype,
                            int64_t N, int64_t W);
 size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,

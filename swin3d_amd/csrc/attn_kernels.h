@@ -41,10 +41,16 @@ int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
 // the shapes where it is the faster of the two kernels: head_dim 16 with nearly full windows (256 voxels on
-// average; measured at window 7: 343-voxel windows 0.88 ms against 0.99 ms, 205 voxels 0.435 against 0.424,
-// 104 voxels 0.165 against 0.145, a room scan with 57 voxels on average 0.43 against 0.35).  At head_dim 8 the
-// sweep kernel's packed fp16 dot products win everywhere.
-inline bool attn_mfma_preferred(const AttnArgs &a) { return a.D > 8 && a.N >= 256 * a.W; }
+// average; measured at window 7 with 6 heads: 343-voxel windows 0.88 ms against 0.99 ms, 205 voxels 0.435 against
+// 0.424, 104 voxels 0.165 against 0.145, a room scan with 57 voxels on average 0.43 against 0.35), or with many
+// heads, over which it spreads the row indices of a tile pair, and 60 voxels on average (Swin3D-L, window 7: 20
+// heads and 61 voxels 0.885 against 0.919 ms, 55 voxels 0.853 against 0.718; 40 heads and 69 voxels 0.571 against
+// 0.700, 45 voxels 0.463 against 0.429; 10 heads and 58 voxels 1.57 against 1.37).  At head_dim 8 the sweep
+// kernel's packed fp16 dot products win everywhere.
+inline bool attn_mfma_preferred(const AttnArgs &a)
+{
+    return a.D > 8 && (a.N >= 256 * a.W || (a.H >= 16 && a.N >= 60 * a.W));
+}
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
 size_t attn_mfma_items_bytes(int64_t W);
 int attn_mfma_key_tiles(int max_window_voxels);

@@ -65,22 +65,32 @@ def lookup_rows(sorted_keys, order, query_keys):
     return torch.where(hit, order[pos], torch.full_like(pos, -1))
 
 
-def sparse_conv3x3x3(voxels, weight):
+def conv3x3x3_neighbours(coords, stride):
+    """[N, 27] long: the row of every voxel's 27 lattice neighbours (offsets ordered x-major), N where the
+    neighbour is missing.  Depends on the coordinates only.  A packed key is linear in the coordinates, so a
+    neighbour's key is the voxel's key plus a constant per offset; taken in sorted key order the 27 query lists are
+    sorted themselves, which keeps the binary searches local."""
+    n = coords.shape[0]
+    sorted_keys, order = torch.sort(pack_coords(coords))
+    deltas = torch.tensor([((dx << _FIELD) + dy << _FIELD) + dz for dx in (-1, 0, 1) for dy in (-1, 0, 1)
+                           for dz in (-1, 0, 1)], dtype=torch.long, device=coords.device) * stride
+    queries = sorted_keys.unsqueeze(0) + deltas.unsqueeze(1)                    # [27, N], rows ascending
+    pos = torch.searchsorted(sorted_keys, queries).clamp_(max=n - 1)
+    rows = torch.where(sorted_keys[pos] == queries, order[pos], torch.full_like(pos, n))
+    out = torch.empty((n, 27), dtype=torch.long, device=coords.device)
+    out[order] = rows.t()
+    return out
+
+
+def sparse_conv3x3x3(voxels, weight, neighbours=None):
     """Submanifold-style 3x3x3 convolution (outputs on the input voxels; missing neighbours are
     zeros).  weight [27, Cin, Cout], offsets ordered x-major.  One gather + one GEMM."""
-    coords, feats, s = voxels.coords, voxels.feats, voxels.stride
+    feats = voxels.feats
     n, cin = feats.shape
-    keys = pack_coords(coords)
-    sorted_keys, order = torch.sort(keys)
+    if neighbours is None:
+        neighbours = conv3x3x3_neighbours(voxels.coords, voxels.stride)
     padded = torch.cat([feats, feats.new_zeros(1, cin)], 0)   # row n = zeros for missing neighbours
-    cols = []
-    for dx in (-1, 0, 1):
-        for dy in (-1, 0, 1):
-            for dz in (-1, 0, 1):
-                off = torch.tensor([0, dx * s, dy * s, dz * s], dtype=coords.dtype, device=coords.device)
-                rows = lookup_rows(sorted_keys, order, pack_coords(coords + off))
-                cols.append(padded[torch.where(rows < 0, torch.full_like(rows, n), rows)])
-    gathered = torch.cat(cols, 1)                              # [N, 27*Cin]
+    gathered = padded[neighbours.reshape(-1)].view(n, 27 * cin)
     return gathered @ weight.reshape(27 * cin, -1).to(gathered.dtype)
 
 
@@ -128,8 +138,8 @@ class StemConv(nn.Module):
         nn.init.kaiming_normal_(self.weight.view(27 * in_channels, out_channels).t())
         self.norm = nn.BatchNorm1d(out_channels)
 
-    def forward(self, voxels):
-        out = sparse_conv3x3x3(voxels, self.weight)
+    def forward(self, voxels, neighbours=None):
+        out = sparse_conv3x3x3(voxels, self.weight, neighbours)
         return voxels.with_feats(F.relu(self.norm(out.float())))
 
 
@@ -151,14 +161,19 @@ class GridKNNDownsample(nn.Module):
         self.norm = nn.LayerNorm(in_channels)
         self.linear = nn.Linear(in_channels, out_channels, bias=False)
 
-    def forward(self, voxels, signals):
-        coarse, cell_of_row = pool_coordinates(voxels.coords, voxels.stride, self.factor)
+    def plan(self, coords, stride, signals):
+        """The part that depends on coordinates and signals only: (coarse coordinates, coarse signals, the K
+        nearest fine rows of every coarse voxel)."""
+        coarse, cell_of_row = pool_coordinates(coords, stride, self.factor)
         pick = pick_cell_representatives(signals, cell_of_row, coarse.shape[0])
         coarse_signals = signals[pick]
         src_xyz = signals[:, 1:4].contiguous().float()
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()
-        idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(voxels.coords[:, 0]),
-                           segment_offsets(coarse[:, 0]))
+        idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(coords[:, 0]), segment_offsets(coarse[:, 0]))
+        return coarse, coarse_signals, idx.view(-1).long().clamp_(min=0)
+
+    def forward(self, voxels, signals, plan=None):
+        coarse, coarse_signals, rows = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
         # LayerNorm and Linear act on single rows, so they commute with the gather: project the Ns fine rows once
         # instead of the K * Nq gathered copies (the reference statement, swin3d_layers.py:292-312, gathers first)
         if _fused_norm_applies(voxels.feats):
@@ -166,7 +181,7 @@ class GridKNNDownsample(nn.Module):
         else:
             normed = self.norm(voxels.feats)
         projected = self.linear(normed)
-        grouped = projected[idx.view(-1).long().clamp_(min=0)].view(coarse.shape[0], self.k, projected.shape[1])
+        grouped = projected[rows].view(coarse.shape[0], self.k, projected.shape[1])
         feats = grouped.amax(dim=1)
         return SparseVoxels(coarse, feats.float(), voxels.stride * self.factor), coarse_signals
 
@@ -277,17 +292,25 @@ class Stage(nn.Module):
             [SwinBlock(dim, num_heads, window_size, quant_size, cRSE=cRSE, fp16_mode=fp16_mode) for _ in range(depth)])
         self.downsample = GridKNNDownsample(dim, out_channels or dim * 2, stride=down_stride) if downsample else None
 
-    def forward(self, voxels, signals):
-        """signals [N, 4|7|10] float = (batch, xyz in voxel units, rgb, normal) of the point kept
-        in every voxel.  Returns (features at this resolution, next voxels, next signals)."""
-        local = (signals[:, 1:4].float() - voxels.coords[:, 1:].float()) / voxels.stride
+    def plan(self, coords, stride, signals):
+        """Everything of the stage that depends on coordinates and signals only: the two window index sets
+        (regular and shifted windows) with their scaled signals, and the downsample's geometry.  This is where
+        the host waits for the device (window counts, unique cells); `forward` with a plan does not."""
+        local = (signals[:, 1:4].float() - coords[:, 1:].float()) / stride
         extra = signals[:, 4:].float()
-        args = [get_index01(voxels.coords, voxels.stride, self.window_size, local, extra, shift=s)
+        args = [get_index01(coords, stride, self.window_size, local, extra, shift=s)
                 for s in (0, self.window_size // 2)]
         if len(self.blocks) > 0:
             # the quantiser scaling of the signals is the same for every block of the stage: once per index set
             attn = self.blocks[0].attn
             args = [tuple(a) + (scale_crse_coords(a[7], attn.quant_size, attn.cRSE),) for a in args]
+        down = self.downsample.plan(coords, stride, signals) if self.downsample is not None else None
+        return args, down
+
+    def forward(self, voxels, signals, plan=None):
+        """signals [N, 4|7|10] float = (batch, xyz in voxel units, rgb, normal) of the point kept
+        in every voxel.  Returns (features at this resolution, next voxels, next signals)."""
+        args, down_plan = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
         feats = voxels.feats
         if len(self.blocks) > 0 and self.blocks[0]._fused_path(feats):
             pending = None
@@ -300,8 +323,27 @@ class Stage(nn.Module):
         voxels = voxels.with_feats(feats)
         if self.downsample is None:
             return voxels, voxels, signals
-        down, down_signals = self.downsample(voxels, signals)
+        down, down_signals = self.downsample(voxels, signals, down_plan)
         return voxels, down, down_signals
+
+
+def geometry_steps(stem_coords, stride, signals, layers):
+    """Generator over the geometry of a forward pass, in the order the feature pass needs it: the stem
+    convolution's neighbour rows, then the plan of every stage (finest first).  None of it depends on features."""
+    yield conv3x3x3_neighbours(stem_coords, stride)
+    coords = stem_coords
+    for layer in layers:
+        plan = layer.plan(coords, stride, signals)
+        yield plan
+        if plan[1] is not None:
+            coords, signals = plan[1][0], plan[1][1]
+            stride = stride * layer.downsample.factor
+
+
+def plan_stages(stem_coords, stride, signals, layers):
+    """(stem neighbours, [stage plans]) computed up front on the current stream."""
+    steps = list(geometry_steps(stem_coords, stride, signals, layers))
+    return steps[0], steps[1:]
 
 
 class Swin3DEncoder(nn.Module):
@@ -324,10 +366,13 @@ class Swin3DEncoder(nn.Module):
                     nn.init.zeros_(m.bias)
 
     def forward(self, voxels, signals):
-        voxels = self.stem_layer(voxels)
+        # geometry first (it needs no features, and it is where the host waits for the device), then the
+        # feature pass in one uninterrupted run of launches
+        neighbours, plans = plan_stages(voxels.coords, voxels.stride, signals, self.layers)
+        voxels = self.stem_layer(voxels, neighbours)
         outputs = []
-        for layer in self.layers:
-            here, voxels, signals = layer(voxels, signals)
+        for layer, plan in zip(self.layers, plans):
+            here, voxels, signals = layer(voxels, signals, plan)
             outputs.append(here)
         return outputs
 
@@ -431,10 +476,11 @@ class Swin3DUNet(nn.Module):
 
     def forward(self, voxels, signals):
         """-> logits [N, num_classes] on the input voxels."""
-        voxels = self.stem_layer(voxels)
+        neighbours, plans = plan_stages(voxels.coords, voxels.stride, signals, self.layers)
+        voxels = self.stem_layer(voxels, neighbours)
         levels = []
-        for layer in self.layers:
-            here, voxels_next, signals_next = layer(voxels, signals)
+        for layer, plan in zip(self.layers, plans):
+            here, voxels_next, signals_next = layer(voxels, signals, plan)
             levels.append((here, signals))
             voxels, signals = voxels_next, signals_next
         voxels, signals = levels.pop()
