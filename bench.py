@@ -25,8 +25,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per s3d_attn_fwd call from the FETCH_SIZE / WRITE_SIZE passes recorded in
 # profiles/attn_fwd_headline.txt (sweep kernel + partial merge + the two list kernels): fetch
-# (62021 + 279 + 196) KiB * 2.00, write (31502 + 98 + 235) KiB * 1.00, factors from the 64 MiB copy
-MEASURED_TRAFFIC_BYTES = int(((62021 + 279 + 196) * 2.00 + (31502 + 98 + 235) * 1.00) * 1024)
+# (58869 + 282 + 212) KiB * 2.00, write (21892 + 98 + 280) KiB * 1.00, factors from the 64 MiB copy
+MEASURED_TRAFFIC_BYTES = int(((58869 + 282 + 212) * 2.00 + (21892 + 98 + 280) * 1.00) * 1024)
 
 
 def algorithmic_bytes(n, c, elem_bytes, nd, w, table_len):
