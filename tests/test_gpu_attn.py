@@ -117,9 +117,9 @@ def test_long_key_blocks_in_large_dense_launches(oracle_lib, hip_lib, heads, blo
 
 
 def boundary_size_case(oracle_lib, heads, dim, seed=41):
-    """One window per size in 1, 16, 31..33, 63..65, 127..129, 192, 193 voxels (window 7): the sizes at which the
-    kernels change their lane mapping (two 32-lane groups up to 32 voxels) and split a window into chunks of 64
-    queries and blocks of 64 (sweep kernel) or 32 (MFMA kernel) keys."""
+    """One window per size in 1, 16, 31..33, 63..65, 127..129, 192, 193 voxels (window 7): the sizes around the
+    tile and block lengths at which the kernels split a window (key blocks of 64 in the sweep kernel, tiles of 32
+    queries and keys in the MFMA kernel; the backward changes its lane mapping at 32 voxels)."""
     ws, quant = 7, 4
     sizes = [1, 16, 31, 32, 33, 63, 64, 65, 127, 128, 129, 192, 193]
     rng = np.random.default_rng(seed)
@@ -157,6 +157,36 @@ def test_single_voxel_windows_and_one_head(oracle_lib, hip_lib):
                                                     1, 5, 4, "XYZ")
     assert case.index["w_sizes"].tolist() == [1, 2, 1]
     _check(oracle_lib, case, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_more_windows_than_list_builder_threads(oracle_lib, hip_lib, dtype):
+    """40 000 windows of one to four voxels (a sparse 3-D lattice of window cells): the work-list kernels of the
+    sweep kernel run at most 128 workgroups of 256 threads, so here every thread places several windows, and
+    all units are of the small kinds."""
+    ws, quant, heads, dim = 5, 4, 6, 8
+    rng = np.random.default_rng(61)
+    cells = np.stack(np.meshgrid(np.arange(50), np.arange(40), np.arange(20), indexing="ij"), -1).reshape(-1, 3)
+    per_cell = rng.integers(1, 5, size=cells.shape[0])
+    rows = []
+    for k in range(4):
+        take = cells[per_cell > k]
+        rows.append(take * (2 * ws) + np.array([k, (k * 2) % ws, (k * 3) % ws]))   # distinct voxels inside the cell
+    g = np.concatenate(rows, 0)
+    g = g[rng.permutation(g.shape[0])]
+    n = g.shape[0]
+    coords = np.concatenate([np.zeros((n, 1), np.int64), g], 1).astype(np.int32)
+    frac = rng.random((n, 3)).astype(np.float32)
+    sig = rng.uniform(-1, 1, (n, 6)).astype(np.float32)
+    case = make_attn_case(oracle_lib, seed=61, n=64, ws=ws, quant=quant, heads=heads, dim=dim, extent=(12, 12, 6))
+    case.coords = coords
+    case.index, case.n_coords = n_coords_from_scene(oracle_lib, coords, frac, sig, 1, ws, quant, case.cRSE)
+    case.q, case.k, case.v, (case.tq, case.tk, case.tv) = synth.layer_inputs(
+        n, heads * dim, heads, int(sum(case.table_sizes)), seed=61, recipe="sharp")
+    assert case.index["w_sizes"].shape[0] == 40000 and int(case.index["w_sizes"].max()) == 4
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
 
 
 def test_upper_edge_rows_are_folded_not_out_of_bounds(oracle_lib, hip_lib):
