@@ -104,9 +104,10 @@ __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 }
 
 // Work list of the launch, built by two small kernels.  A voxel of a window that is split into b key blocks
-// (b = 1 up to 64 voxels) takes b slots, one per key block, and a slot streams the block's keys: at most 64
-// steps.  The windows are sorted by that step count, longest first (a counting sort over the 64 possible
-// counts), their slots laid out back to back in that order - [window][key block][voxel] - and cut into units,
+// (b = 1 up to the launch's block length of 64, 128 or 256 voxels) takes b slots, one per key block, and a slot
+// streams the block's keys: at most that many steps.  The windows are sorted by that step count, longest first
+// (a counting sort over the possible counts), their slots laid out back to back in that order -
+// [window][key block][voxel] - and cut into units,
 // so a wavefront's lanes carry queries of several windows when the windows are small, every lane of a unit
 // runs (almost) the same number of steps, and the launch ends on its shortest units.
 //
