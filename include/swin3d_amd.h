@@ -180,6 +180,26 @@ int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t w
                      int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Signal matrix of the attention op in window-sorted order (the `n_coords` argument of s3d_attn_fwd), one pass.
+ *
+ * Replaces the tensor statements of BasicLayer.get_index01 (Swin3D/modules/swin3d_layers.py:800-804: window-local
+ * voxel position + fractional position, other signals appended, both gathered into sorted order) and, with the
+ * two scales, of WindowAttention.forward (:513-536: xyz columns times quant_size, the others times 2 * quant_size).
+ *
+ *   w_w_id, n2n   device int32 [N]   outputs of s3d_window_index
+ *   frac          device fp32 [N,3]  position of the point inside its voxel, in voxels, original row order
+ *   signals       device fp32 rows of `signals_stride` floats, original row order; the first `num_signals`
+ *                 columns are used (0, 3 or 6: colour, normal); may be null when num_signals = 0
+ *   out           device fp32 [N, 3 + num_signals]:
+ *                 out[p] = ((lx, ly, lz) + frac[n2n[p]]) * xyz_scale, signals[n2n[p]] * other_scale
+ *                 (sum and product rounded separately, as the tensor statements do)
+ *   scales 1, 1 give the reference's unscaled n_coords.
+ */
+int s3d_window_signals(const int32_t *w_w_id, const int32_t *n2n, const float *frac, const float *signals,
+                       int64_t signals_stride, int32_t num_signals, int32_t window, float xyz_scale,
+                       float other_scale, float *out, int64_t N, void *stream);
+
+/*
  * K nearest sources of every query inside the same batch segment.
  *
  * Replaces knn_cuda (Swin3D/src/knn/knn_cuda_kernel.cu:207-244, declared in

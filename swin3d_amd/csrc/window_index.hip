@@ -158,8 +158,51 @@ __global__ __launch_bounds__(kThreads) void segment_size_kernel(const int32_t *_
     }
 }
 
+// one thread per (sorted position, column); the add and the multiply stay separate roundings, as in the
+// reference's tensor statement (sum, then scale)
+__global__ __launch_bounds__(kThreads) void window_signals_kernel(
+    const int32_t *__restrict__ w_w_id, const int32_t *__restrict__ n2n, const float *__restrict__ frac,
+    const float *__restrict__ signals, int64_t signals_stride, int columns, int window, float xyz_scale,
+    float other_scale, float *__restrict__ out, int64_t N)
+{
+#pragma clang fp contract(off)
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (t >= N * columns) return;
+    const int64_t p = t / columns;
+    const int c = static_cast<int>(t - p * columns);
+    const int64_t row = n2n[p];
+    float v;
+    if (c < 3) {
+        const int id = w_w_id[p];
+        const int cell = c == 0 ? id / (window * window) : c == 1 ? (id / window) % window : id % window;
+        v = (static_cast<float>(cell) + frac[row * 3 + c]) * xyz_scale;
+    } else {
+        v = signals[row * signals_stride + (c - 3)] * other_scale;
+    }
+    out[t] = v;
+}
+
 }  // namespace
 }  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) int s3d_window_signals(
+    const int32_t *w_w_id, const int32_t *n2n, const float *frac, const float *signals, int64_t signals_stride,
+    int32_t num_signals, int32_t window, float xyz_scale, float other_scale, float *out, int64_t N, void *stream)
+{
+    using namespace s3d;
+    if (N < 0 || num_signals < 0 || window < 1 || window > 10 || (num_signals > 0 && signals_stride < num_signals))
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_signals: N=%lld num_signals=%d signals_stride=%lld window=%d",
+                    (long long)N, num_signals, (long long)signals_stride, window);
+    if (N == 0) return S3D_OK;
+    if (!w_w_id || !n2n || !frac || !out || (num_signals > 0 && !signals))
+        return fail(S3D_ERR_NULL_POINTER, "s3d_window_signals: null device pointer");
+    const int columns = 3 + num_signals;
+    const dim3 grid(static_cast<unsigned>(ceil_div(N * columns, kThreads)));
+    hipLaunchKernelGGL(window_signals_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), w_w_id, n2n,
+                       frac, signals, signals_stride, columns, window, xyz_scale, other_scale, out, N);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_window_index_workspace_bytes(int64_t N)
 {

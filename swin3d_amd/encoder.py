@@ -30,7 +30,7 @@ from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
 from .fused_norm import add_layernorm
 from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
 from .sparse_dl.knn import KNN, KNNInterpolate, knn_query
-from .window_index import get_index01
+from .window_index import build_window_indices, get_index01, index_arguments, window_signals
 
 
 @dataclass
@@ -298,12 +298,15 @@ class Stage(nn.Module):
         the host waits for the device (window counts, unique cells); `forward` with a plan does not."""
         local = (signals[:, 1:4].float() - coords[:, 1:].float()) / stride
         extra = signals[:, 4:].float()
-        args = [get_index01(coords, stride, self.window_size, local, extra, shift=s)
-                for s in (0, self.window_size // 2)]
+        # both window sets are enqueued before the host waits for their window counts
+        indices = build_window_indices(coords, stride, self.window_size, (0, self.window_size // 2))
+        args = [index_arguments(index, local, extra) for index in indices]
         if len(self.blocks) > 0:
-            # the quantiser scaling of the signals is the same for every block of the stage: once per index set
+            # the quantiser scaling of the signals is the same for every block of the stage: once per index set,
+            # fused with the gather into window order
             attn = self.blocks[0].attn
-            args = [tuple(a) + (scale_crse_coords(a[7], attn.quant_size, attn.cRSE),) for a in args]
+            args = [tuple(a) + (window_signals(index, local, extra, crse_num_axes(attn.cRSE) - 3, attn.quant_size,
+                                               2 * attn.quant_size),) for a, index in zip(args, indices)]
         down = self.downsample.plan(coords, stride, signals) if self.downsample is not None else None
         return args, down
 

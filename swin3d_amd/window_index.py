@@ -37,12 +37,10 @@ class WindowIndex:
         return inv
 
 
-def build_window_index(coords, stride, window_size, shift=0):
-    """coords int32 [N,4] (batch,x,y,z) CUDA tensor -> WindowIndex.
-
-    `shift` is in voxels (0, or window_size // 2 for the shifted window set).
-    Synchronises once to read the window count back.
-    """
+def build_window_indices(coords, stride, window_size, shifts):
+    """One WindowIndex per entry of `shifts` (voxels: 0, or window_size // 2 for the shifted window set) for
+    coords int32 [N,4] (batch,x,y,z) on the GPU.  All index builds are enqueued before the host reads the
+    window counts back, so the call synchronises once however many shifts it is given."""
     if not coords.is_cuda:
         raise RuntimeError("coords must be a CUDA (HIP) tensor")
     if coords.dim() != 2 or coords.shape[1] != 4:
@@ -50,28 +48,68 @@ def build_window_index(coords, stride, window_size, shift=0):
     dev = coords.device
     coords = coords.to(torch.int32).contiguous()
     n = coords.shape[0]
-    n2n = torch.empty(n, dtype=torch.int32, device=dev)
-    wwid = torch.empty(n, dtype=torch.int32, device=dev)
-    w_sizes = torch.empty(n, dtype=torch.int32, device=dev)
-    w2n = torch.empty(n, dtype=torch.int32, device=dev)
-    counts = torch.empty(4, dtype=torch.int64, device=dev)
+    shifts = list(shifts)
+    counts = torch.empty((len(shifts), 4), dtype=torch.int64, device=dev)
     lib = _lib.lib()
+    outputs = []
     with torch.cuda.device(dev):
         ws_bytes = lib.s3d_window_index_workspace_bytes(n)
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
-        status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window_size),
-                                      int(shift), n2n.data_ptr(), wwid.data_ptr(),
-                                      w_sizes.data_ptr(), w2n.data_ptr(), counts.data_ptr(),
-                                      workspace.data_ptr(), ws_bytes, stream)
-    _lib.check(status, "s3d_window_index")
-    num_w, num_m, max_w, err = counts.tolist()
-    if err:
-        raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
-                         "-8192..8191)")
-    sizes = w_sizes[:num_w]
-    sizes.max_window_voxels = int(max_w)   # read by the attention op (sizes its partial-result workspace)
-    return WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window_size))
+        for i, shift in enumerate(shifts):
+            n2n, wwid, w_sizes, w2n = (torch.empty(n, dtype=torch.int32, device=dev) for _ in range(4))
+            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window_size), int(shift),
+                                          n2n.data_ptr(), wwid.data_ptr(), w_sizes.data_ptr(), w2n.data_ptr(),
+                                          counts[i].data_ptr(), workspace.data_ptr(), ws_bytes, stream)
+            _lib.check(status, "s3d_window_index")
+            outputs.append((n2n, wwid, w_sizes, w2n))
+    result = []
+    for (n2n, wwid, w_sizes, w2n), (num_w, num_m, max_w, err) in zip(outputs, counts.tolist()):
+        if err:
+            raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
+                             "-8192..8191)")
+        sizes = w_sizes[:num_w]
+        sizes.max_window_voxels = int(max_w)   # read by the attention op (sizes its partial-result workspace)
+        result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w),
+                                  int(window_size)))
+    return result
+
+
+def build_window_index(coords, stride, window_size, shift=0):
+    """coords int32 [N,4] (batch,x,y,z) CUDA tensor -> WindowIndex.
+
+    `shift` is in voxels (0, or window_size // 2 for the shifted window set).
+    Synchronises once to read the window count back.
+    """
+    return build_window_indices(coords, stride, window_size, [shift])[0]
+
+
+def window_signals(index, local_xyz, colors, num_signals=None, xyz_scale=1.0, other_scale=1.0):
+    """fp32 [N, 3 + num_signals] signal matrix of the attention op in window-sorted order, one kernel:
+    ((window-local voxel + local_xyz) * xyz_scale, colors[:, :num_signals] * other_scale), rows gathered through
+    index.n2n.  Scales 1 give the reference's n_coords (swin3d_layers.py:800-804); quant_size and 2 * quant_size
+    give the scaled signals WindowAttention.forward hands to the operator (:513-536)."""
+    frac = local_xyz.to(torch.float32).contiguous()
+    colors = colors.to(torch.float32)
+    if colors.dim() != 2 or (colors.shape[1] > 0 and colors.stride(1) != 1):
+        colors = colors.contiguous()
+    if num_signals is None:
+        num_signals = colors.shape[1]
+    if num_signals > colors.shape[1]:
+        raise ValueError(f"{num_signals} signal columns asked for, colors has {colors.shape[1]}")
+    n = index.n2n.numel()
+    if frac.shape != (n, 3) or colors.shape[0] != n:
+        raise ValueError(f"local_xyz must be [{n},3] and colors [{n},*], got {tuple(frac.shape)} and "
+                         f"{tuple(colors.shape)}")
+    out = torch.empty((n, 3 + num_signals), dtype=torch.float32, device=frac.device)
+    with torch.cuda.device(frac.device):
+        status = _lib.lib().s3d_window_signals(
+            index.w_w_id.data_ptr(), index.n2n.data_ptr(), frac.data_ptr(),
+            colors.data_ptr() if num_signals > 0 else None, colors.stride(0) if num_signals > 0 else 0,
+            int(num_signals), int(index.window_size), float(xyz_scale), float(other_scale), out.data_ptr(), n,
+            torch.cuda.current_stream(frac.device).cuda_stream)
+    _lib.check(status, "s3d_window_signals")
+    return out
 
 
 def sparse_self_attention(w_w_id, w_sizes, protocol="v1"):
@@ -107,9 +145,12 @@ def get_index01(coords, stride, window_size, local_xyz, colors, shift=0, materia
     materialize_pairs is set.
     """
     index = build_window_index(coords, stride, window_size, shift)
-    order = index.n2n.long()
-    n_xyz = index.local_xyz().to(torch.float32) + local_xyz.to(torch.float32)[order]
-    n_coords = torch.cat([n_xyz, colors.to(torch.float32)[order]], dim=1).contiguous()
+    return index_arguments(index, local_xyz, colors, materialize_pairs)
+
+
+def index_arguments(index, local_xyz, colors, materialize_pairs=False):
+    """The argument tuple of get_index01 for an index that is already built."""
+    n_coords = window_signals(index, local_xyz, colors)
     x_offset = y_offset = m2w = w2m = None
     if materialize_pairs:
         x_offset, y_offset, m2w, _, _, w2m = sparse_self_attention(index.w_w_id, index.w_sizes, "v2")

@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_knn",
+    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_window_signals", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -101,3 +101,14 @@ def test_kernel_choice_is_reported(hip_lib):
     sizes = crse.crse_table_sizes(10, 4, 6, 8, "XYZ")          # 80-row tables: generic kernel
     c_sizes = (ctypes.c_int32 * 3)(*sizes)
     assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, 3, 6, 8, 1, 256000, 1000) == 0
+
+
+def test_window_signals_rejects_bad_arguments(hip_lib):
+    """Argument checks run before anything touches the GPU."""
+    import ctypes
+    f = ctypes.c_float
+    assert hip_lib.s3d_window_signals(None, None, None, None, 0, 0, 5, f(1), f(1), None, 0, None) == 0     # N = 0
+    assert hip_lib.s3d_window_signals(None, None, None, None, 0, 0, 5, f(1), f(1), None, 4, None) < 0      # null pointers
+    assert hip_lib.s3d_window_signals(None, None, None, None, 2, 6, 5, f(1), f(1), None, 4, None) < 0      # stride < columns
+    assert hip_lib.s3d_window_signals(None, None, None, None, 0, 0, 11, f(1), f(1), None, 4, None) < 0     # window > 10
+    assert b"s3d_window_signals" in hip_lib.s3d_last_error_string()

@@ -91,3 +91,38 @@ def test_get_index01_matches_reference_formulas(oracle_lib, hip_lib):
     np.testing.assert_array_equal(y_off.cpu().numpy(), o_y)
     np.testing.assert_array_equal(m2w.cpu().numpy(), o_m2w)
     np.testing.assert_array_equal(w2m.cpu().numpy(), o_w2m)
+
+
+@pytest.mark.parametrize("num_signals", [0, 3, 6])
+def test_window_signals_match_the_tensor_statement(hip_lib, num_signals):
+    """The fused signal-matrix kernel against the reference's tensor statements (window-local voxel + fraction,
+    other signals appended, gathered into sorted order; then the quantiser scales): bit-exact, with the signals
+    given as a strided column slice as the encoder does."""
+    import swin3d_amd
+    rng = np.random.default_rng(7)
+    ws, quant = 7, 4
+    coords = torch.from_numpy(random_scene(rng, 6000, extent=(30, 30, 10), batches=2, stride=2)).cuda()
+    table = torch.from_numpy(rng.uniform(-1, 1, (6000, 10)).astype(np.float32)).cuda()
+    frac, colors = table[:, 1:4].contiguous(), table[:, 4:4 + num_signals]
+    index = swin3d_amd.build_window_index(coords, 2, ws, 3)
+    order = index.n2n.long()
+    ref = torch.cat([index.local_xyz().float() + frac[order], colors[order]], 1)
+    got = swin3d_amd.window_signals(index, frac, colors)
+    assert torch.equal(got, ref)
+    scale = torch.tensor([quant] * 3 + [2 * quant] * num_signals, dtype=torch.float32, device="cuda")
+    got = swin3d_amd.window_signals(index, frac, table[:, 4:], num_signals, quant, 2 * quant)
+    assert torch.equal(got, ref * scale)
+
+
+def test_several_window_sets_in_one_call(oracle_lib, hip_lib):
+    """build_window_indices enqueues all sets before its one host wait; each equals its single build."""
+    import swin3d_amd
+    rng = np.random.default_rng(8)
+    coords = random_scene(rng, 4000, extent=(30, 30, 10), batches=2, stride=1)
+    sets = swin3d_amd.build_window_indices(torch.from_numpy(coords).cuda(), 1, 5, (0, 2))
+    for got, shift in zip(sets, (0, 2)):
+        ref = oracle_lib.window_index(coords, 1, 5, shift)
+        assert got.num_windows == ref["W"] and got.num_pairs == ref["M"]
+        np.testing.assert_array_equal(got.n2n.cpu().numpy(), ref["n2n"])
+        np.testing.assert_array_equal(got.w_sizes.cpu().numpy(), ref["w_sizes"])
+        np.testing.assert_array_equal(got.w2n.cpu().numpy(), ref["w2n"])
