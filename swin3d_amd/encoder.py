@@ -98,6 +98,23 @@ def pool_coordinates(coords, stride, factor):
     """coarse voxel coordinates (floor to the coarse lattice), unique and sorted by (b,x,y,z);
     also the coarse row of every fine voxel."""
     step = stride * factor
+    if coords.is_cuda and 1 <= factor <= 10:
+        # on the GPU a coarse cell is a window of `factor` voxels per side: the window sort gives the cells in the
+        # same ascending (batch, x, y, z) order, one host wait, a third of the time of unique + scatter
+        try:
+            index = build_window_indices(coords, stride, factor, (0,))[0]
+        except ValueError:          # coordinates outside the window sort's range
+            index = None
+        if index is not None:
+            n = coords.shape[0]
+            rows = index.n2n.long()
+            members = coords[rows[index.w2n.long()]]            # one voxel of every cell
+            members[:, 1:] = torch.div(members[:, 1:], step, rounding_mode="floor") * step
+            cell_of_sorted = torch.repeat_interleave(torch.arange(index.num_windows, device=coords.device),
+                                                     index.w_sizes.long(), output_size=n)
+            inverse = torch.empty(n, dtype=torch.long, device=coords.device)
+            inverse[rows] = cell_of_sorted
+            return members, inverse
     coarse = coords.clone()
     coarse[:, 1:] = torch.div(coords[:, 1:], step, rounding_mode="floor") * step
     keys = pack_coords(coarse)
@@ -123,8 +140,12 @@ def pick_cell_representatives(signals, cell_of_row, num_cells):
     return pick
 
 
-def segment_offsets(batch_column):
-    """cumulative END row of every batch element, int32 (what the KNN op takes)."""
+def segment_offsets(batch_column, num_batches=None):
+    """cumulative END row of every batch element, int32 (what the KNN op takes).  With `num_batches` given the
+    host does not wait for the device (batch ids are ascending: the end of batch b is a binary search)."""
+    if num_batches is not None:
+        ids = torch.arange(num_batches, dtype=batch_column.dtype, device=batch_column.device)
+        return torch.searchsorted(batch_column.contiguous(), ids, right=True).to(torch.int32)
     counts = torch.bincount(batch_column.long())
     return torch.cumsum(counts, 0).to(torch.int32)
 
@@ -161,7 +182,7 @@ class GridKNNDownsample(nn.Module):
         self.norm = nn.LayerNorm(in_channels)
         self.linear = nn.Linear(in_channels, out_channels, bias=False)
 
-    def plan(self, coords, stride, signals):
+    def plan(self, coords, stride, signals, num_batches=None):
         """The part that depends on coordinates and signals only: (coarse coordinates, coarse signals, the K
         nearest fine rows of every coarse voxel)."""
         coarse, cell_of_row = pool_coordinates(coords, stride, self.factor)
@@ -169,7 +190,8 @@ class GridKNNDownsample(nn.Module):
         coarse_signals = signals[pick]
         src_xyz = signals[:, 1:4].contiguous().float()
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()
-        idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(coords[:, 0]), segment_offsets(coarse[:, 0]))
+        idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(coords[:, 0], num_batches),
+                           segment_offsets(coarse[:, 0], num_batches))
         return coarse, coarse_signals, idx.view(-1).long().clamp_(min=0)
 
     def forward(self, voxels, signals, plan=None):
@@ -292,7 +314,7 @@ class Stage(nn.Module):
             [SwinBlock(dim, num_heads, window_size, quant_size, cRSE=cRSE, fp16_mode=fp16_mode) for _ in range(depth)])
         self.downsample = GridKNNDownsample(dim, out_channels or dim * 2, stride=down_stride) if downsample else None
 
-    def plan(self, coords, stride, signals):
+    def plan(self, coords, stride, signals, num_batches=None):
         """Everything of the stage that depends on coordinates and signals only: the two window index sets
         (regular and shifted windows) with their scaled signals, and the downsample's geometry.  This is where
         the host waits for the device (window counts, unique cells); `forward` with a plan does not."""
@@ -307,7 +329,7 @@ class Stage(nn.Module):
             attn = self.blocks[0].attn
             args = [tuple(a) + (window_signals(index, local, extra, crse_num_axes(attn.cRSE) - 3, attn.quant_size,
                                                2 * attn.quant_size),) for a, index in zip(args, indices)]
-        down = self.downsample.plan(coords, stride, signals) if self.downsample is not None else None
+        down = self.downsample.plan(coords, stride, signals, num_batches) if self.downsample is not None else None
         return args, down
 
     def forward(self, voxels, signals, plan=None):
@@ -335,8 +357,9 @@ def geometry_steps(stem_coords, stride, signals, layers):
     convolution's neighbour rows, then the plan of every stage (finest first).  None of it depends on features."""
     yield conv3x3x3_neighbours(stem_coords, stride)
     coords = stem_coords
+    num_batches = int(coords[-1, 0]) + 1 if coords.shape[0] else 0    # batch ids are ascending: one read
     for layer in layers:
-        plan = layer.plan(coords, stride, signals)
+        plan = layer.plan(coords, stride, signals, num_batches)
         yield plan
         if plan[1] is not None:
             coords, signals = plan[1][0], plan[1][1]

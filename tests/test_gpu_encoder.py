@@ -166,3 +166,19 @@ def test_window_attention_module_argument_prep(oracle_lib, hip_lib):
     np.testing.assert_allclose(got_xyz, dtk[: 3 * rows_xyz * dim], rtol=1e-3, atol=1e-4 * np.abs(dtk).max())
     got_norm = f64(attn.value_norm_table.grad).reshape(-1)
     np.testing.assert_allclose(got_norm, dtv[-got_norm.size:], rtol=1e-3, atol=1e-4 * np.abs(dtv).max())
+
+
+@pytest.mark.parametrize("stride,factor", [(1, 2), (2, 2), (4, 3)])
+def test_cell_pooling_on_the_gpu_matches_the_host_statement(hip_lib, stride, factor):
+    """On the GPU the coarse cells come from the window sort (a cell is a window of `factor` voxels); the host
+    statement is unique + scatter.  Same cells in the same order, same cell of every row; segment offsets with
+    the batch count given (no host wait) equal the bincount statement."""
+    from conftest import random_scene
+    rng = np.random.default_rng(9)
+    coords = torch.from_numpy(random_scene(rng, 5000, extent=(20, 20, 8), batches=3, stride=stride))
+    ref_coarse, ref_inverse = encoder.pool_coordinates(coords, stride, factor)
+    got_coarse, got_inverse = encoder.pool_coordinates(coords.cuda(), stride, factor)
+    assert torch.equal(got_coarse.cpu(), ref_coarse) and torch.equal(got_inverse.cpu(), ref_inverse)
+    column = got_coarse[:, 0]
+    assert torch.equal(encoder.segment_offsets(column, 3), encoder.segment_offsets(column))
+    assert torch.equal(encoder.segment_offsets(column, 5).cpu()[3:], torch.full((2,), column.numel(), dtype=torch.int32))
