@@ -287,6 +287,30 @@ def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, hea
     _check(oracle_lib, case, dtype)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes(oracle_lib, hip_lib, seed):
+    """Randomly drawn shapes: odd and even head counts (one or two heads per wavefront in the sweep kernel), both
+    head_dims, 3 / 6 / 9 axes, sparse to dense windows (all unit kinds, split and unsplit windows), several batch
+    elements, strides and window shifts; fp32 on even seeds, fp16 (both kernels) on odd ones."""
+    rng = np.random.default_rng(1000 + seed)
+    ws = int(rng.choice([3, 5, 7]))
+    heads = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 12]))
+    dim = int(rng.choice([8, 16]))
+    cRSE = str(rng.choice(["XYZ", "XYZ_RGB", "XYZ_RGB_NORM"]))
+    stride = int(rng.choice([1, 2, 4]))
+    shift = int(rng.choice([0, ws // 2]))
+    batches = int(rng.integers(1, 4))
+    half = tuple(int(v) for v in rng.integers(3, 9, size=3))         # half extent of the box in voxels
+    capacity = batches * 8 * half[0] * half[1] * half[2]
+    n = int(capacity * rng.uniform(0.05, 0.75))
+    case = make_attn_case(oracle_lib, seed=1000 + seed, n=n, ws=ws, quant=4, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=half, batches=batches, stride=stride, shift=shift, recipe="sharp")
+    dtype = torch.float32 if seed % 2 == 0 else torch.float16
+    if dtype == torch.float16:
+        _sharp16(case)
+    _check(oracle_lib, case, dtype)
+
+
 def test_empty_input(hip_lib):
     import swin3d_amd
     dev = torch.device("cuda")

@@ -122,6 +122,27 @@ def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, hea
     _check(oracle_lib, case, dtype)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_shapes(oracle_lib, hip_lib, seed):
+    """Randomly drawn shapes: head counts that do and do not divide the grid of workgroups evenly, both
+    head_dims (VALU and MFMA table-gradient updates), 3 / 6 / 9 axes, sparse to dense windows (every size class of
+    the unit list), several batch elements, strides and window shifts; fp32 on even seeds, fp16 on odd ones."""
+    rng = np.random.default_rng(2000 + seed)
+    ws = int(rng.choice([3, 5, 7]))
+    heads = int(rng.choice([1, 2, 3, 5, 6, 7]))
+    dim = int(rng.choice([8, 16]))
+    cRSE = str(rng.choice(["XYZ", "XYZ_RGB", "XYZ_RGB_NORM"]))
+    stride = int(rng.choice([1, 2, 4]))
+    shift = int(rng.choice([0, ws // 2]))
+    batches = int(rng.integers(1, 4))
+    half = tuple(int(v) for v in rng.integers(3, 8, size=3))         # half extent of the box in voxels
+    capacity = batches * 8 * half[0] * half[1] * half[2]
+    n = int(capacity * rng.uniform(0.05, 0.75))
+    case = make_attn_case(oracle_lib, seed=2000 + seed, n=n, ws=ws, quant=4, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=half, batches=batches, stride=stride, shift=shift, recipe="layer")
+    _check(oracle_lib, case, torch.float32 if seed % 2 == 0 else torch.float16, seed=seed)
+
+
 def test_single_voxel_windows(oracle_lib, hip_lib):
     coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
     case = make_attn_case(oracle_lib, seed=64, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")
