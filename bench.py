@@ -299,11 +299,29 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3):
             outs = model(vox, sig)
             torch.cuda.synchronize()
             times.append((time.perf_counter() - t0) * 1e3)
-    return {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
-            "voxels_per_stage": [int(o.coords.shape[0]) for o in outs],
-            "finite": bool(all(torch.isfinite(o.feats).all().item() for o in outs)),
-            "config": "Swin3D-L channels [80,160,320,640,640] heads [10,10,20,40,40] depths [2,4,9,4,4] "
-                      "windows [5,7,7,7,7] quant 4 cRSE XYZ_RGB_NORM, batch of 2 rooms"}
+    result = {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
+              "voxels_per_stage": [int(o.coords.shape[0]) for o in outs],
+              "finite": bool(all(torch.isfinite(o.feats).all().item() for o in outs)),
+              "config": "Swin3D-L channels [80,160,320,640,640] heads [10,10,20,40,40] depths [2,4,9,4,4] "
+                        "windows [5,7,7,7,7] quant 4 cRSE XYZ_RGB_NORM, batch of 2 rooms"}
+    # the whole segmentation network on the same input: encoder + KNN-interpolation decoder with one attention
+    # block per level + classifier
+    del model, outs
+    torch.manual_seed(0)
+    unet = encoder.Swin3DUNet(**encoder.SWIN3D_L, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=2,
+                              upsample="linear_attn", num_classes=13).to(dev).eval()
+    times = []
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        logits = unet(vox, sig)
+        torch.cuda.synchronize()
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            logits = unet(vox, sig)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+    result["unet_ms"] = float(np.median(times))
+    result["unet_finite"] = bool(torch.isfinite(logits).all().item())
+    return result
 
 
 def cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m):

@@ -320,8 +320,9 @@ class Stage(nn.Module):
         the host waits for the device (window counts, unique cells); `forward` with a plan does not."""
         local = (signals[:, 1:4].float() - coords[:, 1:].float()) / stride
         extra = signals[:, 4:].float()
-        # both window sets are enqueued before the host waits for their window counts
-        indices = build_window_indices(coords, stride, self.window_size, (0, self.window_size // 2))
+        # both window sets (one, for a single block) are enqueued before the host waits for their window counts
+        shifts = (0, self.window_size // 2)[:max(1, min(2, len(self.blocks)))]
+        indices = build_window_indices(coords, stride, self.window_size, shifts)
         args = [index_arguments(index, local, extra) for index in indices]
         if len(self.blocks) > 0:
             # the quantiser scaling of the signals is the same for every block of the stage: once per index set,
@@ -340,11 +341,11 @@ class Stage(nn.Module):
         if len(self.blocks) > 0 and self.blocks[0]._fused_path(feats):
             pending = None
             for i, block in enumerate(self.blocks):
-                feats, pending = block.forward_fused(feats, pending, args[i % 2])
+                feats, pending = block.forward_fused(feats, pending, args[i % len(args)])
             feats = feats + pending
         else:
             for i, block in enumerate(self.blocks):
-                feats = block(feats, args[i % 2])
+                feats = block(feats, args[i % len(args)])
         voxels = voxels.with_feats(feats)
         if self.downsample is None:
             return voxels, voxels, signals
@@ -435,8 +436,10 @@ class Upsample(nn.Module):
             self.block = Stage(out_channels, 1, num_heads, window_size, quant_size, downsample=False, cRSE=cRSE,
                                fp16_mode=fp16_mode)
 
-    def forward(self, voxels, signals, voxels_up, signals_up):
-        """(voxels, signals): the coarse level; (voxels_up, signals_up): the finer level it feeds."""
+    def forward(self, voxels, signals, voxels_up, signals_up, plan_up=None):
+        """(voxels, signals): the coarse level; (voxels_up, signals_up): the finer level it feeds.  plan_up: a
+        stage plan of the finer level's voxel set with the same window size (the encoder's, whose regular window
+        set is the one this level's attention block needs), so that the index is not built a second time."""
         xyz = signals[:, 1:4].detach().contiguous().float()
         support_xyz = signals_up[:, 1:4].detach().contiguous().float()
         feats = self.linear1(voxels_up.feats) + knn_linear_interpolation(
@@ -444,7 +447,9 @@ class Upsample(nn.Module):
             segment_offsets(voxels_up.coords[:, 0]), K=self.up_k)
         voxels_up = voxels_up.with_feats(feats.float())
         if self.attn:
-            voxels_up, _, _ = self.block(voxels_up, signals_up)
+            if plan_up is not None:
+                plan_up = (plan_up[0][:1], None)      # the regular window set; nothing to downsample here
+            voxels_up, _, _ = self.block(voxels_up, signals_up, plan_up)
         return voxels_up
 
 
@@ -510,9 +515,10 @@ class Swin3DUNet(nn.Module):
             levels.append((here, signals))
             voxels, signals = voxels_next, signals_next
         voxels, signals = levels.pop()
-        for upsample in self.upsamples:
+        for level, upsample in zip(range(len(levels) - 1, -1, -1), self.upsamples):
             voxels_up, signals_up = levels.pop()
-            voxels = upsample(voxels, signals, voxels_up, signals_up)
+            # the decoder level works on the encoder level's voxels with the same window size: same window index
+            voxels = upsample(voxels, signals, voxels_up, signals_up, plans[level])
             signals = signals_up
         return self.classifier(voxels.feats.float())
 
