@@ -239,6 +239,19 @@ int s3d_knn(int32_t K, const float *src_xyz, int64_t Ns, const float *query_xyz,
  * LAST source row there, with a weight of about 2e-5); a query with no neighbour at all gets zeros.
  * Accumulation is fp32, one rounding to `dtype`.
  */
+/*
+ * Channel-wise maximum of the source features over the K nearest sources of every query, from the result of s3d_knn.
+ *
+ * Replaces the gather + max of the KNN downsample (Swin3D/modules/swin3d_layers.py:292-312: query_knn_feature
+ * builds [Nq,K,C], then max over K) with one kernel that never writes the gathered copies:
+ *   out[q][c] = max_i src_feat[max(idx[q][i], 0)][c]
+ * A slot padded with row -1 reads row 0, exactly as the clamped index of the tensor statement does.
+ *   idx        device int32 [Nq,K] as written by s3d_knn
+ *   src_feat   device [Ns,C] of `dtype` (Ns >= 1)        out   device [Nq,C] of `dtype`
+ */
+int s3d_knn_max_pool(const int32_t *idx, int32_t K, int64_t Nq, const void *src_feat, int64_t Ns, int32_t C,
+                     int32_t dtype, void *out, void *stream);
+
 int s3d_knn_interpolate(const int32_t *idx, const float *dist2, int32_t K, int64_t Nq, const void *src_feat,
                         int64_t Ns, int32_t C, int32_t dtype, void *out, void *stream);
 

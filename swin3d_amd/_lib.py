@@ -41,6 +41,7 @@ SIGNATURES = {
     "s3d_knn": (ctypes.c_int, [_i32, _vp, _i64, _vp, _i64, _vp, _vp, _i32, _vp, _vp, ctypes.c_float,
                                _vp, ctypes.c_size_t, _vp]),
     "s3d_knn_interpolate": (ctypes.c_int, [_vp, _vp, _i32, _i64, _vp, _i64, _i32, _i32, _vp, _vp]),
+    "s3d_knn_max_pool": (ctypes.c_int, [_vp, _i32, _i64, _vp, _i64, _i32, _i32, _vp, _vp]),
     "s3d_add_layernorm": (ctypes.c_int, [_vp, _vp, _i32, _vp, _vp, ctypes.c_float, _vp, _vp, _i32, _i64, _i32, _vp]),
 }
 

@@ -472,8 +472,76 @@ int launch_interpolate(const int32_t *idx, const float *dist2, int K, int64_t Nq
     return S3D_OK;
 }
 
+// Channel-wise maximum over the K nearest sources of every query (the max-pool of the KNN downsample,
+// Swin3D/modules/swin3d_layers.py:292-312: gather [Nq,K,C], then max over K) without the gathered intermediate.
+// One thread per (query, 16 bytes of channels).  A padded slot (row -1) reads row 0, as the clamped gather of
+// the tensor statement does.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kThreads) void knn_max_pool_kernel(const int32_t *__restrict__ idx, int K, int64_t Nq,
+                                                                const T *__restrict__ feat, int C,
+                                                                T *__restrict__ out)
+{
+    const int groups = C / VEC;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= Nq * groups) return;
+    const int64_t qi = t / groups;
+    const int c0 = static_cast<int>(t - qi * groups) * VEC;
+    T best[VEC];
+    for (int i = 0; i < K; ++i) {
+        const int row = max(idx[qi * K + i], 0);
+        T v[VEC];
+        if constexpr (VEC * sizeof(T) == 16)
+            *reinterpret_cast<uint4 *>(v) = *reinterpret_cast<const uint4 *>(feat + static_cast<int64_t>(row) * C + c0);
+        else
+            v[0] = feat[static_cast<int64_t>(row) * C + c0];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) best[e] = (i == 0 || v[e] > best[e]) ? v[e] : best[e];
+    }
+    if constexpr (VEC * sizeof(T) == 16)
+        *reinterpret_cast<uint4 *>(out + qi * C + c0) = *reinterpret_cast<const uint4 *>(best);
+    else
+        out[qi * C + c0] = best[0];
+}
+
+template <typename T>
+int launch_max_pool(const int32_t *idx, int K, int64_t Nq, const void *feat, int C, void *out, hipStream_t s)
+{
+    const T *f = static_cast<const T *>(feat);
+    T *o = static_cast<T *>(out);
+    constexpr int kVec = 16 / static_cast<int>(sizeof(T));
+    if (C % kVec == 0 && reinterpret_cast<uintptr_t>(feat) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+        const int64_t threads = Nq * (C / kVec);
+        hipLaunchKernelGGL((knn_max_pool_kernel<T, kVec>), dim3(static_cast<unsigned>(ceil_div(threads, kThreads))),
+                           dim3(kThreads), 0, s, idx, K, Nq, f, C, o);
+    } else {
+        const int64_t threads = Nq * C;
+        hipLaunchKernelGGL((knn_max_pool_kernel<T, 1>), dim3(static_cast<unsigned>(ceil_div(threads, kThreads))),
+                           dim3(kThreads), 0, s, idx, K, Nq, f, C, o);
+    }
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
 }  // namespace
 }  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) int s3d_knn_max_pool(const int32_t *idx, int32_t K, int64_t Nq,
+                                                                        const void *src_feat, int64_t Ns, int32_t C,
+                                                                        int32_t dtype, void *out, void *stream)
+{
+    using namespace s3d;
+    if (K < 1 || K > S3D_KNN_KMAX) return fail(S3D_ERR_BAD_SHAPE, "s3d_knn_max_pool: K=%d outside 1..%d", K, S3D_KNN_KMAX);
+    if (Nq < 0 || Ns < 0 || C < 1 || Nq * static_cast<int64_t>(C) > 0x3fffffffffLL || (Nq > 0 && Ns < 1))
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_knn_max_pool: Nq=%lld Ns=%lld C=%d out of range", (long long)Nq, (long long)Ns,
+                    C);
+    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
+        return fail(S3D_ERR_BAD_DTYPE, "s3d_knn_max_pool: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    if (Nq == 0) return S3D_OK;
+    if (!idx || !out || !src_feat) return fail(S3D_ERR_NULL_POINTER, "s3d_knn_max_pool: null device pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == S3D_DTYPE_F16 ? launch_max_pool<_Float16>(idx, K, Nq, src_feat, C, out, s)
+                                  : launch_max_pool<float>(idx, K, Nq, src_feat, C, out, s);
+}
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_knn_workspace_bytes(int64_t Ns, int64_t Nq, int32_t B)
 {

@@ -29,7 +29,7 @@ import torch.nn.functional as F
 from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
 from .fused_norm import add_layernorm
 from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
-from .sparse_dl.knn import KNN, KNNInterpolate, knn_query
+from .sparse_dl.knn import KNN, KNNInterpolate, knn_max_pool, knn_query
 from .window_index import build_window_indices, get_index01, index_arguments, window_signals
 
 
@@ -192,10 +192,10 @@ class GridKNNDownsample(nn.Module):
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()
         idx, _ = KNN.apply(self.k, src_xyz, qry_xyz, segment_offsets(coords[:, 0], num_batches),
                            segment_offsets(coarse[:, 0], num_batches))
-        return coarse, coarse_signals, idx.view(-1).long().clamp_(min=0)
+        return coarse, coarse_signals, idx
 
     def forward(self, voxels, signals, plan=None):
-        coarse, coarse_signals, rows = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
+        coarse, coarse_signals, idx = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
         # LayerNorm and Linear act on single rows, so they commute with the gather: project the Ns fine rows once
         # instead of the K * Nq gathered copies (the reference statement, swin3d_layers.py:292-312, gathers first)
         if _fused_norm_applies(voxels.feats):
@@ -203,8 +203,11 @@ class GridKNNDownsample(nn.Module):
         else:
             normed = self.norm(voxels.feats)
         projected = self.linear(normed)
-        grouped = projected[rows].view(coarse.shape[0], self.k, projected.shape[1])
-        feats = grouped.amax(dim=1)
+        if not torch.is_grad_enabled() and projected.is_cuda and projected.dtype in (torch.float16, torch.float32):
+            feats = knn_max_pool(idx, projected)      # one kernel, no [Nq, K, C] intermediate
+        else:
+            rows = idx.view(-1).long().clamp_(min=0)
+            feats = projected[rows].view(coarse.shape[0], self.k, projected.shape[1]).amax(dim=1)
         return SparseVoxels(coarse, feats.float(), voxels.stride * self.factor), coarse_signals
 
 

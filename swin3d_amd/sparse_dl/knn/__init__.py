@@ -1,3 +1,3 @@
-from .knn import KNN, KNNInterpolate, knn_interpolate, knn_query
+from .knn import KNN, KNNInterpolate, knn_interpolate, knn_max_pool, knn_query
 
-__all__ = ["KNN", "KNNInterpolate", "knn_interpolate", "knn_query"]
+__all__ = ["KNN", "KNNInterpolate", "knn_interpolate", "knn_max_pool", "knn_query"]

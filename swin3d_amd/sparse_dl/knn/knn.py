@@ -89,6 +89,29 @@ def knn_interpolate(idx, dist2, src_feat):
     return out
 
 
+def knn_max_pool(idx, src_feat):
+    """Channel-wise maximum of src_feat [Ns,C] over the K nearest sources of every query (idx int32 [Nq,K] of a
+    knn_query result) -> [Nq,C] in the dtype of src_feat: the gather + max of the KNN downsample
+    (Swin3D/modules/swin3d_layers.py:292-312) without the [Nq,K,C] intermediate.  Padded slots (row -1) read
+    row 0, as the clamped gather does.  No autograd (inference)."""
+    if not (idx.is_cuda and src_feat.is_cuda):
+        raise RuntimeError("idx and src_feat must be CUDA (HIP) tensors")
+    if idx.dtype != torch.int32 or idx.dim() != 2:
+        raise ValueError("idx must be int32 [Nq,K]")
+    if src_feat.dim() != 2 or src_feat.dtype not in _FEAT_DTYPE:
+        raise ValueError(f"src_feat must be float16/float32 [Ns,C], got {src_feat.dtype} {tuple(src_feat.shape)}")
+    idx, src_feat = idx.contiguous(), src_feat.contiguous()
+    nq, k = idx.shape
+    ns, c = src_feat.shape
+    out = torch.empty((nq, c), dtype=src_feat.dtype, device=src_feat.device)
+    with torch.cuda.device(src_feat.device):
+        stream = torch.cuda.current_stream(src_feat.device).cuda_stream
+        status = _lib.lib().s3d_knn_max_pool(idx.data_ptr(), k, nq, src_feat.data_ptr(), ns, c,
+                                             _FEAT_DTYPE[src_feat.dtype], out.data_ptr(), stream)
+    _lib.check(status, "s3d_knn_max_pool")
+    return out
+
+
 class KNNInterpolate(Function):
     """Differentiable (w.r.t. the features) inverse-distance interpolation; the forward is the fused
     HIP kernel, the backward scatters the weighted output gradient back with torch's index_add_."""

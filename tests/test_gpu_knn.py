@@ -157,3 +157,21 @@ def test_interpolate_autograd(oracle_lib, hip_lib):
     weights = oracle_lib.knn_interpolate(idx.cpu().numpy(), d2.cpu().numpy(), basis)     # [700,300]
     ref = weights.T @ dout.astype(np.float64)
     np.testing.assert_allclose(feat.grad.double().cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("channels", [160, 37])
+def test_max_pool_over_neighbours_matches_gather_and_max(hip_lib, dtype, channels):
+    """s3d_knn_max_pool against the tensor statement (clamped gather to [Nq,K,C], max over K): bit-exact, with
+    padded slots (segments with fewer than K sources) in the index."""
+    from swin3d_amd.sparse_dl.knn import knn_max_pool, knn_query
+    rng = np.random.default_rng(12)
+    src = torch.from_numpy(rng.uniform(0, 10, (3000, 3)).astype(np.float32)).cuda()
+    qry = torch.from_numpy(rng.uniform(0, 10, (700, 3)).astype(np.float32)).cuda()
+    so = torch.tensor([2990, 3000], dtype=torch.int32).cuda()      # second segment: 10 sources for K = 16
+    qo = torch.tensor([600, 700], dtype=torch.int32).cuda()
+    idx, _ = knn_query(16, src, qry, so, qo)
+    assert int((idx < 0).sum()) == 100 * 6
+    feat = torch.from_numpy(rng.standard_normal((3000, channels)).astype(np.float32)).cuda().to(dtype)
+    ref = feat[idx.view(-1).long().clamp(min=0)].view(700, 16, channels).amax(dim=1)
+    assert torch.equal(knn_max_pool(idx, feat), ref)
