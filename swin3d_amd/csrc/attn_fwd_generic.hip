@@ -653,7 +653,7 @@ int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels)
 
 size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels)
 {
-    // queue counters, the unit count, the unit descriptors, and one partial record per (key block, head,
+    // queue counters, the totals, the unit list and sorted window list, and one partial record per (key block, head,
     // voxel) when some window may be split along its keys
     const int blocks = attn_generic_key_blocks(H, N, W, max_window_voxels);
     const size_t partials = blocks <= 1 ? 0 : sizeof(float) * static_cast<size_t>(N) * blocks * H * (D + 2);

@@ -30,8 +30,10 @@ struct AttnArgs {
     int32_t padded_rows;                   // row stride of the transposed value table
 };
 
-// Persistent workgroups, one head each with its table slices in LDS; lane = query, keys streamed; VALU math,
-// any dtype.  Needs a.workspace (work queues, unit list), a.partials and a.max_key_tiles (key blocks of 64).
+// Persistent workgroups, one head (or pair of heads) each with its table slices in LDS; lane = one query of some
+// window, which streams that window's keys; VALU math, any dtype.  Needs a.workspace (work queues, sorted window
+// list, unit list), a.partials, a.block_shift (key blocks of 64 << shift keys) and a.max_key_tiles (key blocks of
+// the largest window).
 int attn_generic_block_shift(int H, int64_t N, int64_t W, int max_window_voxels);
 int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels);
 size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels);
