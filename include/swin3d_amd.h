@@ -180,6 +180,21 @@ int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t w
                      int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Rows of the lattice neighbours of every voxel, from the voxels' sorted packed keys.
+ *
+ * A packed coordinate key is linear in (batch, x, y, z), so a neighbour's key is the voxel's key plus a constant
+ * per offset.  Used for the 27 offsets of the stem's 3x3x3 sparse convolution (the reference takes the kernel map
+ * from MinkowskiEngine, Swin3D/models/Swin3D.py:75-86); no counterpart kernel in the reference.
+ *
+ *   sorted_keys  device int64 [N] ascending, distinct      order  device int64 [N]: order[i] = row of sorted_keys[i]
+ *   deltas       device int64 [M] key offsets (1 <= M <= 1024)
+ *   out          device int64 [N,M]: out[order[i]][d] = order[p] with sorted_keys[p] = sorted_keys[i] + deltas[d],
+ *                or N when no voxel has that key
+ */
+int s3d_key_neighbours(const int64_t *sorted_keys, const int64_t *order, int64_t N, const int64_t *deltas, int32_t M,
+                       int64_t *out, void *stream);
+
+/*
  * Signal matrix of the attention op in window-sorted order (the `n_coords` argument of s3d_attn_fwd), one pass.
  *
  * Replaces the tensor statements of BasicLayer.get_index01 (Swin3D/modules/swin3d_layers.py:800-804: window-local

@@ -182,8 +182,47 @@ __global__ __launch_bounds__(kThreads) void window_signals_kernel(
     out[t] = v;
 }
 
+// one thread per (sorted voxel, offset): binary search of key + delta in the sorted keys
+__global__ __launch_bounds__(kThreads) void key_neighbours_kernel(const int64_t *__restrict__ sorted_keys,
+                                                                  const int64_t *__restrict__ order, int64_t N,
+                                                                  const int64_t *__restrict__ deltas, int M,
+                                                                  int64_t *__restrict__ out)
+{
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (t >= N * M) return;
+    const int64_t i = t / M;
+    const int d = static_cast<int>(t - i * M);
+    const int64_t key = sorted_keys[i] + deltas[d];
+    int64_t lo = 0, hi = N;   // first position whose key is not below `key`
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (sorted_keys[mid] < key) lo = mid + 1;
+        else hi = mid;
+    }
+    const bool found = lo < N && sorted_keys[lo] == key;
+    out[order[i] * M + d] = found ? order[lo] : N;
+}
+
 }  // namespace
 }  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) int s3d_key_neighbours(const int64_t *sorted_keys,
+                                                                          const int64_t *order, int64_t N,
+                                                                          const int64_t *deltas, int32_t M,
+                                                                          int64_t *out, void *stream)
+{
+    using namespace s3d;
+    if (N < 0 || M < 1 || M > 1024 || N * static_cast<int64_t>(M) > 0x3fffffffffLL)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_key_neighbours: N=%lld M=%d out of range", (long long)N, M);
+    if (N == 0) return S3D_OK;
+    if (!sorted_keys || !order || !deltas || !out)
+        return fail(S3D_ERR_NULL_POINTER, "s3d_key_neighbours: null device pointer");
+    const dim3 grid(static_cast<unsigned>(ceil_div(N * M, kThreads)));
+    hipLaunchKernelGGL(key_neighbours_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), sorted_keys,
+                       order, N, deltas, M, out);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
 
 extern "C" __attribute__((visibility("default"))) int s3d_window_signals(
     const int32_t *w_w_id, const int32_t *n2n, const float *frac, const float *signals, int64_t signals_stride,

@@ -26,6 +26,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import _lib
 from .crse import crse_num_axes, crse_table_sizes, scale_crse_coords
 from .fused_norm import add_layernorm
 from .sparse_dl.attn.attn_coff import IndexMode, PosEmb, PrecisionMode, SelfAttnAIOFunction, TableDims
@@ -74,6 +75,13 @@ def conv3x3x3_neighbours(coords, stride):
     sorted_keys, order = torch.sort(pack_coords(coords))
     deltas = torch.tensor([((dx << _FIELD) + dy << _FIELD) + dz for dx in (-1, 0, 1) for dy in (-1, 0, 1)
                            for dz in (-1, 0, 1)], dtype=torch.long, device=coords.device) * stride
+    if coords.is_cuda:
+        out = torch.empty((n, 27), dtype=torch.long, device=coords.device)
+        with torch.cuda.device(coords.device):
+            status = _lib.lib().s3d_key_neighbours(sorted_keys.data_ptr(), order.data_ptr(), n, deltas.data_ptr(), 27,
+                                                   out.data_ptr(), torch.cuda.current_stream(coords.device).cuda_stream)
+        _lib.check(status, "s3d_key_neighbours")
+        return out
     queries = sorted_keys.unsqueeze(0) + deltas.unsqueeze(1)                    # [27, N], rows ascending
     pos = torch.searchsorted(sorted_keys, queries).clamp_(max=n - 1)
     rows = torch.where(sorted_keys[pos] == queries, order[pos], torch.full_like(pos, n))

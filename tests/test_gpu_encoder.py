@@ -182,3 +182,16 @@ def test_cell_pooling_on_the_gpu_matches_the_host_statement(hip_lib, stride, fac
     column = got_coarse[:, 0]
     assert torch.equal(encoder.segment_offsets(column, 3), encoder.segment_offsets(column))
     assert torch.equal(encoder.segment_offsets(column, 5).cpu()[3:], torch.full((2,), column.numel(), dtype=torch.int32))
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_stem_neighbour_rows_on_the_gpu_match_the_host_statement(hip_lib, stride):
+    """s3d_key_neighbours (binary search of key + offset in the sorted keys) against the tensor statement that
+    runs on the host: same row, or N, for each of the 27 offsets of every voxel; negative coordinates included."""
+    from conftest import random_scene
+    rng = np.random.default_rng(10)
+    coords = torch.from_numpy(random_scene(rng, 6000, extent=(14, 14, 6), batches=2, stride=stride))
+    ref = encoder.conv3x3x3_neighbours(coords, stride)
+    got = encoder.conv3x3x3_neighbours(coords.cuda(), stride)
+    assert torch.equal(got.cpu(), ref)
+    assert int((ref < coords.shape[0]).sum()) > 27 * 100          # the scene is dense enough to have neighbours
