@@ -180,6 +180,21 @@ int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t w
                      int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Representative voxel of every cell of a window sort: the member whose signal row is nearest (Euclidean, fp32) to
+ * the mean of the cell's signal rows; ties go to the lower row.  With a sort at window = 2 a cell is a coarse voxel
+ * of the stride-2 downsample (GridCoordsDown, Swin3D/modules/swin3d_layers.py:179-231, a chain of scatter
+ * reductions there).  Members are summed in sorted order, so the result is deterministic.
+ *
+ *   n2n, w2n, w_sizes  device int32: outputs of s3d_window_index (W = counts[0] cells)
+ *   signals            device fp32 rows of `signals_stride` floats, original row order; the first `num_signals`
+ *                      columns (1..16) enter the distance
+ *   out                device int64 [W]: the chosen row of every cell
+ */
+int s3d_cell_representatives(const int32_t *n2n, const int32_t *w2n, const int32_t *w_sizes, int64_t W,
+                             const float *signals, int64_t signals_stride, int32_t num_signals, int64_t *out,
+                             void *stream);
+
+/*
  * Rows of the lattice neighbours of every voxel, from the voxels' sorted packed keys.
  *
  * A packed coordinate key is linear in (batch, x, y, z), so a neighbour's key is the voxel's key plus a constant

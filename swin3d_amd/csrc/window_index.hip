@@ -203,8 +203,69 @@ __global__ __launch_bounds__(kThreads) void key_neighbours_kernel(const int64_t 
     out[order[i] * M + d] = found ? order[lo] : N;
 }
 
+// one thread per cell (= window of the sort): mean of the members' signal rows, then the member nearest to it
+constexpr int kMaxCellSignals = 16;
+__global__ __launch_bounds__(kThreads) void cell_representatives_kernel(
+    const int32_t *__restrict__ n2n, const int32_t *__restrict__ w2n, const int32_t *__restrict__ w_sizes, int64_t W,
+    const float *__restrict__ signals, int64_t signals_stride, int S, int64_t *__restrict__ out)
+{
+#pragma clang fp contract(off)
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (w >= W) return;
+    const int begin = w2n[w], size = w_sizes[w];
+    float mean[kMaxCellSignals];
+#pragma unroll
+    for (int c = 0; c < kMaxCellSignals; ++c) mean[c] = 0.0f;
+    for (int p = begin; p < begin + size; ++p) {
+        const float *row = signals + static_cast<int64_t>(n2n[p]) * signals_stride;
+#pragma unroll
+        for (int c = 0; c < kMaxCellSignals; ++c)
+            if (c < S) mean[c] += row[c];
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxCellSignals; ++c) mean[c] /= static_cast<float>(size);
+    float best = INFINITY;
+    int best_row = 0x7fffffff;
+    for (int p = begin; p < begin + size; ++p) {
+        const int r = n2n[p];
+        const float *row = signals + static_cast<int64_t>(r) * signals_stride;
+        float sq = 0.0f;
+#pragma unroll
+        for (int c = 0; c < kMaxCellSignals; ++c) {
+            if (c < S) {
+                const float d = row[c] - mean[c];
+                sq += d * d;
+            }
+        }
+        const float dist = sqrtf(sq);
+        if (dist < best || (dist == best && r < best_row)) {
+            best = dist;
+            best_row = r;
+        }
+    }
+    out[w] = best_row;
+}
+
 }  // namespace
 }  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) int s3d_cell_representatives(
+    const int32_t *n2n, const int32_t *w2n, const int32_t *w_sizes, int64_t W, const float *signals,
+    int64_t signals_stride, int32_t num_signals, int64_t *out, void *stream)
+{
+    using namespace s3d;
+    if (W < 0 || num_signals < 1 || num_signals > kMaxCellSignals || signals_stride < num_signals)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_cell_representatives: W=%lld num_signals=%d (1..%d) signals_stride=%lld",
+                    (long long)W, num_signals, kMaxCellSignals, (long long)signals_stride);
+    if (W == 0) return S3D_OK;
+    if (!n2n || !w2n || !w_sizes || !signals || !out)
+        return fail(S3D_ERR_NULL_POINTER, "s3d_cell_representatives: null device pointer");
+    const dim3 grid(static_cast<unsigned>(ceil_div(W, kThreads)));
+    hipLaunchKernelGGL(cell_representatives_kernel, grid, dim3(kThreads), 0, static_cast<hipStream_t>(stream), n2n, w2n,
+                       w_sizes, W, signals, signals_stride, num_signals, out);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
 
 extern "C" __attribute__((visibility("default"))) int s3d_key_neighbours(const int64_t *sorted_keys,
                                                                           const int64_t *order, int64_t N,

@@ -132,6 +132,34 @@ def pool_coordinates(coords, stride, factor):
     return coarse[first], inverse
 
 
+def pool_and_pick(coords, stride, factor, signals):
+    """(coarse coordinates, representative fine row of every coarse voxel).  On the GPU both come from one window
+    sort at window = factor (a coarse cell is a window) and one kernel over the cells; elsewhere from
+    pool_coordinates and pick_cell_representatives."""
+    sig = signals.float()
+    if coords.is_cuda and 1 <= factor <= 10 and 1 <= sig.shape[1] <= 16:
+        try:
+            index = build_window_indices(coords, stride, factor, (0,))[0]
+        except ValueError:          # coordinates outside the window sort's range
+            index = None
+        if index is not None:
+            step = stride * factor
+            members = coords[index.n2n.long()[index.w2n.long()]]            # one voxel of every cell
+            members[:, 1:] = torch.div(members[:, 1:], step, rounding_mode="floor") * step
+            if sig.stride(1) != 1:
+                sig = sig.contiguous()
+            pick = torch.empty(index.num_windows, dtype=torch.long, device=coords.device)
+            with torch.cuda.device(coords.device):
+                status = _lib.lib().s3d_cell_representatives(
+                    index.n2n.data_ptr(), index.w2n.data_ptr(), index.w_sizes.data_ptr(), index.num_windows,
+                    sig.data_ptr(), sig.stride(0), sig.shape[1], pick.data_ptr(),
+                    torch.cuda.current_stream(coords.device).cuda_stream)
+            _lib.check(status, "s3d_cell_representatives")
+            return members, pick
+    coarse, cell_of_row = pool_coordinates(coords, stride, factor)
+    return coarse, pick_cell_representatives(signals, cell_of_row, coarse.shape[0])
+
+
 def pick_cell_representatives(signals, cell_of_row, num_cells):
     """For every coarse cell the fine row whose signal vector (all columns of the coordinate
     features) is nearest to the cell mean; ties go to the lower row."""
@@ -193,8 +221,7 @@ class GridKNNDownsample(nn.Module):
     def plan(self, coords, stride, signals, num_batches=None):
         """The part that depends on coordinates and signals only: (coarse coordinates, coarse signals, the K
         nearest fine rows of every coarse voxel)."""
-        coarse, cell_of_row = pool_coordinates(coords, stride, self.factor)
-        pick = pick_cell_representatives(signals, cell_of_row, coarse.shape[0])
+        coarse, pick = pool_and_pick(coords, stride, self.factor, signals)
         coarse_signals = signals[pick]
         src_xyz = signals[:, 1:4].contiguous().float()
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()

@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_knn_max_pool", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_window_signals", "s3d_key_neighbours", "s3d_knn",
+    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_knn_max_pool", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_window_signals", "s3d_key_neighbours", "s3d_cell_representatives", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 

@@ -195,3 +195,17 @@ def test_stem_neighbour_rows_on_the_gpu_match_the_host_statement(hip_lib, stride
     got = encoder.conv3x3x3_neighbours(coords.cuda(), stride)
     assert torch.equal(got.cpu(), ref)
     assert int((ref < coords.shape[0]).sum()) > 27 * 100          # the scene is dense enough to have neighbours
+
+
+def test_cell_representatives_on_the_gpu_match_the_host_statement(hip_lib):
+    """s3d_cell_representatives against the host statement (scatter sums, mean, distances, scatter minimum) on
+    signals that are multiples of 1/64, for which every sum is exact whatever its order: same coarse voxels, same
+    representative rows, ties to the lower row."""
+    from conftest import random_scene
+    rng = np.random.default_rng(11)
+    coords = torch.from_numpy(random_scene(rng, 5000, extent=(12, 12, 6), batches=2, stride=2))
+    signals = torch.from_numpy((rng.integers(-64, 65, (5000, 10)) / 64.0).astype(np.float32))
+    signals[:40] = signals[40:80]                      # duplicates: exact ties somewhere
+    ref_coarse, ref_pick = encoder.pool_and_pick(coords, 2, 2, signals)
+    got_coarse, got_pick = encoder.pool_and_pick(coords.cuda(), 2, 2, signals.cuda())
+    assert torch.equal(got_coarse.cpu(), ref_coarse) and torch.equal(got_pick.cpu(), ref_pick)
