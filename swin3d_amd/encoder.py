@@ -132,16 +132,17 @@ def pool_coordinates(coords, stride, factor):
     return coarse[first], inverse
 
 
-def pool_and_pick(coords, stride, factor, signals):
+def pool_and_pick(coords, stride, factor, signals, index=None):
     """(coarse coordinates, representative fine row of every coarse voxel).  On the GPU both come from one window
-    sort at window = factor (a coarse cell is a window) and one kernel over the cells; elsewhere from
-    pool_coordinates and pick_cell_representatives."""
+    sort at window = factor (a coarse cell is a window; `index`, when the caller has built it already) and one
+    kernel over the cells; elsewhere from pool_coordinates and pick_cell_representatives."""
     sig = signals.float()
     if coords.is_cuda and 1 <= factor <= 10 and 1 <= sig.shape[1] <= 16:
-        try:
-            index = build_window_indices(coords, stride, factor, (0,))[0]
-        except ValueError:          # coordinates outside the window sort's range
-            index = None
+        if index is None:
+            try:
+                index = build_window_indices(coords, stride, factor, (0,))[0]
+            except ValueError:          # coordinates outside the window sort's range
+                index = None
         if index is not None:
             step = stride * factor
             members = coords[index.n2n.long()[index.w2n.long()]]            # one voxel of every cell
@@ -218,10 +219,11 @@ class GridKNNDownsample(nn.Module):
         self.norm = nn.LayerNorm(in_channels)
         self.linear = nn.Linear(in_channels, out_channels, bias=False)
 
-    def plan(self, coords, stride, signals, num_batches=None):
+    def plan(self, coords, stride, signals, num_batches=None, cell_index=None):
         """The part that depends on coordinates and signals only: (coarse coordinates, coarse signals, the K
-        nearest fine rows of every coarse voxel)."""
-        coarse, pick = pool_and_pick(coords, stride, self.factor, signals)
+        nearest fine rows of every coarse voxel).  cell_index: the window index at window = stride factor, when
+        the caller built it along with its own."""
+        coarse, pick = pool_and_pick(coords, stride, self.factor, signals, cell_index)
         coarse_signals = signals[pick]
         src_xyz = signals[:, 1:4].contiguous().float()
         qry_xyz = coarse_signals[:, 1:4].contiguous().float()
@@ -359,8 +361,12 @@ class Stage(nn.Module):
         local = (signals[:, 1:4].float() - coords[:, 1:].float()) / stride
         extra = signals[:, 4:].float()
         # both window sets (one, for a single block) are enqueued before the host waits for their window counts
-        shifts = (0, self.window_size // 2)[:max(1, min(2, len(self.blocks)))]
+        shifts = list((0, self.window_size // 2)[:max(1, min(2, len(self.blocks)))])
+        pooled = self.downsample is not None and coords.is_cuda and 1 <= self.downsample.factor <= 10
+        if pooled:
+            shifts.append((self.downsample.factor, 0))      # the downsample's cells: the same host wait
         indices = build_window_indices(coords, stride, self.window_size, shifts)
+        cell_index = indices.pop() if pooled else None
         args = [index_arguments(index, local, extra) for index in indices]
         if len(self.blocks) > 0:
             # the quantiser scaling of the signals is the same for every block of the stage: once per index set,
@@ -368,7 +374,8 @@ class Stage(nn.Module):
             attn = self.blocks[0].attn
             args = [tuple(a) + (window_signals(index, local, extra, crse_num_axes(attn.cRSE) - 3, attn.quant_size,
                                                2 * attn.quant_size),) for a, index in zip(args, indices)]
-        down = self.downsample.plan(coords, stride, signals, num_batches) if self.downsample is not None else None
+        down = (self.downsample.plan(coords, stride, signals, num_batches, cell_index)
+                if self.downsample is not None else None)
         return args, down
 
     def forward(self, voxels, signals, plan=None):

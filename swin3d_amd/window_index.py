@@ -38,9 +38,10 @@ class WindowIndex:
 
 
 def build_window_indices(coords, stride, window_size, shifts):
-    """One WindowIndex per entry of `shifts` (voxels: 0, or window_size // 2 for the shifted window set) for
-    coords int32 [N,4] (batch,x,y,z) on the GPU.  All index builds are enqueued before the host reads the
-    window counts back, so the call synchronises once however many shifts it is given."""
+    """One WindowIndex per entry of `shifts` (voxels: 0, or window_size // 2 for the shifted window set; an entry
+    may also be a pair (window size, shift) for a set with a window size of its own) for coords int32 [N,4]
+    (batch,x,y,z) on the GPU.  All index builds are enqueued before the host reads the window counts back, so
+    the call synchronises once however many sets it is given."""
     if not coords.is_cuda:
         raise RuntimeError("coords must be a CUDA (HIP) tensor")
     if coords.dim() != 2 or coords.shape[1] != 4:
@@ -48,30 +49,29 @@ def build_window_indices(coords, stride, window_size, shifts):
     dev = coords.device
     coords = coords.to(torch.int32).contiguous()
     n = coords.shape[0]
-    shifts = list(shifts)
-    counts = torch.empty((len(shifts), 4), dtype=torch.int64, device=dev)
+    sets = [s if isinstance(s, (tuple, list)) else (window_size, s) for s in shifts]
+    counts = torch.empty((len(sets), 4), dtype=torch.int64, device=dev)
     lib = _lib.lib()
     outputs = []
     with torch.cuda.device(dev):
         ws_bytes = lib.s3d_window_index_workspace_bytes(n)
         stream = torch.cuda.current_stream(dev).cuda_stream
-        for i, shift in enumerate(shifts):
+        for i, (window, shift) in enumerate(sets):
             n2n, wwid, w_sizes, w2n = (torch.empty(n, dtype=torch.int32, device=dev) for _ in range(4))
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window_size), int(shift),
+            status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window), int(shift),
                                           n2n.data_ptr(), wwid.data_ptr(), w_sizes.data_ptr(), w2n.data_ptr(),
                                           counts[i].data_ptr(), workspace.data_ptr(), ws_bytes, stream)
             _lib.check(status, "s3d_window_index")
             outputs.append((n2n, wwid, w_sizes, w2n))
     result = []
-    for (n2n, wwid, w_sizes, w2n), (num_w, num_m, max_w, err) in zip(outputs, counts.tolist()):
+    for (n2n, wwid, w_sizes, w2n), (num_w, num_m, max_w, err), (window, _) in zip(outputs, counts.tolist(), sets):
         if err:
             raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
                              "-8192..8191)")
         sizes = w_sizes[:num_w]
         sizes.max_window_voxels = int(max_w)   # read by the attention op (sizes its partial-result workspace)
-        result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w),
-                                  int(window_size)))
+        result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window)))
     return result
 
 
