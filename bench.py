@@ -26,6 +26,7 @@ HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per s3d_attn_fwd call from the FETCH_SIZE / WRITE_SIZE passes recorded in
 # profiles/attn_fwd_headline.txt (sweep kernel + partial merge + the two list kernels): fetch
 # (58869 + 282 + 212) KiB * 2.00, write (21892 + 98 + 280) KiB * 1.00, factors from the 64 MiB copy
+VALU_ISSUE_FRAC = 0.77   # share of the sweep kernel's clocks in which a SIMD issues a VALU instruction
 MEASURED_TRAFFIC_BYTES = int(((58869 + 282 + 212) * 2.00 + (21892 + 98 + 280) * 1.00) * 1024)
 
 
@@ -147,7 +148,11 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS,
                      "traffic": MEASURED_TRAFFIC_BYTES if args.flags == 0 else None,
-                     "algorithmic_bytes": bytes_alg},
+                     "algorithmic_bytes": bytes_alg,
+                     # what the dominant kernel is bound by instead (constant from the committed profile:
+                     # SQ_INSTS_VALU * 4 clocks / 1024 SIMDs against the kernel's clocks)
+                     "limiter": ({"kind": "valu_issue", "frac": VALU_ISSUE_FRAC,
+                                  "source": "profiles/attn_fwd_headline.txt"} if args.flags == 0 else None)},
     }
 
     # cold figure: a 512 MiB fill between launches evicts q/k/v and the tables from L2 and the
