@@ -1,15 +1,19 @@
 """Swin3D encoder on the swin3d_amd operators, without MinkowskiEngine (inference path).
 
-Everything around the two hot operators is plain PyTorch-ROCm: the sparse voxel set is a pair
-of tensors (`SparseVoxels`), coordinate lookups are sort + searchsorted on packed 64-bit keys,
-dense math (Linear / LayerNorm / GELU, the 27-offset stem convolution as one GEMM) goes to
-hipBLASLt through torch.  Window attention runs through `SelfAttnAIOFunction`, the window index
-through `get_index01`, neighbour gathering through `KNN`.
+The sparse voxel set is a pair of tensors (`SparseVoxels`); dense math (Linear, GELU, the 27-offset stem
+convolution as one GEMM) goes to hipBLASLt through torch.  Window attention runs through
+`SelfAttnAIOFunction`, the window index through `build_window_indices` / `window_signals`, neighbour
+gathering through `KNN` / `knn_max_pool`.  On the GPU the coordinate work runs on the library's kernels too
+(coarse cells and their representatives from the window sort, the stem's neighbour rows by binary search in
+sorted packed keys, the fused add + LayerNorm); the same functions have a tensor statement for host tensors,
+against which the kernels are tested.  The geometry of all stages is computed first (`plan_stages`): it
+needs no features and is the only place where the host waits for the device.
 
 What each piece mirrors in the reference (semantics, not code):
   sparse_conv3x3x3 + BatchNorm + ReLU   MinkConvBNRelu stem            Swin3D/modules/mink_layers.py:50-80
   pool_coordinates                      MinkowskiMaxPooling on coords  Swin3D/modules/swin3d_layers.py:284-286
   pick_cell_representatives             GridCoordsDown                 :179-231
+  pool_and_pick                         the two above on the GPU (window sort + one kernel over the cells)
   segment_offsets                       get_offset                     :234-241
   GridKNNDownsample                     same name                      :272-315
   WindowAttention / SwinBlock / Stage   WindowAttention, SwinTransformerBlock, BasicLayer  :382-871
