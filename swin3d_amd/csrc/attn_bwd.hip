@@ -181,8 +181,9 @@ __global__ void bwd_reset_counters_kernel(BwdArgs a)
 
 // MODE (key-owned sweep only): 0 = dk, dv, dTq, dTv in one sweep - what the library launches: two wavefronts per
 // SIMD at head_dim 8, one at head_dim 16 (up to 512 registers, 192 to 256 of them MFMA accumulation registers
-// for the two sets of table gradients); 1 = dk, dTq and 2 = dv, dTv are the halves of that sweep, which at
-// head_dim 16 measured 3.44 ms as two launches against 2.83 ms fused (the logits are computed once).
+// for the two sets of table gradients); 1 = dk, dTq and 2 = dv, dTv are the halves of that sweep, used at
+// head_dim 16 when the table has more than 384 rows per head; at 360 rows they measured 3.44 ms as two launches
+// against 2.83 ms fused (the logits are computed once).
 // The query-owned sweep produces dq and dTk.
 // BLK: 64-row blocks of the head's flat table (all axes back to back) that the wavefront's
 // table-gradient registers cover; lane l of block m owns flat row 64 m + l.
@@ -631,8 +632,15 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
     hipLaunchKernelGGL(bwd_units_kernel, dim3(1), dim3(1024), 0, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     const int grid = bwd_grid(a.H);
-    // one key-owned sweep for dk, dv and both of its table gradients
-    if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
+    // one key-owned sweep for dk, dv and both of its table gradients; at head_dim 16 with more than six 64-row
+    // blocks of table rows (quant 8) the two sets of accumulation registers no longer fit one wavefront
+    // (250-320 registers spilled) and the sweep runs as its two halves
+    if (D <= 8 || (a.total_rows + 63) / 64 <= 6) {
+        if (int rc = launch_sweep<T, D, ND, true, 0>(a, grid, stream)) return rc;
+    } else {
+        if (int rc = launch_sweep<T, D, ND, true, 1>(a, grid, stream)) return rc;
+        if (int rc = launch_sweep<T, D, ND, true, 2>(a, grid, stream)) return rc;
+    }
     return launch_sweep<T, D, ND, false, 0>(a, grid, stream);
 }
 
