@@ -35,14 +35,14 @@ __host__ __device__ inline int key_block_size(int n, int shift) { const int b = 
 // The key block length of a launch, 64 << shift.  A window longer than that is split and passes partial results
 // through memory (72 bytes per voxel, head and block at head_dim 16, written and read back), so longer blocks
 // are better as long as the longest slot stays short against what a wavefront does in the whole launch:
-// N^2 / W pairs at least, H heads, over the lanes of about 3072 resident wavefronts.  64 unless half of that
-// covers a longer block.
+// N^2 / W pairs at least, H heads, over the lanes of about 3072 resident wavefronts.  64 unless two thirds of
+// that cover a longer block.
 __host__ inline int block_shift_for(int H, int64_t N, int64_t W, int max_window_voxels)
 {
     if (N <= 0 || W <= 0) return 6;
     const double steps_per_wave = static_cast<double>(N) * static_cast<double>(N) / static_cast<double>(W) * H / (64.0 * 3072.0);
     int shift = 6;
-    while ((1 << shift) < kMaxBlockSteps && (1 << shift) < max_window_voxels && 2.0 * (2 << shift) <= steps_per_wave) ++shift;
+    while ((1 << shift) < kMaxBlockSteps && (1 << shift) < max_window_voxels && 1.5 * (2 << shift) <= steps_per_wave) ++shift;
     return shift;
 }
 
