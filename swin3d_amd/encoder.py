@@ -485,15 +485,23 @@ class Upsample(nn.Module):
             self.block = Stage(out_channels, 1, num_heads, window_size, quant_size, downsample=False, cRSE=cRSE,
                                fp16_mode=fp16_mode)
 
+    @staticmethod
+    def _norm_linear(block, feats):
+        """LayerNorm + Linear; for inference under fp16 autocast the norm is the fused kernel that writes fp16."""
+        if _fused_norm_applies(feats):
+            _, normed = add_layernorm(feats, None, block[0])
+            return block[1](normed)
+        return block(feats)
+
     def forward(self, voxels, signals, voxels_up, signals_up, plan_up=None):
         """(voxels, signals): the coarse level; (voxels_up, signals_up): the finer level it feeds.  plan_up: a
         stage plan of the finer level's voxel set with the same window size (the encoder's, whose regular window
         set is the one this level's attention block needs), so that the index is not built a second time."""
         xyz = signals[:, 1:4].detach().contiguous().float()
         support_xyz = signals_up[:, 1:4].detach().contiguous().float()
-        feats = self.linear1(voxels_up.feats) + knn_linear_interpolation(
-            xyz, support_xyz, self.linear2(voxels.feats).float(), segment_offsets(voxels.coords[:, 0]),
-            segment_offsets(voxels_up.coords[:, 0]), K=self.up_k)
+        feats = self._norm_linear(self.linear1, voxels_up.feats) + knn_linear_interpolation(
+            xyz, support_xyz, self._norm_linear(self.linear2, voxels.feats).float(),
+            segment_offsets(voxels.coords[:, 0]), segment_offsets(voxels_up.coords[:, 0]), K=self.up_k)
         voxels_up = voxels_up.with_feats(feats.float())
         if self.attn:
             if plan_up is not None:
