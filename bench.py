@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-encoder", action="store_true",
                     help="skip the Swin3D-L encoder end-to-end latency")
+    ap.add_argument("--encoder-only", action="store_true",
+                    help="run only the Swin3D-L encoder forward (1 warm-up + 3 timed passes, no UNet) and print its "
+                         "figures: the command the encoder's kernel trace is taken with")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (windows are independent, so the path would shard over "
@@ -64,6 +67,9 @@ def main():
         return 3
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.encoder_only:
+        print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False)}))
+        return 0
 
     # ---- workload: the Swin3D-S stage-1 layer on a 200k-voxel synthetic room ------------------------
     heads, dim, ws, quant, cRSE = 6, 8, 5, 4, "XYZ_RGB_NORM"
@@ -282,7 +288,7 @@ def extras_cpu(oracle, synth, scene, ws):
     return out
 
 
-def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3):
+def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=True):
     """Swin3D-L encoder forward, fp16 attention (fp16_mode 2 under autocast),
     random-init weights, a batch of two synthetic rooms of ~300k voxels each; attention, window
     index and KNN on the HIP kernels, the dense layers on torch/hipBLASLt."""
@@ -309,6 +315,8 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3):
               "finite": bool(all(torch.isfinite(o.feats).all().item() for o in outs)),
               "config": "Swin3D-L channels [80,160,320,640,640] heads [10,10,20,40,40] depths [2,4,9,4,4] "
                         "windows [5,7,7,7,7] quant 4 cRSE XYZ_RGB_NORM, batch of 2 rooms"}
+    if not unet:
+        return result
     # the whole segmentation network on the same input: encoder + KNN-interpolation decoder with one attention
     # block per level + classifier
     del model, outs
