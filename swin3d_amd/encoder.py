@@ -235,13 +235,18 @@ class GridKNNDownsample(nn.Module):
                            segment_offsets(coarse[:, 0], num_batches))
         return coarse, coarse_signals, idx
 
-    def forward(self, voxels, signals, plan=None):
+    def forward(self, voxels, signals, plan=None, pending=None):
+        """pending: a term still to be added to voxels.feats (the last block's MLP output on the fused inference
+        path): the add runs inside the LayerNorm kernel and voxels.feats is updated in place.  Returns (coarse
+        voxels, coarse signals)."""
         coarse, coarse_signals, idx = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
         # LayerNorm and Linear act on single rows, so they commute with the gather: project the Ns fine rows once
         # instead of the K * Nq gathered copies (the reference statement, swin3d_layers.py:292-312, gathers first)
         if _fused_norm_applies(voxels.feats):
-            _, normed = add_layernorm(voxels.feats, None, self.norm)
+            _, normed = add_layernorm(voxels.feats, pending, self.norm, inplace=True)
         else:
+            if pending is not None:
+                voxels.feats += pending
             normed = self.norm(voxels.feats)
         projected = self.linear(normed)
         if not torch.is_grad_enabled() and projected.is_cuda and projected.dtype in (torch.float16, torch.float32):
@@ -387,18 +392,20 @@ class Stage(nn.Module):
         in every voxel.  Returns (features at this resolution, next voxels, next signals)."""
         args, down_plan = plan if plan is not None else self.plan(voxels.coords, voxels.stride, signals)
         feats = voxels.feats
+        pending = None
         if len(self.blocks) > 0 and self.blocks[0]._fused_path(feats):
-            pending = None
             for i, block in enumerate(self.blocks):
                 feats, pending = block.forward_fused(feats, pending, args[i % len(args)])
-            feats = feats + pending
+            if self.downsample is None or not feats.is_contiguous():
+                feats, pending = feats + pending, None
+            # else: the downsample's LayerNorm kernel adds the last MLP output, in place
         else:
             for i, block in enumerate(self.blocks):
                 feats = block(feats, args[i % len(args)])
         voxels = voxels.with_feats(feats)
         if self.downsample is None:
             return voxels, voxels, signals
-        down, down_signals = self.downsample(voxels, signals, down_plan)
+        down, down_signals = self.downsample(voxels, signals, down_plan, pending)
         return voxels, down, down_signals
 
 

@@ -70,3 +70,30 @@ def test_swin_block_fused_path_matches_torch_path(hip_lib):
     torch.cuda.synchronize()
     assert fused.dtype == torch.float32
     assert (fused - plain.detach()).abs().max().item() <= 2e-2 * plain.detach().abs().max().item()
+
+
+def test_stage_with_downsample_fused_path_matches_torch_path(hip_lib):
+    """A whole stage (two blocks + KNN downsample) on the inference path, where the last block's MLP output is
+    added inside the downsample's LayerNorm kernel, against the same stage with autograd enabled (torch adds and
+    LayerNorms); the caller's input features stay untouched."""
+    from swin3d_amd import encoder, synth
+    dev = torch.device("cuda")
+    scene = synth.make_room((3.0, 3.0, 2.0), 4, 6000, seed=5)
+    coords = torch.from_numpy(scene.coords).to(dev)
+    signals = torch.from_numpy(synth.encoder_inputs(scene)[1][:, :7].copy()).to(dev)      # batch, xyz, rgb
+    torch.manual_seed(1)
+    stage = encoder.Stage(48, 2, 6, 5, 4, out_channels=96, cRSE="XYZ_RGB", fp16_mode=2).to(dev).eval()
+    feats = torch.randn(coords.shape[0], 48, device=dev)
+    kept = feats.clone()
+    voxels = encoder.SparseVoxels(coords, feats, 1)
+    with torch.autocast("cuda", dtype=torch.float16):
+        with torch.no_grad():
+            plan = stage.plan(coords, 1, signals)
+            fine_f, down_f, sig_f = stage(voxels, signals, plan)
+        fine_p, down_p, sig_p = stage(voxels, signals, plan)          # grad mode on: torch kernels
+    torch.cuda.synchronize()
+    assert torch.equal(feats, kept)
+    assert torch.equal(down_f.coords, down_p.coords) and torch.equal(sig_f, sig_p)
+    for fused, plain in ((fine_f.feats, fine_p.feats.detach()), (down_f.feats, down_p.feats.detach())):
+        assert fused.dtype == torch.float32 and fused.shape == plain.shape
+        assert (fused - plain).abs().max().item() <= 2e-2 * plain.abs().max().item()
