@@ -97,4 +97,3 @@ def test_stage_with_downsample_fused_path_matches_torch_path(hip_lib):
     for fused, plain in ((fine_f.feats, fine_p.feats.detach()), (down_f.feats, down_p.feats.detach())):
         assert fused.dtype == torch.float32 and fused.shape == plain.shape
         assert (fused - plain).abs().max().item() <= 2e-2 * plain.abs().max().item()
-
