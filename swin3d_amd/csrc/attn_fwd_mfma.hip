@@ -117,7 +117,6 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
     typedef typename Frag<D>::type frag_t;
     typedef WaveLds<RMAX> L;
     constexpr int kIdxWords = (16 * ND + 3) / 4;
-    constexpr int kOut = D / 2;   // output channels a lane keeps for its query
 
     const int H = a.H;
     const int HD = H * D;
@@ -557,7 +556,7 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(AttnArgs a)
         int v = wave_total[threadIdx.x];
         for (int off = 1; off < 16; off <<= 1) {
             const int up = __shfl_up(v, off);
-            if (threadIdx.x >= off) v += up;
+            if (static_cast<int>(threadIdx.x) >= off) v += up;
         }
         wave_total[threadIdx.x] = v;
     }
