@@ -122,7 +122,7 @@ def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, hea
     _check(oracle_lib, case, dtype)
 
 
-@pytest.mark.parametrize("seed", range(10))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_shapes(oracle_lib, hip_lib, seed):
     """Randomly drawn shapes: head counts that do and do not divide the grid of workgroups evenly, both
     head_dims (VALU and MFMA table-gradient updates), 3 / 6 / 9 axes, sparse to dense windows (every size class of
