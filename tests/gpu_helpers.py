@@ -39,3 +39,12 @@ def assert_attn_close(got, ref, dtype):
     worst = np.unravel_index(np.argmax(err - tol), err.shape)
     assert (err <= tol).all(), (f"max err {err.max():.3e} (tol there {tol[worst]:.3e}) at {worst}: "
                                 f"got {got[worst]:.6f} ref {ref[worst]:.6f}")
+
+
+def elementwise_bound_failures(got, ref):
+    """Elements outside the purely element-wise fp32 bound |a-b| <= 1e-5 * max(|b|, 1e-2 * max|ref|)
+    -> (count, elements, largest |a-b| / bound)."""
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    bound = 1e-5 * np.maximum(np.abs(ref), 1e-2 * np.abs(ref).max())
+    ratio = np.abs(got - ref) / bound
+    return int((ratio > 1.0).sum()), int(ref.size), float(ratio.max())

@@ -83,3 +83,21 @@ def to_half_and_back(case):
     case.q, case.k, case.v = h(case.q), h(case.k), h(case.v)
     case.tq, case.tk, case.tv = h(case.tq), h(case.tk), h(case.tv)
     return case
+
+
+def downsampled_stage_case(oracle, scene, levels, ws, quant, heads, dim, cRSE="XYZ_RGB_NORM", shift=0,
+                           recipe="sharp", seed=0):
+    """AttnCase of an encoder stage below the first: `scene` grid-downsampled by 2, `levels` times (tensor
+    stride 2^levels), the kept point's position inside its coarse voxel as the fractional signal."""
+    stride = 1
+    for _ in range(levels):
+        scene, _ = synth.grid_downsample(scene, 2 * stride)
+        stride *= 2
+    frac = ((scene.xyz - scene.coords[:, 1:]) / np.float32(stride)).astype(np.float32)
+    frac = np.clip(frac, 0.0, np.float32(1.0 - 2.0 ** -24))
+    sig = synth.signals(scene, cRSE)
+    index, n_coords = n_coords_from_scene(oracle, scene.coords, frac, sig, stride, ws, quant, cRSE, shift)
+    sizes = crse.crse_table_sizes(ws, quant, heads, dim, cRSE)
+    n = scene.coords.shape[0]
+    q, k, v, tables = synth.layer_inputs(n, heads * dim, heads, int(sum(sizes)), seed=seed, recipe=recipe)
+    return AttnCase(scene.coords, stride, ws, quant, heads, dim, cRSE, index, n_coords, q, k, v, tables, sizes)

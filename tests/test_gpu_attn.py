@@ -311,6 +311,30 @@ def test_random_shapes(oracle_lib, hip_lib, seed):
     _check(oracle_lib, case, dtype)
 
 
+def test_fp32_elementwise_bound_report(oracle_lib, hip_lib, capsys):
+    """How many fp32 output elements fall outside the purely element-wise bound |a-b| <= 1e-5 * max(|b|,
+    1e-2 * max|ref|) (the head-vector bound of assert_attn_close is what the other tests assert).  The count is
+    printed; it must stay below 2 % of the elements, and no element may be off by more than 20x that bound
+    (measured: none outside for the layer recipe; 0.2 % outside, worst 5.3x, for the sharp recipe at head_dim 8 with
+    logits of magnitude ~10; 0.85 % outside, worst 8.7x, at head_dim 16 and window 7)."""
+    from gpu_helpers import run_attention, elementwise_bound_failures
+    scene = synth.make_room((6, 5, 3), 8, 20000, seed=0)
+    cases = {
+        "config 1 room, layer recipe": scene_attn_case(oracle_lib, scene, 5, 4, 6, 8, "XYZ_RGB", recipe="layer"),
+        "config 1 room, sharp recipe": scene_attn_case(oracle_lib, scene, 5, 4, 6, 8, "XYZ_RGB", recipe="sharp"),
+        "window 7, head_dim 16, sharp": make_attn_case(oracle_lib, seed=31, n=1500, ws=7, quant=4, heads=6, dim=16,
+                                                       extent=(9, 9, 4), batches=2, recipe="sharp"),
+    }
+    lines = []
+    for name, case in cases.items():
+        ref = oracle_lib.attn_fwd(*case.oracle_args())
+        bad, total, worst = elementwise_bound_failures(run_attention(case, torch.float32), ref)
+        lines.append(f"element-wise 1e-5 bound, {name}: {bad} of {total} elements outside, worst {worst:.2f}x")
+        assert bad <= 2e-2 * total and worst <= 20.0, lines[-1]
+    with capsys.disabled():
+        print("\n" + "\n".join(lines))
+
+
 def test_empty_input(hip_lib):
     import swin3d_amd
     dev = torch.device("cuda")
