@@ -68,7 +68,8 @@ const char *s3d_last_error_string(void);
  *                  that the row counts travel as kernel arguments)
  *   table_len      elements per table = sum_n table_sizes[n]
  *   w_sizes, w2n   device int32 [W]: voxels per window, exclusive prefix sum
- *   n2n            device int32 [N]: window-sorted position -> original row
+ *   n2n            device int32 [N]: window-sorted position -> original row, or NULL when the rows of q, k,
+ *                  v and out are in window-sorted order already (position = row; sweep kernel)
  *   n_coords       device fp32 [N,nd], window-sorted order, scaled by the quant sizes
  *   out            device [N,H,D] of `dtype`: softmax-normalised attention output
  *   out_max        device fp32 [N,H] or NULL: max logit per (voxel, head)
@@ -76,21 +77,21 @@ const char *s3d_last_error_string(void);
  *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
  *   max_window_voxels  an upper bound of every w_sizes entry (e.g. counts[2] of s3d_window_index, or
- *                  window^3), >= 1.  It sizes the partial results of windows that are split along their
- *                  keys (blocks of 64 voxels in the sweep kernel, 32 in the MFMA kernel); a window with
- *                  more key blocks than the bound allows is skipped (its output rows are not written),
- *                  so the bound must hold for a complete result.
+ *                  window^3), or 0 when none is known.  Only the MFMA kernel needs it (it sizes the partial
+ *                  results of windows of more than 32 voxels with it); without a bound the sweep kernel,
+ *                  which takes windows of any size, serves the call.  With an understated bound the MFMA
+ *                  kernel fills the rows of the windows beyond it (out, out_max, out_sum) with NaN.
  *   qkv_row_stride elements between consecutive voxel rows of q, k and v (0 = H*D, dense).  A multiple
  *                  of 8 that is >= H*D: with 3*H*D and q, k, v pointing H*D apart the kernels read the
  *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
  *                  place, without the reference's reshape / permute / contiguous copy.
  *   flags          0 (the library picks the kernel), S3D_ATTN_FORCE_GENERIC to run the VALU sweep kernel
  *                  for every case, or S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies
- *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes: work-queue
- *                  counters, the unit list, and N * ceil(max_window_voxels / 64) * H * (D + 2) floats of
- *                  partial results when max_window_voxels > 64 (sweep kernel); a transposed copy of the
- *                  value table, the work list and N * ceil(max_window_voxels / 32) * H * (D + 2) floats
- *                  when max_window_voxels > 32 (MFMA kernel)
+ *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes.  Sweep kernel:
+ *                  work-queue counters, one record per unit of 8 to 64 queries and one per window, about
+ *                  2 N + 24 W bytes + 0.3 MB.  MFMA kernel: a transposed copy of the value table, the work
+ *                  list and N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
+ *                  max_window_voxels > 32.  The size function returns the larger of the two.
  *   w2n must be ascending (the exclusive prefix sum of w_sizes, as the reference builds it:
  *   Swin3D/modules/swin3d_layers.py:100-103).
  *   D in {8,16}, nd in {3,6,9}, H >= 1.
@@ -138,8 +139,9 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W) bytes
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
- * dq, dk, dv are sums in a fixed order (deterministic); the table gradients are accumulated per
- * wavefront and added to global memory with fp32 atomics (order varies between runs).
+ * Every output is a sum in a fixed order (deterministic, no global atomics): dq, dk, dv have one owning
+ * lane per row; the table gradients are accumulated per wavefront, left in a slot of the workspace and
+ * summed per head by a reduction kernel.
  */
 size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W);
 int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,

@@ -60,8 +60,9 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_
         const int64_t rows = table_sizes[n] / (static_cast<int64_t>(H) * D);
         padded += (rows + 15) / 16 * 16;
     }
-    if (max_window_voxels < 1 || N < 0 || W < 0) return 0;
-    const size_t generic = attn_generic_workspace_bytes(H, D, W, N, max_window_voxels);
+    if (N < 0 || W < 0) return 0;
+    const size_t generic = attn_generic_workspace_bytes(H, W, N);
+    if (max_window_voxels < 1) return generic;      // no bound: the sweep kernel serves the call
     // the MFMA kernel's share only for shapes it can run (fp16 is not known here)
     AttnArgs a{};
     a.H = H;
@@ -116,7 +117,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.W = W;
     if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
     if (N == 0 || W == 0) return S3D_OK;
-    if (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n2n || !n_coords || !out)
+    if (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n_coords || !out)
         return fail(S3D_ERR_NULL_POINTER, "s3d_attn_fwd: null device pointer");
     a.q = q;
     a.k = k;
@@ -134,11 +135,9 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.out_sum = out_sum;
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && attn_mfma_supported(a, dtype) &&
-                           (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
-    if (max_window_voxels < 1)
-        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: max_window_voxels = %d (an upper bound of w_sizes, >= 1)",
-                    max_window_voxels);
+    // the MFMA kernel needs the window bound (it sizes partial results with it) and the row map
+    const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && max_window_voxels >= 1 && n2n &&
+                           attn_mfma_supported(a, dtype) && (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
     if (want_mfma) {
         const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
         if (!workspace || workspace_bytes < need)
@@ -149,12 +148,9 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         a.max_key_tiles = attn_mfma_key_tiles(max_window_voxels);
         return launch_attn_mfma(a, s);
     }
-    const size_t need = attn_generic_workspace_bytes(H, D, W, N, max_window_voxels);
+    const size_t need = attn_generic_workspace_bytes(H, W, N);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
-    a.partials = attn_generic_partials(workspace, H, W, N, max_window_voxels);
-    a.block_shift = attn_generic_block_shift(H, N, W, max_window_voxels);
-    a.max_key_tiles = attn_generic_key_blocks(H, N, W, max_window_voxels);
     return launch_attn_generic(a, dtype, s);
 }

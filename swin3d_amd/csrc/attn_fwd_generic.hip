@@ -3,9 +3,9 @@
 // Covers every dtype / shape the library accepts on the vector ALU (fp32 arithmetic; fp16 inputs enter through
 // packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one head (or two)
 // for its whole life and keeps the slices of the three relative-signal tables in LDS (loaded once, not once
-// per window).  Lane = slot = one query against a block of at most 64 keys of its window: q_i, the running
+// per window).  Lane = one query against (a share of) the keys of its window: q_i, the running
 // maximum, sum and output stay in the lane's registers while the lane streams its own window's keys, one per
-// step, so there is no cross-lane reduction, no atomic on data and no O(pairs) index array; the result is
+// step, no atomic on data and no O(pairs) index array; the result is
 // deterministic.  The slots of all windows, sorted by step count, are packed into units of 64 (the lanes of a
 // wavefront carry queries of several small windows); wavefronts draw units from the head's work queues.
 // Windows of more than 64 voxels leave one partial result per key block, combined by generic_merge_kernel.
@@ -25,72 +25,83 @@ namespace {
 using namespace sweep;
 
 constexpr int kThreads = 256;
-constexpr int kChunk = 64;   // slots per unit at most = lanes of a wavefront
+constexpr int kChunk = 64;   // lanes of a wavefront = lanes of a unit
 constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
 constexpr float kSlack = 10.0f;   // how far a logit may exceed the softmax reference exponent before it moves
-constexpr int kMaxBlockSteps = 256;   // the longest key block a launch may choose
-// key blocks a window of n voxels is split into when a slot streams at most 2^shift keys, and their even size
-__host__ __device__ inline int key_blocks(int n, int shift) { return (n + (1 << shift) - 1) >> shift; }
-__host__ __device__ inline int key_block_size(int n, int shift) { const int b = key_blocks(n, shift); return (n + b - 1) / b; }
-// The key block length of a launch, 64 << shift.  A window longer than that is split and passes partial results
-// through memory (72 bytes per voxel, head and block at head_dim 16, written and read back), so longer blocks
-// are better as long as the longest slot stays short against what a wavefront does in the whole launch:
-// N^2 / W pairs at least, H heads, over the lanes of about 3072 resident wavefronts.  64 unless two thirds of
-// that cover a longer block.
-__host__ inline int block_shift_for(int H, int64_t N, int64_t W, int max_window_voxels)
+// A window of n voxels belongs to class g (0..kMaxSplit): each of its queries is served by 2^g adjacent lanes that
+// take alternate keys, g the smallest value for which a lane streams at most `target` keys (the launch's step
+// target: 64, or 32 / 16 in small launches that would otherwise not fill the chip).  Windows of more than
+// target << kMaxSplit voxels stay in the last class and take more steps.
+constexpr int kMaxSplit = 3;
+constexpr int kClasses = kMaxSplit + 1;
+constexpr int kMaxSteps = 64;                    // step counts that have a bin of their own; longer ones share the last
+constexpr int kBins = kClasses * kMaxSteps;      // (class, steps), class 3 first, longest first inside a class
+constexpr int kSections = kMaxSplit + 3;         // classes 3..1, then class 0 in units of 64, 32 and 16 queries
+static_assert(kBins == kListThreads, "one thread per bin");
+__host__ __device__ inline int window_class(int n, int target_shift)
+{
+    int g = 0;
+    while (g < kMaxSplit && ((n + (1 << g) - 1) >> g) > (1 << target_shift)) ++g;
+    return g;
+}
+__host__ __device__ inline int window_bin(int n, int g)
+{
+    const int steps = (n + (1 << g) - 1) >> g;
+    return (kMaxSplit - g) * kMaxSteps + (kMaxSteps - (steps < kMaxSteps ? steps : kMaxSteps));
+}
+// The step target of a launch, as a shift.  The launch ends when its last wavefront does, so a unit must stay
+// short against what a wavefront does in the whole launch: N^2 / W pairs at least, per head group, over the
+// lanes of `waves` wavefronts that serve the group.  64 steps unless that leaves fewer than about six units per
+// wavefront.
+__host__ inline int target_shift_for(int64_t N, int64_t W, int waves)
 {
     if (N <= 0 || W <= 0) return 6;
-    const double steps_per_wave = static_cast<double>(N) * static_cast<double>(N) / static_cast<double>(W) * H / (64.0 * 3072.0);
+    const double lane_steps = static_cast<double>(N) * static_cast<double>(N) / static_cast<double>(W);
     int shift = 6;
-    while ((1 << shift) < kMaxBlockSteps && (1 << shift) < max_window_voxels && 1.5 * (2 << shift) <= steps_per_wave) ++shift;
+    while (shift > 4 && lane_steps / (64.0 * (1 << shift)) < 6.0 * (waves > 0 ? waves : 1)) --shift;
     return shift;
 }
 
-// byte offsets inside the workspace: the queue counters, the totals (units, split windows, slots), the first
-// entry of every unit, the sorted window entries, the placement notes and per-workgroup bin totals of the list
-// builder, the list of split windows, the partial results
+// byte offsets inside the workspace: the queue counters, the totals, one record per unit, the sorted window
+// entries, the placement notes and per-workgroup bin totals of the list builder
 __host__ __device__ inline size_t ws_round(size_t bytes) { return (bytes + 255) / 256 * 256; }
 __host__ __device__ inline size_t ws_total_offset(int H) { return sizeof(int32_t) * static_cast<size_t>(H) * kQueues * kCounterStride; }
 __host__ __device__ inline size_t ws_units_offset(int H) { return ws_total_offset(H) + 256; }
-// a voxel of a window with b key blocks takes b slots; a unit is at least 16 slots
-__host__ __device__ inline size_t ws_max_units(int64_t N, int max_blocks)
+// a unit holds at least 64 >> kMaxSplit = 8 queries, except the last one of each section
+__host__ __device__ inline size_t ws_max_units(int64_t N)
 {
-    return static_cast<size_t>(N > 0 ? N : 0) * max_blocks / (kChunk / 4) + 4;
+    return static_cast<size_t>(N > 0 ? N : 0) / (kChunk >> kMaxSplit) + kSections + 1;
 }
-__host__ __device__ inline size_t ws_entries_offset(int H, int64_t N, int max_blocks)
+__host__ __device__ inline size_t ws_entries_offset(int H, int64_t N)
 {
-    return ws_units_offset(H) + ws_round(sizeof(int32_t) * ws_max_units(N, max_blocks));
+    return ws_units_offset(H) + ws_round(sizeof(int4) * ws_max_units(N));
 }
-__host__ __device__ inline size_t ws_place_offset(int H, int64_t W, int64_t N, int max_blocks)
+__host__ __device__ inline size_t ws_place_offset(int H, int64_t W, int64_t N)
 {
-    return ws_entries_offset(H, N, max_blocks) + ws_round(sizeof(int4) * (static_cast<size_t>(W > 0 ? W : 0) + kChunk));
+    return ws_entries_offset(H, N) + ws_round(sizeof(int4) * (static_cast<size_t>(W > 0 ? W : 0) + kChunk));
 }
-__host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N, int max_blocks)
+__host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N)
 {
-    return ws_place_offset(H, W, N, max_blocks) + ws_round(sizeof(int2) * static_cast<size_t>(W > 0 ? W : 1));
+    return ws_place_offset(H, W, N) + ws_round(sizeof(int2) * static_cast<size_t>(W > 0 ? W : 1));
 }
-__host__ __device__ inline size_t ws_split_offset(int H, int64_t W, int64_t N, int max_blocks)
+__host__ __device__ inline size_t ws_end_offset(int H, int64_t W, int64_t N)
 {
-    return ws_bins_offset(H, W, N, max_blocks) + ws_round(sizeof(unsigned long long) * kListGroups * (kMaxBlockSteps + 1));
-}
-__host__ __device__ inline size_t ws_partials_offset(int H, int64_t W, int64_t N, int max_blocks)
-{
-    return ws_split_offset(H, W, N, max_blocks) + ws_round(sizeof(int32_t) * static_cast<size_t>(W > 0 ? W : 1));
+    return ws_bins_offset(H, W, N) + ws_round(sizeof(unsigned long long) * kListGroups * kBins);
 }
 
-// How the slots of a launch (sorted by steps, longest first) are cut into units.  A unit is one pass of a
-// wavefront: 64 slots, or 32 slots whose lanes l and l + 32 share a query and take alternate keys (half the
-// steps), or 16 slots in four such groups (a quarter).  The launch ends when the last wavefront ends, so the
-// last slots go into the finer units: about two 16-slot units and one 32-slot unit per wavefront of a head
-// group (`waves`), everything before them into 64-slot units.
+// How the queries of class 0 (sorted by steps, longest first) are cut into units.  A unit is one pass of a
+// wavefront: 64 queries, or 32 queries with two adjacent lanes each (alternate keys, half the steps), or 16
+// queries with four lanes each (a quarter).  The launch ends when the last wavefront ends, so the last queries
+// go into the finer units: about two 16-query units and one 32-query unit per wavefront of a head group
+// (`waves`), everything before them into 64-query units.
 struct UnitPlan {
-    int units[3];   // units of 64, 32 and 16 slots, in this order along the slots
+    int units[3];   // units of 64, 32 and 16 queries, in this order along the queries
     __host__ __device__ int first_slot(int g) const { return g == 0 ? 0 : g == 1 ? units[0] * kChunk : units[0] * kChunk + units[1] * (kChunk / 2); }
     __host__ __device__ int first_unit(int g) const { return g == 0 ? 0 : g == 1 ? units[0] : units[0] + units[1]; }
 };
 __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 {
-    const int fine = 32 * (waves > 0 ? waves : 1);   // slots of each finer kind
+    const int fine = 32 * (waves > 0 ? waves : 1);   // queries of each finer kind
     const int in_c = total_slots < fine ? total_slots : fine;
     const int in_b = total_slots - in_c < fine ? total_slots - in_c : fine;
     UnitPlan plan;
@@ -103,79 +114,69 @@ __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
     return plan;
 }
 
-// Work list of the launch, built by two small kernels.  A voxel of a window that is split into b key blocks
-// (b = 1 up to the launch's block length of 64, 128 or 256 voxels) takes b slots, one per key block, and a slot
-// streams the block's keys: at most that many steps.  The windows are sorted by that step count, longest first
-// (a counting sort over the possible counts), their slots laid out back to back in that order -
-// [window][key block][voxel] - and cut into units,
-// so a wavefront's lanes carry queries of several windows when the windows are small, every lane of a unit
-// runs (almost) the same number of steps, and the launch ends on its shortest units.
+// Work list of the launch, built by two small kernels.  The windows are sorted by (class, steps), highest class and
+// longest first - a counting sort over the kBins possible keys - and the queries of each class are numbered
+// back to back in that order, [window][voxel], and cut into units: 64 >> g queries of class g, each on 2^g
+// adjacent lanes.  A wavefront's lanes so carry queries of several windows when the windows are small, every
+// lane of a unit runs (almost) the same number of steps, a query's keys never leave its wavefront (the lanes
+// that share a query merge their softmax states by shuffles), and the launch ends on its shortest units.
 //
 // generic_count_kernel: every workgroup takes a run of windows; a window takes a place in the workgroup's bin
-// of its step count - its rank there and the slots before it (one 64-bit LDS atomic returns both, so the two
-// orders agree; the order inside a bin does not affect results) - and the workgroup leaves its bin totals.
+// of its (class, steps) - its rank there and the queries before it (one 64-bit LDS atomic returns both, so the
+// two orders agree; the order inside a bin does not affect results) - and the workgroup leaves its bin totals.
 __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
 {
-    __shared__ unsigned long long bin[kMaxBlockSteps + 1];   // per step count: windows << 32 | slots
-    for (int t = threadIdx.x; t <= kMaxBlockSteps; t += kListThreads) bin[t] = 0;
+    __shared__ unsigned long long bin[kBins];   // per bin: windows << 32 | queries
+    for (int t = threadIdx.x; t < kBins; t += kListThreads) bin[t] = 0;
     __syncthreads();
     char *ws = static_cast<char *>(a.workspace);
-    int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
-    int2 *place = reinterpret_cast<int2 *>(ws + ws_place_offset(a.H, a.W, a.N, a.max_key_tiles));
-    unsigned long long *group_bins =
-        reinterpret_cast<unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N, a.max_key_tiles));
+    int2 *place = reinterpret_cast<int2 *>(ws + ws_place_offset(a.H, a.W, a.N));
+    unsigned long long *group_bins = reinterpret_cast<unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N));
     const int W = static_cast<int>(a.W);
     const int per = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
     const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
     for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
         const int n = a.w_sizes[w];
-        const int blocks = key_blocks(n, a.block_shift);
         int2 got = make_int2(-1, 0);
-        if (n > 0 && blocks <= a.max_key_tiles) {
+        if (n > 0) {
             const unsigned long long before =
-                atomicAdd(&bin[key_block_size(n, a.block_shift)], (1ull << 32) | static_cast<unsigned>(n * blocks));
+                atomicAdd(&bin[window_bin(n, window_class(n, a.block_shift))], (1ull << 32) | static_cast<unsigned>(n));
             got = make_int2(static_cast<int>(before >> 32), static_cast<int>(before & 0xffffffffu));
         }
         place[w] = got;
     }
     __syncthreads();
-    for (int t = threadIdx.x; t <= kMaxBlockSteps; t += kListThreads)
-        group_bins[blockIdx.x * (kMaxBlockSteps + 1) + t] = bin[t];
-    if (blockIdx.x == 0 && threadIdx.x == 0) total[1] = 0;   // split windows, counted by the second kernel
+    for (int t = threadIdx.x; t < kBins; t += kListThreads) group_bins[blockIdx.x * kBins + t] = bin[t];
 }
 
-// generic_place_kernel (same grid): bins in descending step order, workgroups in order inside a bin.  Writes one
-// entry (first slot, voxels, first sorted position, steps) per window in sorted order, the entry that holds
-// the first slot of every unit, the list of split windows for the merge, the totals, and the queue counters
-// at zero.  Windows beyond the caller's size bound get no slots.
+// generic_place_kernel (same grid): bins in order, workgroups in order inside a bin.  Writes one entry (first
+// query of its class, voxels, first sorted position, class) per window in sorted order, one record per unit
+// (the entry that holds its first query, lanes per query as a shift, first query, queries), the totals, and
+// the queue counters at zero.
 __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
 {
-    __shared__ int bin_entry[kMaxBlockSteps + 1], bin_slot[kMaxBlockSteps + 1];
+    __shared__ int bin_entry[kBins], bin_slot[kBins];
     __shared__ int wave_c[kListThreads / 64], wave_s[kListThreads / 64];
-    __shared__ int sums[2];
+    __shared__ int class_base[kClasses + 1];       // queries before each class (index = kMaxSplit - g), and all
+    __shared__ int total_entries_s;
     char *ws = static_cast<char *>(a.workspace);
     int *counters = reinterpret_cast<int *>(ws);
     int *total = reinterpret_cast<int *>(ws + ws_total_offset(a.H));
-    int *unit_first = reinterpret_cast<int *>(ws + ws_units_offset(a.H));
-    int4 *entries = reinterpret_cast<int4 *>(ws + ws_entries_offset(a.H, a.N, a.max_key_tiles));
-    const int2 *place = reinterpret_cast<const int2 *>(ws + ws_place_offset(a.H, a.W, a.N, a.max_key_tiles));
+    int4 *unit_info = reinterpret_cast<int4 *>(ws + ws_units_offset(a.H));
+    int4 *entries = reinterpret_cast<int4 *>(ws + ws_entries_offset(a.H, a.N));
+    const int2 *place = reinterpret_cast<const int2 *>(ws + ws_place_offset(a.H, a.W, a.N));
     const unsigned long long *group_bins =
-        reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N, a.max_key_tiles));
-    int *split = reinterpret_cast<int *>(ws + ws_split_offset(a.H, a.W, a.N, a.max_key_tiles));
-    static_assert(kListThreads == kMaxBlockSteps, "one thread per bin");
-    // thread t holds the bin of (longest block) - t steps: the launch's total, and what the workgroups before
-    // this one put there; an exclusive scan over the threads gives the bins their places
+        reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N));
+    // thread t holds bin t: the launch's total, and what the workgroups before this one put there; an exclusive
+    // scan over the threads gives the bins their places (entries over all bins, queries restarting per class)
     {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-        const int steps = (1 << a.block_shift) - static_cast<int>(threadIdx.x);
         unsigned long long all = 0, before = 0;
-        if (steps >= 1) {
 #pragma unroll 8
-            for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
-                const unsigned long long v = group_bins[g * (kMaxBlockSteps + 1) + steps];
-                all += v;
-                before += g < static_cast<int>(blockIdx.x) ? v : 0;
-            }
+        for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
+            const unsigned long long v = group_bins[g * kBins + threadIdx.x];
+            all += v;
+            before += g < static_cast<int>(blockIdx.x) ? v : 0;
         }
         const int cnt = static_cast<int>(all >> 32), slots = static_cast<int>(all & 0xffffffffu);
         int incl_c = cnt, incl_s = slots;
@@ -187,88 +188,71 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
         __syncthreads();
         int base_c = 0, base_s = 0;
         for (int v = 0; v < wave; ++v) { base_c += wave_c[v]; base_s += wave_s[v]; }
-        if (steps >= 1) {
-            bin_entry[steps] = base_c + incl_c - cnt + static_cast<int>(before >> 32);
-            bin_slot[steps] = base_s + incl_s - slots + static_cast<int>(before & 0xffffffffu);
-        }
-        if (threadIdx.x == kListThreads - 1) { sums[0] = base_c + incl_c; sums[1] = base_s + incl_s; }
+        static_assert(kMaxSteps == 64, "a class is the bins of one wavefront of the scan");
+        // queries are numbered per class: the class's bins are this wavefront's, so drop the earlier wavefronts' sum
+        bin_entry[threadIdx.x] = base_c + incl_c - cnt + static_cast<int>(before >> 32);
+        bin_slot[threadIdx.x] = incl_s - slots + static_cast<int>(before & 0xffffffffu);
+        if (lane == 0) class_base[wave] = base_s;
+        if (threadIdx.x == kListThreads - 1) { class_base[kClasses] = base_s + incl_s; total_entries_s = base_c + incl_c; }
     }
     __syncthreads();
-    const int total_entries = sums[0], total_slots = sums[1];
-    const UnitPlan plan = plan_units(total_slots, a.target_items);
+    const int total_entries = total_entries_s;
+    // sections: classes kMaxSplit..1 in units of 64 >> g queries, then class 0 in its three kinds of unit
+    int sec_unit[kSections + 1], class_total[kClasses];
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) class_total[c] = class_base[c + 1] - class_base[c];
+    const UnitPlan plan = plan_units(class_total[kMaxSplit], a.target_items);
+    sec_unit[0] = 0;
+#pragma unroll
+    for (int c = 0; c < kMaxSplit; ++c) {
+        const int per = kChunk >> (kMaxSplit - c);
+        sec_unit[c + 1] = sec_unit[c] + (class_total[c] + per - 1) / per;
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) sec_unit[kMaxSplit + k + 1] = sec_unit[kMaxSplit + k] + plan.units[k];
     const int W = static_cast<int>(a.W);
-    const int per = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
-    const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
+    const int per_group = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    const int begin = min(static_cast<int>(blockIdx.x) * per_group, W), end = min(begin + per_group, W);
     for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
         const int2 got = place[w];
         if (got.x < 0) continue;
         const int n = a.w_sizes[w];
-        const int blocks = key_blocks(n, a.block_shift), steps = key_block_size(n, a.block_shift);
-        const int e = bin_entry[steps] + got.x;
-        const int s = bin_slot[steps] + got.y;
-        entries[e] = make_int4(s, n, a.w2n[w], steps);
-        // the units whose first slot is one of this window's
-        const int s_end = s + n * blocks;
+        const int g = window_class(n, a.block_shift), b = window_bin(n, g);
+        const int e = bin_entry[b] + got.x;
+        const int s = bin_slot[b] + got.y;               // first query of the window inside its class
+        entries[e] = make_int4(s, n, a.w2n[w], g);
+        const int s_end = s + n;
+        if (g > 0) {
+            // the units whose first query is one of this window's
+            const int size = kChunk >> g, c = kMaxSplit - g, all = class_total[c];
+            for (int v = (s + size - 1) / size; v * size < s_end; ++v)
+                unit_info[sec_unit[c] + v] = make_int4(e, g, v * size, min(size, all - v * size));
+        } else {
+            const int all = class_total[kMaxSplit];
 #pragma unroll
-        for (int g = 0; g < 3; ++g) {
-            const int size = kChunk >> g, from = plan.first_slot(g), count = plan.units[g];
-            int v = s <= from ? 0 : (s - from + size - 1) / size;
-            for (; v < count && from + v * size < s_end; ++v) unit_first[plan.first_unit(g) + v] = e;
+            for (int k = 0; k < 3; ++k) {
+                const int size = kChunk >> k, from = plan.first_slot(k), count = plan.units[k];
+                int v = s <= from ? 0 : (s - from + size - 1) / size;
+                for (; v < count && from + v * size < s_end; ++v)
+                    unit_info[sec_unit[kMaxSplit + k] + v] = make_int4(e, k, from + v * size, min(size, all - (from + v * size)));
+            }
         }
-        if (blocks > 1) split[atomicAdd(total + 1, 1)] = w;   // any order: the merge treats windows independently
     }
     if (blockIdx.x == 0) {
-        // a wavefront reads 64 entries from a unit's first one: pad the list with entries no slot belongs to
-        if (threadIdx.x < kChunk) entries[total_entries + threadIdx.x] = make_int4(total_slots, 1, 0, 1);
-        if (threadIdx.x == 0) {
-            total[0] = plan.units[0] + plan.units[1] + plan.units[2];
-            total[2] = total_slots;
-            total[3] = plan.units[0];
-            total[4] = plan.units[1];
-        }
+        // a wavefront reads 64 entries from a unit's first one: pad the list with entries no query belongs to
+        if (threadIdx.x < kChunk) entries[total_entries + threadIdx.x] = make_int4(0x7fffffff, 1, 0, -1);
+        if (threadIdx.x == 0) total[0] = sec_unit[kSections];
         for (int t = threadIdx.x; t < a.H * kQueues; t += kListThreads) counters[t * kCounterStride] = 0;
     }
 }
 
-// Windows of more than 64 voxels: combine the per-key-block partial results (unnormalised output, running
-// maximum, sum) of every (voxel, head).  Workgroups take the split windows of the launch in turn; one thread
-// per (voxel of the window, head), voxel fastest.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void generic_merge_kernel(AttnArgs a)
+inline int device_cus()
 {
-    const int H = a.H;
-    const char *ws = static_cast<const char *>(a.workspace);
-    const int count = reinterpret_cast<const int *>(ws + ws_total_offset(H))[1];
-    const int *split = reinterpret_cast<const int *>(ws + ws_split_offset(H, a.W, a.N, a.max_key_tiles));
-    const int64_t block_stride = static_cast<int64_t>(H) * a.N * (D + 2);
-    for (int e = blockIdx.x; e < count; e += gridDim.x) {
-        const int w = split[e];
-        const int n_w = a.w_sizes[w], s0 = a.w2n[w];
-        const int blocks = key_blocks(n_w, a.block_shift);
-        for (int t = threadIdx.x; t < n_w * H; t += blockDim.x) {
-            const int h = t / n_w, pos = s0 + (t - h * n_w);
-            const float *part = a.partials + (static_cast<int64_t>(h) * a.N + pos) * (D + 2);
-            float m = -INFINITY;
-            for (int kb = 0; kb < blocks; ++kb) m = fmaxf(m, part[kb * block_stride + D]);
-            float l = 0.0f, o[D];
-#pragma unroll
-            for (int c = 0; c < D; ++c) o[c] = 0.0f;
-            for (int kb = 0; kb < blocks; ++kb) {
-                const float *pk = part + kb * block_stride;
-                const float wgt = __expf(pk[D] - m);
-                l += pk[D + 1] * wgt;
-#pragma unroll
-                for (int c = 0; c < D; ++c) o[c] += pk[c] * wgt;
-            }
-            const int row = a.n2n[pos];
-            const float inv = 1.0f / l;
-#pragma unroll
-            for (int c = 0; c < D; ++c) o[c] *= inv;
-            store_row<D>(static_cast<T *>(a.out) + (static_cast<int64_t>(row) * H + h) * D, o);
-            if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = m;
-            if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = l;
-        }
-    }
+    int device = 0, v = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0)
+        return v;
+    return 256;
 }
 
 // workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
@@ -285,7 +269,8 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int table_row
 
 // HP: heads a wavefront carries through a unit (adjacent heads HP * g .. HP * g + HP - 1).  The cRSE rows and
 // LDS addresses of a pair do not depend on the head, so two heads share that part of the work.
-template <typename T, int D, int ND, int HP>
+// kSorted: q, k, v and out rows are in window-sorted order already (no n2n).
+template <typename T, int D, int ND, int HP, bool kSorted>
 __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fwd_sweep_kernel(AttnArgs a)
 {
     // streamed keys per loop iteration: at head_dim 16 two interleaved chains hide the LDS round trips,
@@ -326,14 +311,9 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
     const T *gk = static_cast<const T *>(a.k);
     const T *gv = static_cast<const T *>(a.v);
     const char *ws = static_cast<const char *>(a.workspace);
-    const int *unit_first = reinterpret_cast<const int *>(ws + ws_units_offset(H));
-    const int4 *entries = reinterpret_cast<const int4 *>(ws + ws_entries_offset(H, a.N, a.max_key_tiles));
+    const int4 *unit_info = reinterpret_cast<const int4 *>(ws + ws_units_offset(H));
+    const int4 *entries = reinterpret_cast<const int4 *>(ws + ws_entries_offset(H, a.N));
     const int total_units = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[0]);
-    const int total_slots = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[2]);
-    UnitPlan plan;
-    plan.units[0] = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[3]);
-    plan.units[1] = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[4]);
-    plan.units[2] = 0;
     int *counters = static_cast<int *>(a.workspace) + hg * kQueues * kCounterStride;
     constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
     constexpr uint32_t kHeadBytes = 3 * D * sizeof(T);   // one head's slices inside a row
@@ -361,34 +341,35 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
             unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
         }
         if (unit >= total_units) break;
-        // the lane's slot: a query of a window and one block of at most 64 of the window's keys.  The unit's 64
-        // slots lie in at most 64 consecutive entries from the unit's first one; each lane reads one entry and
-        // finds its own (the last entry that starts at or before its slot) by a search across the lanes.
-        const int first = __builtin_amdgcn_readfirstlane(unit_first[unit]);
+        // The unit: 64 >> gshift queries (consecutive in the sorted numbering of their class), each on 2^gshift
+        // adjacent lanes that take alternate keys.  The queries lie in at most 64 consecutive entries from the
+        // unit's first one; each lane reads one entry and finds its own (the last entry of the class that starts at
+        // or before its query) by a search across the lanes.
+        const int4 info = unit_info[unit];
+        const int first = __builtin_amdgcn_readfirstlane(info.x);
+        const int gshift = __builtin_amdgcn_readfirstlane(info.y);
+        const int queries = __builtin_amdgcn_readfirstlane(info.w);
+        const int sub = lane & ((1 << gshift) - 1);
+        const bool own_valid = (lane >> gshift) < queries;
+        const int query = __builtin_amdgcn_readfirstlane(info.z) + min(lane >> gshift, queries - 1);   // lanes past the end repeat the last one
         const int4 seen = entries[first + lane];
-        // the unit's kind: 2^gshift groups of lanes that share queries and take alternate keys
-        const int gshift = unit < plan.first_unit(1) ? 0 : unit < plan.first_unit(2) ? 1 : 2;
-        const int gs = kChunk >> gshift;
-        const int grp = lane >> (6 - gshift);
-        const int slot_raw = plan.first_slot(gshift) + (unit - plan.first_unit(gshift)) * gs + (lane & (gs - 1));
-        const bool own_valid = slot_raw < total_slots;
-        const int slot = min(slot_raw, total_slots - 1);   // lanes past the end repeat the last slot
+        const int seen_from = seen.w == __builtin_amdgcn_readfirstlane(seen.w) ? seen.x : 0x7fffffff;   // the next class restarts at 0
         int at = 0;
 #pragma unroll
         for (int half = 32; half > 0; half >>= 1)
-            if (__shfl(seen.x, at + half) <= slot) at += half;
-        const int n_w = __shfl(seen.y, at), s0 = __shfl(seen.z, at), block_size = __shfl(seen.w, at);
-        const int in_window = slot - __shfl(seen.x, at);               // [key block][voxel]
-        // entries are sorted by steps, longest first
-        const int max_steps = (__builtin_amdgcn_readfirstlane(seen.w) + (1 << gshift) - 1) >> gshift;
-        const int blocks = key_blocks(n_w, a.block_shift);
-        const int kb = blocks == 1 ? 0 : in_window / n_w;
-        const int own_pos = s0 + (in_window - kb * n_w);
-        const int own_row = a.n2n[own_pos];
-        // the slot's keys: block kb of the window's even split into blocks of at most 64
-        const int k_begin = kb * block_size;
-        const int n_k = min(block_size, n_w - k_begin);
-        const int k0 = s0 + k_begin;
+            if (__shfl(seen_from, at + half) <= query) at += half;
+        const int n_w = __shfl(seen.y, at), s0 = __shfl(seen.z, at);
+        const int own_pos = s0 + (query - __shfl(seen.x, at));
+        const int own_row = kSorted ? own_pos : a.n2n[own_pos];
+        // the longest lane of the unit (entries are sorted by steps, but windows beyond the longest bin are not)
+        int max_steps = (n_w + (1 << gshift) - 1) >> gshift;
+#pragma unroll
+        for (int other = 32; other > 0; other >>= 1) max_steps = max(max_steps, __shfl_xor(max_steps, other));
+        max_steps = __builtin_amdgcn_readfirstlane(max_steps);
+        // the lane's keys: sub, sub + 2^gshift, ... of the window's n_k
+        const int n_k = n_w;
+        const int k0 = s0;
+        const int grp = sub;
 
         Slice<T, D> qv[HP];
         float ci[ND], acc[HP][D], m[HP], top[HP], l[HP];
@@ -407,7 +388,7 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
         // LDS and cache round trips a single chain would wait out one after the other
         int row_next[kKeys];
 #pragma unroll
-        for (int u = 0; u < kKeys; ++u) row_next[u] = a.n2n[k0 + min((u << gshift) + grp, n_k - 1)];
+        for (int u = 0; u < kKeys; ++u) row_next[u] = kSorted ? 0 : a.n2n[k0 + min((u << gshift) + grp, n_k - 1)];
         for (int it = 0; it < max_steps; it += kKeys) {
             // the next unit's ticket is drawn during the last iteration: the atomic's round trip overlaps that
             // work, and a unit is not held back (out of reach of idle wavefronts) for longer than one step
@@ -421,8 +402,8 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
                 const int st = ((it + u) << gshift) + grp;
                 valid[u] = st < n_k;
                 const int st_pos = k0 + min(st, n_k - 1);
-                const int st_row = row_next[u];
-                row_next[u] = a.n2n[k0 + min(st + (kKeys << gshift), n_k - 1)];
+                const int st_row = kSorted ? st_pos : row_next[u];
+                if (!kSorted) row_next[u] = a.n2n[k0 + min(st + (kKeys << gshift), n_k - 1)];
 #pragma unroll
                 for (int hh = 0; hh < HP; ++hh) {
                     kv[u][hh].load(gk + static_cast<int64_t>(st_row) * a.row_stride + (h + hh) * D);
@@ -544,8 +525,8 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
         }
 #pragma unroll
         for (int hh = 0; hh < HP; ++hh) {
-            // groups saw alternate keys of the same queries: merge their softmax states
-            for (int other = 32; other >= gs; other >>= 1) {
+            // lanes that share a query saw alternate keys: merge their softmax states
+            for (int other = 1; other < (1 << gshift); other <<= 1) {
                 const float m_o = __shfl_xor(m[hh], other), l_o = __shfl_xor(l[hh], other);
                 const float m_all = fmaxf(m[hh], m_o);
                 const float w_me = (m[hh] == -INFINITY) ? 0.0f : __expf(m[hh] - m_all);
@@ -555,52 +536,38 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
                 for (int c = 0; c < D; ++c) acc[hh][c] = acc[hh][c] * w_me + __shfl_xor(acc[hh][c], other) * w_ot;
                 m[hh] = m_all;
             }
-            if (own_valid && grp == 0) {
-                if (blocks == 1) {
-                    const float inv = 1.0f / l[hh];
+            if (own_valid && sub == 0) {
+                const float inv = 1.0f / l[hh];
 #pragma unroll
-                    for (int c = 0; c < D; ++c) acc[hh][c] *= inv;
-                    store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + (h + hh) * D, acc[hh]);
-                    if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h + hh] = m[hh];
-                    if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h + hh] = l[hh];
-                } else {
-                    float *part = a.partials + ((static_cast<int64_t>(kb) * H + h + hh) * a.N + own_pos) * (D + 2);
-#pragma unroll
-                    for (int c = 0; c < D; ++c) part[c] = acc[hh][c];
-                    part[D] = m[hh];
-                    part[D + 1] = l[hh];
-                }
+                for (int c = 0; c < D; ++c) acc[hh][c] *= inv;
+                store_row<D>(static_cast<T *>(a.out) + static_cast<int64_t>(own_row) * HD + (h + hh) * D, acc[hh]);
+                if (a.out_max) a.out_max[static_cast<int64_t>(own_row) * H + h + hh] = m[hh];
+                if (a.out_sum) a.out_sum[static_cast<int64_t>(own_row) * H + h + hh] = l[hh];
             }
         }
     }
 }
 
-template <typename T, int D, int ND, int HP>
+template <typename T, int D, int ND, int HP, bool kSorted>
 int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
 {
     const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride_heads<T, D, HP>(), 16);
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
-    if (a.N * a.max_key_tiles > INT32_MAX - kChunk)
-        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %lld voxels x %d key blocks exceed the 32-bit slot count",
-                    (long long)a.N, a.max_key_tiles);
-    auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP>;
+    auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP, kSorted>;
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    int device = 0, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
-    }
     // a workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow,
     // in whole sets of (XCDs x head groups)
     int per_cu = groups_per_cu<T, D, HP>();
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
     const int set = kQueues * (a.H / HP);
+    const int cus = device_cus();
     const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
     AttnArgs b = a;
     b.target_items = sets * kQueues * (kThreads / 64);   // wavefronts that serve one head group
+    b.block_shift = target_shift_for(a.N, a.W, b.target_items);
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
     const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
     hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
@@ -608,12 +575,6 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     S3D_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
     S3D_HIP_CHECK(hipGetLastError());
-    if (a.max_key_tiles > 1) {
-        const int64_t want = a.W < 1024 ? a.W : 1024;
-        hipLaunchKernelGGL((generic_merge_kernel<T, D>), dim3(static_cast<unsigned>(want > 0 ? want : 1)), dim3(256),
-                           0, stream, a);
-        S3D_HIP_CHECK(hipGetLastError());
-    }
     return S3D_OK;
 }
 
@@ -622,9 +583,10 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream)
 {
     // two heads per wavefront where the registers allow it (head_dim 8, fp16) and the heads pair up
     if constexpr (D <= 8 && sizeof(T) == 2) {
-        if (a.H % 2 == 0) return launch_sweep_heads<T, D, ND, 2>(a, stream);
+        if (a.H % 2 == 0)
+            return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream) : launch_sweep_heads<T, D, ND, 2, true>(a, stream);
     }
-    return launch_sweep_heads<T, D, ND, 1>(a, stream);
+    return a.n2n ? launch_sweep_heads<T, D, ND, 1, false>(a, stream) : launch_sweep_heads<T, D, ND, 1, true>(a, stream);
 }
 
 template <typename T>
@@ -641,29 +603,10 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream)
 
 }  // namespace
 
-int attn_generic_block_shift(int H, int64_t N, int64_t W, int max_window_voxels)
+size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N)
 {
-    return block_shift_for(H, N, W, max_window_voxels);
-}
-
-int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels)
-{
-    return key_blocks(max_window_voxels > 0 ? max_window_voxels : 1, block_shift_for(H, N, W, max_window_voxels));
-}
-
-size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels)
-{
-    // queue counters, the totals, the unit list and sorted window list, and one partial record per (key block, head,
-    // voxel) when some window may be split along its keys
-    const int blocks = attn_generic_key_blocks(H, N, W, max_window_voxels);
-    const size_t partials = blocks <= 1 ? 0 : sizeof(float) * static_cast<size_t>(N) * blocks * H * (D + 2);
-    return ws_partials_offset(H, W, N, blocks) + align_up(partials, 256);
-}
-
-float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels)
-{
-    return reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                     ws_partials_offset(H, W, N, attn_generic_key_blocks(H, N, W, max_window_voxels)));
+    // queue counters, the totals, one record per unit, the sorted window list and the list builder's notes
+    return ws_end_offset(H, W, N);
 }
 
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream)

@@ -202,8 +202,23 @@ __global__ __launch_bounds__(kWaves * 64) void attn_fwd_mfma_kernel(AttnArgs a)
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         const int nkt = (n_w + kTile - 1) / kTile;   // key tiles (= query tiles)
         const bool single_key_tile = nkt == 1;
-        // a window beyond the caller's size bound has no room for its partial results: leave it out
-        if (nkt > a.max_key_tiles) continue;
+        // A window beyond the caller's size bound has no room for its partial results.  Its rows are not left
+        // as the buffer held them: the item of a query tile's first key tile fills them (and the statistics)
+        // with NaN, so an understated bound shows in the result.
+        if (nkt > a.max_key_tiles) {
+            const int local = pair - (w > 0 ? __builtin_amdgcn_readfirstlane(item_end[w - 1]) : 0);
+            const int q_in = (local / nkt) * kTile + il;
+            if (local % nkt == 0 && half == 0 && q_in < n_w) {
+                const int row = a.n2n[s0 + q_in];
+                const _Float16 nan16 = static_cast<_Float16>(__builtin_nanf(""));
+                for (int h = h_begin; h < h_end; ++h) {
+                    for (int c = 0; c < D; ++c) gout[static_cast<int64_t>(row) * HD + h * D + c] = nan16;
+                    if (a.out_max) a.out_max[static_cast<int64_t>(row) * H + h] = __builtin_nanf("");
+                    if (a.out_sum) a.out_sum[static_cast<int64_t>(row) * H + h] = __builtin_nanf("");
+                }
+            }
+            continue;
+        }
         // one item = one (query tile, key tile) pair of a window and a group of heads: the pair row
         // indices are computed once and reused by every head of the group.  A window of at most 32
         // voxels writes the final output; larger windows write per-key-tile partial results

@@ -18,9 +18,9 @@ struct AttnArgs {
     float *out_max, *out_sum;              // [N,H] or null
     void *workspace;                       // the caller's workspace
     void *items;                           // int32 [W+1] work-item prefix + counter (MFMA path)
-    float *partials;                       // per-key-tile partial results of multi-tile windows
-    int32_t max_key_tiles;                 // key tiles of the largest window (stride of `partials`)
-    int32_t block_shift;                   // sweep kernel: a slot streams at most 2^block_shift keys
+    float *partials;                       // MFMA path: per-key-tile partial results of multi-tile windows
+    int32_t max_key_tiles;                 // MFMA path: key tiles of the largest window (stride of `partials`)
+    int32_t block_shift;                   // sweep kernel: the step target, a lane streams about 2^block_shift keys
     int32_t target_items;                  // work items the launch wants at least (heads are split to reach it)
     int32_t H, D, nd, total_rows;
     int64_t N, W;
@@ -31,13 +31,9 @@ struct AttnArgs {
 };
 
 // Persistent workgroups, one head (or pair of heads) each with its table slices in LDS; lane = one query of some
-// window, which streams that window's keys; VALU math, any dtype.  Needs a.workspace (work queues, sorted window
-// list, unit list), a.partials, a.block_shift (key blocks of 64 << shift keys) and a.max_key_tiles (key blocks of
-// the largest window).
-int attn_generic_block_shift(int H, int64_t N, int64_t W, int max_window_voxels);
-int attn_generic_key_blocks(int H, int64_t N, int64_t W, int max_window_voxels);
-size_t attn_generic_workspace_bytes(int H, int D, int64_t W, int64_t N, int max_window_voxels);
-float *attn_generic_partials(void *workspace, int H, int64_t W, int64_t N, int max_window_voxels);
+// window, which streams that window's keys; VALU math, any dtype, windows of any size.  Needs a.workspace (work
+// queues, sorted window list, unit list); a.n2n may be null (rows already in window-sorted order).
+size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N);
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.

@@ -89,11 +89,19 @@ def _as_int32(name, t, device):
 
 
 def _host_table_sizes(table_sizes):
-    """The op reads the per-axis table sizes on the host.  A CUDA tensor (what the reference's
-    caller builds on every call) costs one synchronising device-to-host copy here; pass a list
-    or a CPU tensor to avoid it."""
+    """The op reads the per-axis table sizes on the host.  A CUDA tensor costs one synchronising
+    device-to-host copy; the values are then kept on the tensor object (with its version counter), so a
+    module that keeps its table_offsets tensor pays the copy once.  The reference's caller builds a new
+    tensor from a Python list on every call (Swin3D/modules/swin3d_layers.py:511): pass the list, or a CPU
+    tensor, to avoid the copy altogether."""
     if isinstance(table_sizes, torch.Tensor):
-        return [int(x) for x in table_sizes.reshape(-1).tolist()]
+        if not table_sizes.is_cuda:
+            return [int(x) for x in table_sizes.reshape(-1).tolist()]
+        kept = getattr(table_sizes, "_s3d_host_sizes", None)
+        if kept is None or kept[0] != table_sizes._version:
+            kept = (table_sizes._version, [int(x) for x in table_sizes.reshape(-1).tolist()])
+            table_sizes._s3d_host_sizes = kept
+        return list(kept[1])
     return [int(x) for x in table_sizes]
 
 
@@ -107,14 +115,17 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
     table_sizes    int tensor / list [nd], per-axis element counts rows*H*D (read on the host)
     w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
-    n2n            [N] window-sorted position -> row of q/k/v
+    n2n            [N] window-sorted position -> row of q/k/v, or None when the rows are in window-sorted
+                   order already (the sweep kernel then reads and writes them without the indirection)
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
     force_generic  run the VALU sweep kernel for every case
     force_mfma     run the MFMA kernel wherever it applies (fp16, axis tables of at most 64 rows); by default
                    it serves head_dim 16 only
     max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
-                   (set by build_window_index) or, failing that, read back from the device
+                   (set by build_window_index) when not given.  Without a bound the sweep kernel serves the
+                   call (it takes windows of any size); the host waits for the device to find one only under
+                   force_mfma
     """
     _require_cuda("query", q, strided_rows=True)
     dev = q.device
@@ -154,11 +165,14 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     w_sizes_in = w_sizes
     w_sizes = _as_int32("w_sizes", w_sizes, dev)
     w2n = _as_int32("w2n_indices", w2n, dev)
-    n2n = _as_int32("n2n_indices", n2n, dev)
+    if n2n is not None:
+        n2n = _as_int32("n2n_indices", n2n, dev)
+        if n2n.shape != (n,):
+            raise ValueError(f"n2n_indices must be [{n}], got {tuple(n2n.shape)}")
+    elif force_mfma:
+        raise ValueError("the MFMA kernel needs n2n_indices")
     if w_sizes.shape != w2n.shape or w_sizes.dim() != 1:
         raise ValueError("w_sizes and w2n_indices must be 1-D of equal length")
-    if n2n.shape != (n,):
-        raise ValueError(f"n2n_indices must be [{n}], got {tuple(n2n.shape)}")
     _require_cuda("n_coords", n_coords, dev)
     if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
         raise ValueError(f"n_coords must be float32 [{n},{nd}], got {n_coords.dtype} {tuple(n_coords.shape)}")
@@ -168,9 +182,10 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     if max_window_voxels is None:
         max_window_voxels = getattr(w_sizes_in, "max_window_voxels", None)
-    if max_window_voxels is None:
+    max_window_voxels = max(int(max_window_voxels), 0) if max_window_voxels is not None else 0
+    if force_mfma and max_window_voxels < 1:
+        # the MFMA kernel needs the bound: forcing it without one costs a device read-back
         max_window_voxels = int(w_sizes.max().item()) if w_sizes.numel() else 1
-    max_window_voxels = max(int(max_window_voxels), 1)
     lib = _lib.lib()
     with torch.cuda.device(dev):
         ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, w_sizes.numel(), max_window_voxels)
@@ -179,7 +194,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
         status = lib.s3d_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), table_q.data_ptr(), table_k.data_ptr(),
             table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
-            w2n.data_ptr(), n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(),
+            w2n.data_ptr(), n2n.data_ptr() if n2n is not None else None, n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
             n, h, d, w_sizes.numel(), max_window_voxels, row_stride, _DTYPE_CODE[q.dtype],
             (_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |

@@ -15,7 +15,8 @@ def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", 
         t(case.q).to(dtype), t(case.k).to(dtype), t(case.v).to(dtype),
         t(case.tq).to(dtype), t(case.tk).to(dtype), t(case.tv).to(dtype),
         t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
-        return_stats=return_stats, force_generic=force_generic, force_mfma=force_mfma)
+        return_stats=return_stats, force_generic=force_generic, force_mfma=force_mfma,
+        max_window_voxels=int(i["w_sizes"].max()) if len(i["w_sizes"]) else 0)
     torch.cuda.synchronize()
     if return_stats:
         return tuple(r.double().cpu().numpy() for r in res)

@@ -82,11 +82,11 @@ def test_dense_windows_up_to_343_voxels(oracle_lib, hip_lib, dtype):
     _check(oracle_lib, case, dtype)
 
 
-@pytest.mark.parametrize("heads,block", [(6, 128), (12, 256)])
-def test_long_key_blocks_in_large_dense_launches(oracle_lib, hip_lib, heads, block):
-    """A 56x56x28 grid at 62 % fill, window 7: 256 windows of about 210 voxels.  With this much work per
-    wavefront the sweep kernel streams key blocks of 128 (6 heads) or 256 keys (12 heads) instead of 64, so these
-    windows are split in two or not at all; checked through the partial-result part of the workspace size
+@pytest.mark.parametrize("heads", [6, 12])
+def test_large_dense_windows_stay_inside_a_wavefront(oracle_lib, hip_lib, heads):
+    """A 56x56x28 grid at 62 % fill, window 7: 256 windows of about 210 voxels.  The sweep kernel gives each query
+    of such a window four adjacent lanes that take alternate keys and merge their softmax states by shuffles, so no
+    partial result passes through memory: the workspace holds the work list only, whatever the window sizes
     (quant 5 gives 70-row axis tables, which only the sweep kernel takes, so the size is that kernel's)."""
     import ctypes
     ws, quant, dim = 7, 5, 16
@@ -109,9 +109,8 @@ def test_long_key_blocks_in_large_dense_launches(oracle_lib, hip_lib, heads, blo
     c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
     assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, n, 256) == 0
     ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), heads, dim, n, 256, int(w_sizes.max()))
-    record = n * heads * (dim + 2) * 4           # one partial record per voxel and head
-    blocks = -(-int(w_sizes.max()) // block)     # 2 at 128 keys per block, 1 (no partial results) at 256
-    assert (blocks - 1) * record <= ws_bytes < blocks * record + (8 << 20)
+    assert ws_bytes == hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), heads, dim, n, 256, 0)   # no bound needed
+    assert ws_bytes < 2 * n + 24 * 256 + (1 << 20)     # a unit record per 8 queries, 24 bytes per window, fixed part
     _sharp16(case)
     _check(oracle_lib, case, torch.float16)
 
@@ -213,10 +212,11 @@ def test_stats_outputs(oracle_lib, hip_lib):
 
 
 @pytest.mark.parametrize("kernel", ["sweep", "mfma"])
-def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib, kernel):
-    """max_window_voxels below the real maximum: windows beyond the bound (rounded up to the kernel's key
-    block: 64 voxels for the sweep kernel, 32 for the MFMA kernel) are left out (their output rows keep what
-    the buffer held), every other window is complete, nothing is written out of bounds."""
+def test_understated_window_bound_is_visible(oracle_lib, hip_lib, kernel):
+    """max_window_voxels below the real maximum.  The sweep kernel does not use the bound: every row is complete.
+    The MFMA kernel sizes its partial results with it (rounded up to its key tile of 32 voxels): the rows of
+    windows beyond the bound, and their statistics, read NaN instead of what the buffer held; every other window
+    is complete and nothing is written out of bounds."""
     import swin3d_amd
     case = make_attn_case(oracle_lib, seed=38, n=1000, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
     to_half_and_back(_sharp16(case))
@@ -227,16 +227,22 @@ def test_understated_window_bound_skips_large_windows(oracle_lib, hip_lib, kerne
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     h = lambda a: t(a).half()
     i = case.index
-    got = swin3d_amd.window_attention_forward(
+    got, gmax, gsum = swin3d_amd.window_attention_forward(
         h(case.q), h(case.k), h(case.v), h(case.tq), h(case.tk), h(case.tv), t(case.table_sizes),
-        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32,
+        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32, return_stats=True,
         force_generic=kernel == "sweep", force_mfma=kernel == "mfma")
     torch.cuda.synchronize()
     got = got.double().cpu().numpy()
     small = np.repeat(w_sizes <= 32, w_sizes)           # per sorted position
-    rows_small = i["n2n"][small]
+    rows_small, rows_large = i["n2n"][small], i["n2n"][~small]
     from gpu_helpers import assert_attn_close
     assert_attn_close(got[rows_small], ref[rows_small], torch.float16)
+    if kernel == "sweep":
+        assert_attn_close(got[rows_large], ref[rows_large], torch.float16)
+    else:
+        assert np.isnan(got[rows_large]).all()
+        assert torch.isnan(gmax[t(rows_large).long()]).all() and torch.isnan(gsum[t(rows_large).long()]).all()
+        assert np.isfinite(got[rows_small]).all()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
