@@ -122,6 +122,27 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
                  int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same forward without a workspace argument and without any allocation.
+ *
+ * It has no counterpart in the reference.  It is for callers that cannot allocate device memory around the
+ * call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Always the sweep
+ * kernel (the MFMA kernel's partial results do not fit a fixed buffer); its work list lives in a device array of
+ * 8 MiB that is part of the library's code object, one copy per GPU, held until the process ends.  The call
+ * fails with S3D_ERR_WORKSPACE when s3d_attn_fwd_workspace_bytes(table_sizes, nd, H, D, N, W, 0) exceeds
+ * 8 MiB (about 2 N + 24 W bytes + 0.3 MB: e.g. one million voxels in up to 200 000 windows fit).  The first
+ * call on a device looks up the array's address there (hipGetSymbolAddress); no call allocates or frees.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two host
+ * threads) race on it and must be serialised by the caller; calls in stream order on one stream are safe,
+ * and nothing is carried over from one call to the next.
+ * Arguments, results and status codes as for s3d_attn_fwd.
+ */
+int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void *table_q,
+                         const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
+                         int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
+                         const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
+                         int32_t H, int32_t D, int64_t W, int64_t qkv_row_stride, int32_t dtype, void *stream);
+
+/*
  * Windowed self-attention backward.
  *
  * Replaces cal_exp_sum_grads and self_attn_indir_backward

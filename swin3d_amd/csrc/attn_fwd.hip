@@ -1,6 +1,8 @@
 // Entry point of the windowed self-attention forward: argument checks and kernel choice.
 #include "attn_kernels.h"
 
+#include <mutex>
+
 namespace s3d {
 namespace {
 
@@ -92,24 +94,26 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
     return attn_mfma_supported(a, dtype) && attn_mfma_preferred(a) ? 1 : 0;
 }
 
-extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
-    const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
-    const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
-    const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
-    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W,
-    int32_t max_window_voxels, int64_t qkv_row_stride, int32_t dtype, int32_t flags, void *workspace,
-    size_t workspace_bytes, void *stream)
+namespace s3d {
+namespace {
+
+// Argument checks shared by the two forward entry points; fills `a` (everything but the workspace).
+// *empty is set when there is nothing to compute.
+int prepare_attn_args(const char *who, AttnArgs &a, bool *empty, const void *q, const void *k, const void *v,
+                      const void *table_q, const void *table_k, const void *table_v, const int32_t *table_sizes,
+                      int32_t nd, int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
+                      const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N, int32_t H,
+                      int32_t D, int64_t W, int64_t qkv_row_stride, int32_t dtype)
 {
-    using namespace s3d;
+    *empty = true;
     if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
     if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
-        return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_fwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
-    if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_fwd: table_sizes (host) is null");
+        return fail(S3D_ERR_BAD_DTYPE, "%s: dtype %d (0 = fp32, 1 = fp16)", who, dtype);
+    if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "%s: table_sizes (host) is null", who);
     // rows of q, k, v are read with 16-byte loads: the stride must keep them aligned
     if (qkv_row_stride != 0 && (qkv_row_stride < static_cast<int64_t>(H) * D || qkv_row_stride % 8 != 0))
-        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: qkv_row_stride = %lld (0, or a multiple of 8 that is >= H*D = %d)",
+        return fail(S3D_ERR_BAD_SHAPE, "%s: qkv_row_stride = %lld (0, or a multiple of 8 that is >= H*D = %d)", who,
                     (long long)qkv_row_stride, H * D);
-    AttnArgs a{};
     a.H = H;
     a.D = D;
     a.nd = nd;
@@ -118,7 +122,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
     if (N == 0 || W == 0) return S3D_OK;
     if (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n_coords || !out)
-        return fail(S3D_ERR_NULL_POINTER, "s3d_attn_fwd: null device pointer");
+        return fail(S3D_ERR_NULL_POINTER, "%s: null device pointer", who);
     a.q = q;
     a.k = k;
     a.v = v;
@@ -133,6 +137,55 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.out = out;
     a.out_max = out_max;
     a.out_sum = out_sum;
+    *empty = false;
+    return S3D_OK;
+}
+
+// Scratch of s3d_attn_fwd_noalloc: the sweep kernel's work list (queue counters, unit and window records, the
+// list builder's notes) in a device array that lives as long as the process, one copy per GPU.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; kernels and copies get the address it returns.
+constexpr size_t kScratchBytes = size_t(8) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+void *scratch_address[kMaxDevices];   // per device; looked up on the first call there
+std::mutex scratch_mutex;
+
+int scratch_of_current_device(void **address)
+{
+    int device = -1;
+    S3D_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd_noalloc: device %d (at most %d devices)", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_address[device]) {
+        void *p = nullptr;
+        S3D_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd_noalloc: no device address for the scratch array");
+        scratch_address[device] = p;
+    }
+    *address = scratch_address[device];
+    return S3D_OK;
+}
+
+}  // namespace
+}  // namespace s3d
+
+extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
+    const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
+    const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
+    const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
+    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W,
+    int32_t max_window_voxels, int64_t qkv_row_stride, int32_t dtype, int32_t flags, void *workspace,
+    size_t workspace_bytes, void *stream)
+{
+    using namespace s3d;
+    AttnArgs a{};
+    bool empty = true;
+    if (int rc = prepare_attn_args("s3d_attn_fwd", a, &empty, q, k, v, table_q, table_k, table_v, table_sizes, nd,
+                                   table_len, w_sizes, w2n, n2n, n_coords, out, out_max, out_sum, N, H, D, W,
+                                   qkv_row_stride, dtype))
+        return rc;
+    if (empty) return S3D_OK;
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the MFMA kernel needs the window bound (it sizes partial results with it) and the row map
@@ -153,4 +206,32 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
     return launch_attn_generic(a, dtype, s);
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_noalloc(
+    const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
+    const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
+    const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
+    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W, int64_t qkv_row_stride,
+    int32_t dtype, void *stream)
+{
+    using namespace s3d;
+    AttnArgs a{};
+    bool empty = true;
+    if (int rc = prepare_attn_args("s3d_attn_fwd_noalloc", a, &empty, q, k, v, table_q, table_k, table_v, table_sizes,
+                                   nd, table_len, w_sizes, w2n, n2n, n_coords, out, out_max, out_sum, N, H, D, W,
+                                   qkv_row_stride, dtype))
+        return rc;
+    if (empty) return S3D_OK;
+    const size_t need = attn_generic_workspace_bytes(H, W, N);
+    if (need > kScratchBytes)
+        return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd_noalloc: N = %lld voxels in W = %lld windows need %zu B of work "
+                    "list, the built-in scratch holds %zu B; use s3d_attn_fwd with a workspace",
+                    (long long)N, (long long)W, need, kScratchBytes);
+    void *address = nullptr;
+    if (int rc = scratch_of_current_device(&address)) return rc;
+    a.workspace = address;
+    // the list kernels write every word of the work list that the sweep kernel reads (the queue counters
+    // included), so nothing of an earlier call's contents is used
+    return launch_attn_generic(a, dtype, static_cast<hipStream_t>(stream));
 }
