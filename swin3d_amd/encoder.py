@@ -191,18 +191,58 @@ def segment_offsets(batch_column, num_batches=None):
     return torch.cumsum(counts, 0).to(torch.int32)
 
 
-class StemConv(nn.Module):
-    """3x3x3 sparse convolution + BatchNorm + ReLU."""
+class _ConvKernel(nn.Module):
+    """Holds the stem convolution's weight under the name MinkowskiConvolution gives it: `kernel`
+    [27, Cin, Cout] (kernel volume, in, out)."""
 
     def __init__(self, in_channels, out_channels):
         super().__init__()
-        self.weight = nn.Parameter(torch.empty(27, in_channels, out_channels))
-        nn.init.kaiming_normal_(self.weight.view(27 * in_channels, out_channels).t())
-        self.norm = nn.BatchNorm1d(out_channels)
+        self.kernel = nn.Parameter(torch.empty(27, in_channels, out_channels))
+        nn.init.kaiming_normal_(self.kernel.view(27 * in_channels, out_channels).t())
+
+
+class _BatchNorm(nn.Module):
+    """BatchNorm1d under the name MinkowskiBatchNorm gives it: `bn`."""
+
+    def __init__(self, channels):
+        super().__init__()
+        self.bn = nn.BatchNorm1d(channels)
+
+    def forward(self, x):
+        return self.bn(x)
+
+
+class StemConv(nn.Module):
+    """3x3x3 sparse convolution + BatchNorm + ReLU (MinkConvBNRelu, Swin3D/modules/mink_layers.py:50-80).  The
+    parameters carry the reference's checkpoint names: `conv_layers.0.kernel` and `conv_layers.1.bn.*`.  The
+    27 kernel offsets are ordered x-major here; which order MinkowskiEngine uses for its kernel rows is not
+    pinned by anything available offline, so a stem loaded from a published checkpoint is parity unpinned."""
+
+    def __init__(self, in_channels, out_channels):
+        super().__init__()
+        self.conv_layers = nn.Sequential(_ConvKernel(in_channels, out_channels), _BatchNorm(out_channels))
+
+    @property
+    def weight(self):
+        return self.conv_layers[0].kernel
 
     def forward(self, voxels, neighbours=None):
         out = sparse_conv3x3x3(voxels, self.weight, neighbours)
-        return voxels.with_feats(F.relu(self.norm(out.float())))
+        return voxels.with_feats(F.relu(self.conv_layers[1](out.float())))
+
+
+class Mlp(nn.Module):
+    """fc1 -> GELU -> fc2 with the reference's attribute names (Swin3D/modules/swin3d_layers.py:153-176);
+    dropout is 0 in every shipped configuration and left out."""
+
+    def __init__(self, in_features, hidden_features):
+        super().__init__()
+        self.fc1 = nn.Linear(in_features, hidden_features)
+        self.act = nn.GELU()
+        self.fc2 = nn.Linear(hidden_features, in_features)
+
+    def forward(self, x):
+        return self.fc2(self.act(self.fc1(x)))
 
 
 def _fused_norm_applies(feats):
@@ -329,7 +369,7 @@ class SwinBlock(nn.Module):
         self.attn = WindowAttention(dim, window_size, quant_size, num_heads, cRSE, fp16_mode)
         self.norm2 = nn.LayerNorm(dim)
         hidden = int(dim * mlp_ratio)
-        self.mlp = nn.Sequential(nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
+        self.mlp = Mlp(dim, hidden)
 
     def forward(self, feats, attn_args):
         if self._fused_path(feats):
@@ -522,24 +562,22 @@ def load_state_with_same_shape(model, weights, skip_first_conv=False, verbose=Tr
     a `module.` prefix is stripped, decoder (`upsamples`) and `classifier` entries are dropped, so is
     `stem_layer` on request, and so is every entry whose name or shape the model does not have."""
     if weights and next(iter(weights)).startswith("module."):
-        if verbose:
-            print("Loading multigpu weights with module. prefix...")
         weights = {k.partition("module.")[2]: v for k, v in weights.items()}
     model_state = model.state_dict()
-    dropped = [k for k in weights if "upsamples" in k or "classifier" in k]
-    weights = {k: v for k, v in weights.items() if "upsamples" not in k and "classifier" not in k}
-    if skip_first_conv:
-        dropped += [k for k in weights if "stem_layer" in k]
-        weights = {k: v for k, v in weights.items() if "stem_layer" not in k}
-    filtered = {k: v for k, v in weights.items() if k in model_state and v.size() == model_state[k].size()}
-    dropped += [k for k, v in weights.items() if k in model_state and v.size() != model_state[k].size()]
-    missing = [k for k in model_state if k not in weights]
+    wanted = {k: v for k, v in weights.items()
+              if "upsamples" not in k and "classifier" not in k and not (skip_first_conv and "stem_layer" in k)}
+    filtered = {k: v for k, v in wanted.items() if k in model_state and v.size() == model_state[k].size()}
     if verbose:
-        print("Not Loading weights: " + ", ".join(dropped))
-        print("=" * 100)
-        print("Not found weights: " + ", ".join(missing))
-        print("=" * 100)
+        print("checkpoint entries left out:", ", ".join(sorted(set(weights) - set(filtered))) or "none")
+        print("model entries without a checkpoint value:", ", ".join(k for k in model_state if k not in filtered) or "none")
     return filtered
+
+
+def unmatched_encoder_parameters(model, matched):
+    """Parameters and buffers of the encoder stages (`layers.*`) that a filtered checkpoint leaves at their
+    initial values; `num_batches_tracked` counters aside."""
+    return [k for k in model.state_dict()
+            if k.startswith("layers.") and k not in matched and not k.endswith("num_batches_tracked")]
 
 
 class Swin3DUNet(nn.Module):
@@ -586,9 +624,11 @@ class Swin3DUNet(nn.Module):
             signals = signals_up
         return self.classifier(voxels.feats.float())
 
-    def load_pretrained_model(self, ckpt, skip_first_conv=True, verbose=True):
+    def load_pretrained_model(self, ckpt, skip_first_conv=True, verbose=True, strict_encoder=True):
         """Load the entries of a checkpoint that fit (Swin3D/models/Swin3D.py:173-183); the file is read
-        with a loader that executes nothing from it."""
+        with a loader that executes nothing from it.  The reference loads with strict=False and says nothing
+        about stages that got no weights; here, with strict_encoder, a checkpoint that leaves any parameter
+        of the encoder stages (`layers.*`) without a value raises instead of leaving it at random."""
         import os
         if not os.path.isfile(ckpt):
             if verbose:
@@ -597,6 +637,10 @@ class Swin3DUNet(nn.Module):
         checkpoint = torch.load(ckpt, map_location="cpu", weights_only=True)
         weights = checkpoint["state_dict"] if "state_dict" in checkpoint else checkpoint
         matched = load_state_with_same_shape(self, weights, skip_first_conv=skip_first_conv, verbose=verbose)
+        left = unmatched_encoder_parameters(self, matched)
+        if strict_encoder and left:
+            raise RuntimeError(f"checkpoint '{ckpt}' has no fitting value for {len(left)} encoder entries: "
+                               + ", ".join(left[:8]) + (" ..." if len(left) > 8 else ""))
         self.load_state_dict(matched, strict=False)
         if verbose:
             print("=> loaded weight '{}'".format(ckpt))

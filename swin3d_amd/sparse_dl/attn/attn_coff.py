@@ -43,6 +43,9 @@ class PrecisionMode(enum.Enum):
 
 _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_F16}
 
+# s3d_attn_bwd keeps a head's table gradients in registers: at most 64 rows per axis on average
+BWD_MAX_ROWS_PER_AXIS = 64
+
 # debugging / ablation switch: run the generic VALU kernel even where the MFMA kernel applies
 FORCE_GENERIC = False
 
@@ -232,8 +235,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_len:
         raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
                          f"to the table length {table_len}")
-    if sum(sizes) // (h * d) > 64 * nd:
-        raise NotImplementedError(f"attention backward supports at most {64 * nd} table rows per head")
+    if sum(sizes) // (h * d) > BWD_MAX_ROWS_PER_AXIS * nd:
+        raise NotImplementedError(f"attention backward supports at most {BWD_MAX_ROWS_PER_AXIS * nd} table rows per head")
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
         if t.dtype != q.dtype or t.numel() != table_len:
@@ -297,6 +300,15 @@ class SelfAttnAIOFunction(Function):
         tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
         n_coords = n_coords.to(torch.float32).contiguous()
         needs_grad = any(ctx.needs_input_grad[:6])
+        if needs_grad:
+            # the backward's limit, reported where the op is called and not from inside autograd
+            sizes = _host_table_sizes(table_offsets)
+            rows = sum(sizes) // max(raw_query_feats.shape[1] * raw_query_feats.shape[2], 1)
+            if rows > BWD_MAX_ROWS_PER_AXIS * len(sizes):
+                raise NotImplementedError(
+                    f"attention backward supports at most {BWD_MAX_ROWS_PER_AXIS} table rows per axis on average "
+                    f"({BWD_MAX_ROWS_PER_AXIS * len(sizes)} per head for {len(sizes)} axes), got {rows}; "
+                    "run the forward under torch.no_grad() or use smaller tables")
         res = window_attention_forward(*feats, *tables, table_offsets, w_sizes, w2n, n2n, n_coords,
                                        return_stats=needs_grad)
         if not needs_grad:
