@@ -23,11 +23,35 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
-# HBM bytes per s3d_attn_fwd call from the FETCH_SIZE / WRITE_SIZE passes recorded in
-# profiles/attn_fwd_headline.txt (sweep kernel + partial merge + the two list kernels): fetch
-# (58869 + 282 + 212) KiB * 2.00, write (21892 + 98 + 280) KiB * 1.00, factors from the 64 MiB copy
-VALU_ISSUE_FRAC = 0.77   # share of the sweep kernel's clocks in which a SIMD issues a VALU instruction
-MEASURED_TRAFFIC_BYTES = int(((58869 + 282 + 212) * 2.00 + (21892 + 98 + 280) * 1.00) * 1024)
+HEADLINE_PROFILE = os.path.join("profiles", "attn_fwd_headline.txt")
+# the sources of the headline kernel: counter figures taken from a profile are only quoted while these are unchanged
+KERNEL_SOURCES = ["attn_fwd.hip", "attn_fwd_generic.hip", "attn_kernels.h", "sweep_common.h", "s3d_common.h"]
+
+
+def kernel_sources_sha256():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "swin3d_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def profile_figures():
+    """Counter-derived figures of the headline kernel (HBM traffic per call from FETCH_SIZE / WRITE_SIZE, VALU
+    issue share) are not measured by this program: they come from the rocprofv3 --pmc runs summarised in
+    HEADLINE_PROFILE, whose `key: value` lines under "machine-readable" also record the hash of the kernel
+    sources they were taken with.  -> (figures dict, still valid for the sources in the tree)"""
+    figures = {}
+    try:
+        with open(os.path.join(ROOT, HEADLINE_PROFILE)) as f:
+            for line in f:
+                key, sep, value = line.partition(":")
+                if sep and key.strip() in ("sources_sha256", "traffic_bytes", "valu_issue_frac", "sweep_kernel_us"):
+                    figures[key.strip()] = value.strip()
+    except OSError:
+        return {}, False
+    return figures, figures.get("sources_sha256") == kernel_sources_sha256()
 
 
 def algorithmic_bytes(n, c, elem_bytes, nd, w, table_len):
@@ -46,10 +70,15 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-encoder", action="store_true",
                     help="skip the Swin3D-L encoder end-to-end latency")
+    ap.add_argument("--sources-hash", action="store_true",
+                    help="print the hash of the headline kernel's sources (recorded in the profile summary) and exit")
     ap.add_argument("--encoder-only", action="store_true",
                     help="run only the Swin3D-L encoder forward (1 warm-up + 3 timed passes, no UNet) and print its "
                          "figures: the command the encoder's kernel trace is taken with")
     args = ap.parse_args()
+    if args.sources_hash:
+        print(kernel_sources_sha256())
+        return 0
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (windows are independent, so the path would shard over "
               "windows or scenes without any exchange); --gpus must be 1", file=sys.stderr)
@@ -98,13 +127,25 @@ def main():
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
 
-    def step():
+    # The sweep kernel's work list depends on the window set only; like the index arrays it is built once per set
+    # and shared by the blocks that use the set (s3d_attn_plan), so the timed call runs on a prebuilt plan.  The
+    # same call with the list built inside it is timed beside it (kernel_ms.with_list_build).
+    planned = args.flags == 0 and not lib.s3d_attn_fwd_uses_mfma(c_sizes, nd, heads, dim, _lib.S3D_DTYPE_F16, n, num_w)
+    plan = torch.empty(max(lib.s3d_attn_plan_bytes(heads, n, num_w), 1), dtype=torch.uint8, device=dev)
+    if planned:
+        _lib.check(lib.s3d_attn_plan(c_sizes, nd, table_len, index.w_sizes.data_ptr(), index.w2n.data_ptr(), n, heads, dim,
+                                     num_w, _lib.S3D_DTYPE_F16, plan.data_ptr(), plan.numel(), stream.cuda_stream),
+                   "s3d_attn_plan")
+
+    def step(use_plan=planned):
         status = lib.s3d_attn_fwd(q_d.data_ptr(), k_d.data_ptr(), v_d.data_ptr(), tq_d.data_ptr(),
                                   tk_d.data_ptr(), tv_d.data_ptr(), c_sizes, nd, table_len,
                                   index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
                                   n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16, args.flags, workspace.data_ptr(), ws_bytes,
-                                  stream.cuda_stream)
+                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16,
+                                  (args.flags | _lib.S3D_ATTN_PLANNED) if use_plan else args.flags,
+                                  plan.data_ptr() if use_plan else workspace.data_ptr(),
+                                  plan.numel() if use_plan else ws_bytes, stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")
 
@@ -151,15 +192,23 @@ def main():
         "voxels_per_s": n / (wall_ms * 1e-3),
         "kernel_ms": {"mean": kernel_ms, "median": float(np.median(launch_ms)),
                       "p10": float(np.percentile(launch_ms, 10)), "p90": float(np.percentile(launch_ms, 90))},
+        # achieved / frac: algorithmic bytes of this run over the launch time measured in this run.  traffic is a
+        # counter figure: it is quoted from the committed profile only while the kernel sources are the ones the
+        # profile was taken with (from_profile says so), and is null otherwise
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES if args.flags == 0 else None,
-                     "algorithmic_bytes": bytes_alg,
-                     # what the dominant kernel is bound by instead (constant from the committed profile:
-                     # SQ_INSTS_VALU * 4 clocks / 1024 SIMDs against the kernel's clocks)
-                     "limiter": ({"kind": "valu_issue", "frac": VALU_ISSUE_FRAC,
-                                  "source": "profiles/attn_fwd_headline.txt"} if args.flags == 0 else None)},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": bytes_alg},
     }
+    figures, current = profile_figures()
+    if args.flags == 0 and figures:
+        result["roofline"]["from_profile"] = {
+            "file": HEADLINE_PROFILE, "sources_sha256": figures.get("sources_sha256"),
+            "matches_sources_in_tree": current,
+            "sweep_kernel_us": float(figures["sweep_kernel_us"]) if "sweep_kernel_us" in figures else None}
+        if current:
+            result["roofline"]["traffic"] = int(figures["traffic_bytes"]) if "traffic_bytes" in figures else None
+            if "valu_issue_frac" in figures:
+                result["roofline"]["from_profile"]["limiter"] = {"kind": "valu_issue",
+                                                                 "frac": float(figures["valu_issue_frac"])}
 
     # cold figure: a 512 MiB fill between launches evicts q/k/v and the tables from L2 and the
     # Infinity Cache (outside the timed steps above; 10 launches)
@@ -175,6 +224,17 @@ def main():
         cold.append(s_ev.elapsed_time(e_ev))
     del flush
     result["kernel_ms"]["cold_median"] = float(np.median(cold))
+    result["kernel_ms"]["planned"] = bool(planned)
+    if planned:
+        unplanned = []
+        for _ in range(20):
+            s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_ev.record(stream)
+            step(use_plan=False)
+            e_ev.record(stream)
+            torch.cuda.synchronize()
+            unplanned.append(s_ev.elapsed_time(e_ev))
+        result["kernel_ms"]["with_list_build"] = float(np.median(unplanned))
 
     # one plain device-to-device copy of known size (64 MiB read + 64 MiB written): the yardstick
     # that the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled against

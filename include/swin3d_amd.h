@@ -86,7 +86,8 @@ const char *s3d_last_error_string(void);
  *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
  *                  place, without the reference's reshape / permute / contiguous copy.
  *   flags          0 (the library picks the kernel), S3D_ATTN_FORCE_GENERIC to run the VALU sweep kernel
- *                  for every case, or S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies
+ *                  for every case, S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies, or
+ *                  S3D_ATTN_PLANNED (sweep kernel on a work list built by s3d_attn_plan, see below)
  *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes.  Sweep kernel:
  *                  work-queue counters, one record per unit of 8 to 64 queries and one per window, about
  *                  2 N + 24 W bytes + 0.3 MB.  MFMA kernel: a transposed copy of the value table, the work
@@ -107,6 +108,7 @@ const char *s3d_last_error_string(void);
  */
 #define S3D_ATTN_FORCE_GENERIC 1
 #define S3D_ATTN_FORCE_MFMA 2
+#define S3D_ATTN_PLANNED 4   /* `workspace` holds a plan written by s3d_attn_plan: see there */
 /* 1 if s3d_attn_fwd with flags 0 runs these shapes on the MFMA kernel (fp16, head_dim 16, every axis
  * table <= 64 rows, and windows of at least 256 voxels on average, N >= 256 W, or 60 with 16 heads or more),
  * 0 if on the VALU sweep kernel.  No counterpart in the reference (it has one kernel). */
@@ -120,6 +122,24 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
                  const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
                  int32_t H, int32_t D, int64_t W, int32_t max_window_voxels, int64_t qkv_row_stride,
                  int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Work list of the sweep kernel, built once per window set ("plan").
+ *
+ * The reference builds its O(pairs) index arrays once per window set and hands them to every attention call
+ * of the blocks that share the set (Swin3D/modules/swin3d_layers.py:857-871: one `get_index01` per window
+ * set, `indices` reused by the blocks).  The counterpart here is O(N + W): the windows sorted by size and cut into
+ * units of 64 lanes.  s3d_attn_fwd builds it on every call (two small kernels); a caller that keeps a window set
+ * for several calls builds it once with s3d_attn_plan and passes the plan buffer as `workspace` together with
+ * the flag S3D_ATTN_PLANNED, for calls with the same w_sizes, w2n, N, W, H, D, dtype and table_sizes.  Such a call
+ * runs the sweep kernel and nothing else.  The plan holds the launch's work counters, which a launch leaves at
+ * zero again: a plan serves one call at a time (calls in stream order; not two streams at once).
+ *   plan           device buffer of at least s3d_attn_plan_bytes(H, N, W) bytes
+ */
+size_t s3d_attn_plan_bytes(int32_t H, int64_t N, int64_t W);
+int s3d_attn_plan(const int32_t *table_sizes, int32_t nd, int64_t table_len, const int32_t *w_sizes,
+                  const int32_t *w2n, int64_t N, int32_t H, int32_t D, int64_t W, int32_t dtype, void *plan,
+                  size_t plan_bytes, void *stream);
 
 /*
  * The same forward without a workspace argument and without any allocation.

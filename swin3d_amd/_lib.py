@@ -14,6 +14,7 @@ S3D_DTYPE_F16 = 1
 KNN_KMAX = 64
 S3D_ATTN_FORCE_GENERIC = 1
 S3D_ATTN_FORCE_MFMA = 2
+S3D_ATTN_PLANNED = 4
 
 _lib = None
 
@@ -29,6 +30,8 @@ SIGNATURES = {
     "s3d_attn_fwd_workspace_bytes": (ctypes.c_size_t, [_vp, _i32, _i32, _i32, _i64, _i64, _i32]),
     "s3d_attn_fwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
                      [_i64, _i32, _i32, _i64, _i32, _i64, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
+    "s3d_attn_plan_bytes": (ctypes.c_size_t, [_i32, _i64, _i64]),
+    "s3d_attn_plan": (ctypes.c_int, [_vp, _i32, _i64, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_attn_fwd_noalloc": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
                              [_i64, _i32, _i32, _i64, _i64, _i32, _vp]),
     "s3d_attn_bwd_workspace_bytes": (ctypes.c_size_t, [_i32, _i32, _i32, _i64, _i64]),

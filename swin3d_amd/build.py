@@ -33,7 +33,8 @@ def _hipcc():
 
 def _compile(src):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    extra = os.environ.get("S3D_HIPCC_EXTRA", "").split()   # e.g. -D switches of a kernel experiment
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass reports that it does not know the device-only target feature
     log = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)

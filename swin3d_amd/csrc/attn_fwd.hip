@@ -189,7 +189,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the MFMA kernel needs the window bound (it sizes partial results with it) and the row map
-    const bool want_mfma = !(flags & S3D_ATTN_FORCE_GENERIC) && max_window_voxels >= 1 && n2n &&
+    const bool want_mfma = !(flags & (S3D_ATTN_FORCE_GENERIC | S3D_ATTN_PLANNED)) && max_window_voxels >= 1 && n2n &&
                            attn_mfma_supported(a, dtype) && (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
     if (want_mfma) {
         const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
@@ -205,7 +205,41 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
-    return launch_attn_generic(a, dtype, s);
+    // with a plan the work list is in the workspace already
+    return launch_attn_generic(a, dtype, s, (flags & S3D_ATTN_PLANNED) ? kAttnSweep : (kAttnBuildList | kAttnSweep));
+}
+
+extern "C" __attribute__((visibility("default"))) size_t s3d_attn_plan_bytes(int32_t H, int64_t N, int64_t W)
+{
+    if (H < 1 || N < 0 || W < 0) return 0;
+    return s3d::attn_generic_workspace_bytes(H, W, N);
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_attn_plan(
+    const int32_t *table_sizes, int32_t nd, int64_t table_len, const int32_t *w_sizes, const int32_t *w2n,
+    int64_t N, int32_t H, int32_t D, int64_t W, int32_t dtype, void *plan, size_t plan_bytes, void *stream)
+{
+    using namespace s3d;
+    if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
+    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
+        return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_plan: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_plan: table_sizes (host) is null");
+    AttnArgs a{};
+    a.H = H;
+    a.D = D;
+    a.nd = nd;
+    a.N = N;
+    a.W = W;
+    if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
+    if (N == 0 || W == 0) return S3D_OK;
+    if (!w_sizes || !w2n) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_plan: null device pointer");
+    const size_t need = attn_generic_workspace_bytes(H, W, N);
+    if (!plan || plan_bytes < need)
+        return fail(S3D_ERR_WORKSPACE, "s3d_attn_plan: plan buffer %zu B < required %zu B", plan ? plan_bytes : size_t(0), need);
+    a.w_sizes = w_sizes;
+    a.w2n = w2n;
+    a.workspace = plan;
+    return launch_attn_generic(a, dtype, static_cast<hipStream_t>(stream), kAttnBuildList);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_noalloc(

@@ -66,7 +66,8 @@ __host__ inline int target_shift_for(int64_t N, int64_t W, int waves)
 // entries, the placement notes and per-workgroup bin totals of the list builder
 __host__ __device__ inline size_t ws_round(size_t bytes) { return (bytes + 255) / 256 * 256; }
 __host__ __device__ inline size_t ws_total_offset(int H) { return sizeof(int32_t) * static_cast<size_t>(H) * kQueues * kCounterStride; }
-__host__ __device__ inline size_t ws_units_offset(int H) { return ws_total_offset(H) + 256; }
+// after the totals (one cache line): one exit counter per queue index, each on a cache line of its own
+__host__ __device__ inline size_t ws_units_offset(int H) { return ws_total_offset(H) + 256 * (1 + kQueues); }
 // a unit holds at least 64 >> kMaxSplit = 8 queries, except the last one of each section
 __host__ __device__ inline size_t ws_max_units(int64_t N)
 {
@@ -241,7 +242,11 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
     if (blockIdx.x == 0) {
         // a wavefront reads 64 entries from a unit's first one: pad the list with entries no query belongs to
         if (threadIdx.x < kChunk) entries[total_entries + threadIdx.x] = make_int4(0x7fffffff, 1, 0, -1);
-        if (threadIdx.x == 0) total[0] = sec_unit[kSections];
+        if (threadIdx.x == 0) {
+            total[0] = sec_unit[kSections];
+            total[1] = 0;   // exit counters of a sweep launch: cache lines that are complete, and one per line
+        }
+        if (threadIdx.x < kQueues) total[(1 + threadIdx.x) * kCounterStride] = 0;
         for (int t = threadIdx.x; t < a.H * kQueues; t += kListThreads) counters[t * kCounterStride] = 0;
     }
 }
@@ -278,7 +283,11 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
     constexpr int kKeys = D <= 8 ? 1 : 2;
     // lazy softmax reference (see the loop): -4 % for fp16; fp32 measured no gain (head_dim 8) or a loss (16)
     constexpr bool kLazy = sizeof(T) == 2;
-    extern __shared__ float smem[];
+    // 16-byte aligned like the table rows behind it, which are read 16 bytes at a time
+    extern __shared__ __align__(16) float smem[];
+    __shared__ __align__(16) int group_exit_counter[4];   // [0]: wavefronts of this workgroup that have left their loop
+    int &group_exited = group_exit_counter[0];
+    if (threadIdx.x == 0) group_exited = 0;
     const int H = a.H;
     const int HD = H * D;
     // workgroups go to the XCDs in turn: consecutive runs of eight serve one head group, so every XCD gets every head
@@ -546,10 +555,30 @@ __global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fw
             }
         }
     }
+    // The work list can serve further launches (a plan kept by the caller): the last wavefront of the launch to
+    // leave its loop - by then no wavefront draws tickets any more - puts every queue counter back to zero.  The
+    // exits are counted in three levels (workgroup in LDS, one of kQueues cache lines, all lines), so that no
+    // cache line sees more than a few hundred of these atomics.
+    if (lane == 0 && atomicAdd(&group_exited, 1) == kThreads / 64 - 1) {
+        __threadfence();
+        int *total = static_cast<int *>(a.workspace) + ws_total_offset(H) / sizeof(int);
+        const int groups = static_cast<int>(gridDim.x), line = static_cast<int>(blockIdx.x) % kQueues;
+        const int on_line = (groups - line + kQueues - 1) / kQueues;
+        int *line_counter = total + (1 + line) * kCounterStride;
+        if (atomicAdd(line_counter, 1) == on_line - 1) {
+            *line_counter = 0;
+            if (atomicAdd(total + 1, 1) == min(groups, kQueues) - 1) {
+                total[1] = 0;
+                int *all_counters = static_cast<int *>(a.workspace);
+                for (int t = 0; t < H * kQueues; ++t) all_counters[t * kCounterStride] = 0;
+                __threadfence();
+            }
+        }
+    }
 }
 
 template <typename T, int D, int ND, int HP, bool kSorted>
-int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
+int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
 {
     const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride_heads<T, D, HP>(), 16);
     if (lds > 160 * 1024)
@@ -570,30 +599,36 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream)
     b.block_shift = target_shift_for(a.N, a.W, b.target_items);
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
     const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
-    hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
-    hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b);
-    S3D_HIP_CHECK(hipGetLastError());
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
-    S3D_HIP_CHECK(hipGetLastError());
+    if (what & 1) {
+        hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+        hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+        S3D_HIP_CHECK(hipGetLastError());
+    }
+    if (what & 2) {
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
+        S3D_HIP_CHECK(hipGetLastError());
+    }
     return S3D_OK;
 }
 
 template <typename T, int D, int ND>
-int launch_sweep(const AttnArgs &a, hipStream_t stream)
+int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
 {
     // two heads per wavefront where the registers allow it (head_dim 8, fp16) and the heads pair up
     if constexpr (D <= 8 && sizeof(T) == 2) {
         if (a.H % 2 == 0)
-            return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream) : launch_sweep_heads<T, D, ND, 2, true>(a, stream);
+            return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
+                         : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
     }
-    return a.n2n ? launch_sweep_heads<T, D, ND, 1, false>(a, stream) : launch_sweep_heads<T, D, ND, 1, true>(a, stream);
+    return a.n2n ? launch_sweep_heads<T, D, ND, 1, false>(a, stream, what)
+                 : launch_sweep_heads<T, D, ND, 1, true>(a, stream, what);
 }
 
 template <typename T>
-int dispatch_shape(const AttnArgs &a, hipStream_t stream)
+int dispatch_shape(const AttnArgs &a, hipStream_t stream, int what)
 {
 #define S3D_CASE(DD, NN) \
-    if (a.D == DD && a.nd == NN) return launch_sweep<T, DD, NN>(a, stream);
+    if (a.D == DD && a.nd == NN) return launch_sweep<T, DD, NN>(a, stream, what);
     S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
     S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
 #undef S3D_CASE
@@ -609,11 +644,11 @@ size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N)
     return ws_end_offset(H, W, N);
 }
 
-int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream)
+int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int what)
 {
     switch (dtype) {
-    case S3D_DTYPE_F32: return dispatch_shape<float>(a, stream);
-    case S3D_DTYPE_F16: return dispatch_shape<__half>(a, stream);
+    case S3D_DTYPE_F32: return dispatch_shape<float>(a, stream, what);
+    case S3D_DTYPE_F16: return dispatch_shape<__half>(a, stream, what);
     default: return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_fwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
     }
 }

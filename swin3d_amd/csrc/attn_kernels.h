@@ -34,7 +34,10 @@ struct AttnArgs {
 // window, which streams that window's keys; VALU math, any dtype, windows of any size.  Needs a.workspace (work
 // queues, sorted window list, unit list); a.n2n may be null (rows already in window-sorted order).
 size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N);
-int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream);
+// what: kAttnBuildList (the two list kernels: needs w_sizes, w2n and the shape only), kAttnSweep (the sweep on a
+// work list that is already in a.workspace; the launch leaves it ready for the next one), or both.
+constexpr int kAttnBuildList = 1, kAttnSweep = 2;
+int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int what = kAttnBuildList | kAttnSweep);
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);

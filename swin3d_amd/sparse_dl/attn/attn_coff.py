@@ -108,6 +108,35 @@ def _host_table_sizes(table_sizes):
     return [int(x) for x in table_sizes]
 
 
+# keep the sweep kernel's work list ("plan") on the w_sizes tensor between calls (False: build it in every call)
+REUSE_PLANS = True
+
+
+def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, table_len, n, h, d, code, stream):
+    """The plan buffer (s3d_attn_plan) of this window set and shape, built on first use and kept as an attribute
+    of the caller's w_sizes tensor; None when there is no tensor object to keep it on.  A plan is valid for the
+    contents it was built from (the tensors' version counters are checked) and for one stream (it holds the work
+    counters of the launch that uses it)."""
+    if not isinstance(w_sizes_in, torch.Tensor) or not isinstance(w2n_in, torch.Tensor) or w_sizes.numel() == 0 or n == 0:
+        return None
+    plans = getattr(w_sizes_in, "_s3d_attn_plans", None)
+    if plans is None:
+        plans = w_sizes_in._s3d_attn_plans = {}
+    key = (h, d, code, tuple(sizes), n, stream)
+    stamp = (w_sizes_in._version, w2n_in._version, w2n_in.data_ptr())
+    kept = plans.get(key)
+    if kept is not None and kept[0] == stamp:
+        return kept[1]
+    num_w = w_sizes.numel()
+    nbytes = lib.s3d_attn_plan_bytes(h, n, num_w)
+    plan = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=w_sizes.device)
+    status = lib.s3d_attn_plan(c_sizes, len(sizes), table_len, w_sizes.data_ptr(), w2n.data_ptr(), n, h, d, num_w, code,
+                               plan.data_ptr(), nbytes, stream)
+    _lib.check(status, "s3d_attn_plan")
+    plans[key] = (stamp, plan)
+    return plan
+
+
 def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
                              n_coords, return_stats=False, force_generic=False, max_window_voxels=None,
                              force_mfma=False):
@@ -165,7 +194,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
             raise ValueError("the three tables must have the same number of elements")
     if table_len == 0 or table_len % (h * d) != 0:
         raise ValueError(f"table length {table_len} is not a positive multiple of H*D = {h * d}")
-    w_sizes_in = w_sizes
+    w_sizes_in, w2n_in = w_sizes, w2n
     w_sizes = _as_int32("w_sizes", w_sizes, dev)
     w2n = _as_int32("w2n_indices", w2n, dev)
     if n2n is not None:
@@ -190,19 +219,29 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
         # the MFMA kernel needs the bound: forcing it without one costs a device read-back
         max_window_voxels = int(w_sizes.max().item()) if w_sizes.numel() else 1
     lib = _lib.lib()
+    code = _DTYPE_CODE[q.dtype]
+    num_w = w_sizes.numel()
+    flags = ((_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |
+             (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0))
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, w_sizes.numel(), max_window_voxels)
-        workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
+        # the sweep kernel's work list depends on the window set only: it is built once and kept on the
+        # caller's w_sizes tensor, so the blocks that share a window set share it
+        mfma = (not flags & _lib.S3D_ATTN_FORCE_GENERIC and n2n is not None and max_window_voxels >= 1 and
+                (force_mfma or lib.s3d_attn_fwd_uses_mfma(c_sizes, nd, h, d, code, n, num_w)))
+        plan = None if mfma or not REUSE_PLANS else _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes,
+                                                              table_len, n, h, d, code, stream)
+        if plan is not None:
+            workspace, ws_bytes, flags = plan, plan.numel(), flags | _lib.S3D_ATTN_PLANNED
+        else:
+            ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, num_w, max_window_voxels)
+            workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         status = lib.s3d_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), table_q.data_ptr(), table_k.data_ptr(),
             table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
             w2n.data_ptr(), n2n.data_ptr() if n2n is not None else None, n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
-            n, h, d, w_sizes.numel(), max_window_voxels, row_stride, _DTYPE_CODE[q.dtype],
-            (_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |
-            (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0), workspace.data_ptr(),
-            ws_bytes, stream)
+            n, h, d, num_w, max_window_voxels, row_stride, code, flags, workspace.data_ptr(), ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
     if return_stats:
         return out, omax, osum

@@ -460,3 +460,63 @@ def test_swin3d_l_stage1_shape(oracle_lib, hip_lib):
     to_half_and_back(case)
     got = run_attention(case, torch.float16)
     _sampled_parity(oracle_lib, case, got, torch.float16, 300)
+
+
+def test_planned_forward_reuses_one_work_list(oracle_lib, hip_lib):
+    """s3d_attn_plan + S3D_ATTN_PLANNED through the C ABI: the sweep on a work list built once gives the bits of the
+    call that builds its own, on every one of several launches in a row (a launch leaves the plan's work counters
+    at zero for the next one); and the Python wrapper keeps one plan per window set on the w_sizes tensor."""
+    import ctypes
+    import swin3d_amd
+    from swin3d_amd import _lib
+    from swin3d_amd.sparse_dl.attn import attn_coff
+    case = make_attn_case(oracle_lib, seed=71, n=5000, ws=7, quant=4, heads=6, dim=16, extent=(28, 28, 8), recipe="layer")
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    h16 = lambda a: t(a).half()
+    i = case.index
+    q, k, v, tq, tk, tv = (h16(x) for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv))
+    w_sizes, w2n, n2n, n_coords = t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)
+    n, h, d = q.shape
+    w = w_sizes.numel()
+    sizes = [int(x) for x in case.table_sizes]
+    c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(flags, workspace, out):
+        status = hip_lib.s3d_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                      c_sizes, len(sizes), tq.numel(), w_sizes.data_ptr(), w2n.data_ptr(), n2n.data_ptr(),
+                                      n_coords.data_ptr(), out.data_ptr(), None, None, n, h, d, w, 0, 0, _lib.S3D_DTYPE_F16,
+                                      flags, workspace.data_ptr(), workspace.numel(), stream)
+        _lib.check(status, "s3d_attn_fwd")
+
+    ws = torch.empty(hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), h, d, n, w, 0), dtype=torch.uint8, device=dev)
+    ref = torch.empty_like(q)
+    call(_lib.S3D_ATTN_FORCE_GENERIC, ws, ref)
+    plan = torch.empty(hip_lib.s3d_attn_plan_bytes(h, n, w), dtype=torch.uint8, device=dev)
+    _lib.check(hip_lib.s3d_attn_plan(c_sizes, len(sizes), tq.numel(), w_sizes.data_ptr(), w2n.data_ptr(), n, h, d, w,
+                                     _lib.S3D_DTYPE_F16, plan.data_ptr(), plan.numel(), stream), "s3d_attn_plan")
+    for _ in range(3):
+        got = torch.full_like(q, float("nan"))
+        call(_lib.S3D_ATTN_PLANNED, plan, got)
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref)
+    # Python surface: the plan lives on the w_sizes tensor and is built once
+    assert not hasattr(w_sizes, "_s3d_attn_plans")
+    a = swin3d_amd.window_attention_forward(q, k, v, tq, tk, tv, sizes, w_sizes, w2n, n2n, n_coords)
+    (kept,) = w_sizes._s3d_attn_plans.values()
+    b = swin3d_amd.window_attention_forward(q, k, v, tq, tk, tv, sizes, w_sizes, w2n, n2n, n_coords)
+    assert list(w_sizes._s3d_attn_plans.values())[0][1] is kept[1]
+    torch.cuda.synchronize()
+    assert torch.equal(a, ref) and torch.equal(b, ref)
+    # a changed window set invalidates it (in-place edit bumps the tensor's version counter)
+    w_sizes.add_(0)
+    swin3d_amd.window_attention_forward(q, k, v, tq, tk, tv, sizes, w_sizes, w2n, n2n, n_coords)
+    assert list(w_sizes._s3d_attn_plans.values())[0][1] is not kept[1]
+    attn_coff.REUSE_PLANS = False
+    try:
+        c = swin3d_amd.window_attention_forward(q, k, v, tq, tk, tv, sizes, w_sizes, w2n, n2n, n_coords)
+    finally:
+        attn_coff.REUSE_PLANS = True
+    torch.cuda.synchronize()
+    assert torch.equal(c, ref)
