@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-encoder", action="store_true",
                     help="skip the Swin3D-L encoder end-to-end latency")
+    ap.add_argument("--window-ordered", action="store_true",
+                    help="with --encoder-only: keep every level's voxels in the order of its regular windows")
     ap.add_argument("--sources-hash", action="store_true",
                     help="print the hash of the headline kernel's sources (recorded in the profile summary) and exit")
     ap.add_argument("--encoder-only", action="store_true",
@@ -97,7 +99,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.encoder_only:
-        print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False)}))
+        print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False,
+                                                              window_ordered=args.window_ordered)}))
         return 0
 
     # ---- workload: the Swin3D-S stage-1 layer on a 200k-voxel synthetic room ------------------------
@@ -225,16 +228,39 @@ def main():
     del flush
     result["kernel_ms"]["cold_median"] = float(np.median(cold))
     result["kernel_ms"]["planned"] = bool(planned)
-    if planned:
-        unplanned = []
-        for _ in range(20):
-            s_ev, e_ev = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    def back_to_back(fn, reps=30, warm=5):
+        """median launch time as in the timed region above: all calls enqueued, one wait at the end"""
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for s_ev, e_ev in evs:
             s_ev.record(stream)
-            step(use_plan=False)
+            fn()
             e_ev.record(stream)
-            torch.cuda.synchronize()
-            unplanned.append(s_ev.elapsed_time(e_ev))
-        result["kernel_ms"]["with_list_build"] = float(np.median(unplanned))
+        torch.cuda.synchronize()
+        return float(np.median([s_ev.elapsed_time(e_ev) for s_ev, e_ev in evs]))
+
+    if planned:
+        result["kernel_ms"]["with_list_build"] = back_to_back(lambda: step(use_plan=False))
+    # the same call on rows that are in window order already (q, k, v, out permuted by n2n; n2n = identity):
+    # what a caller gets who keeps a stage's voxels in the order of its regular windows
+    ident = torch.arange(n, dtype=torch.int32, device=dev)
+    qs_d, ks_d, vs_d = q_d[order].contiguous(), k_d[order].contiguous(), v_d[order].contiguous()
+
+    def step_ordered():
+        status = lib.s3d_attn_fwd(qs_d.data_ptr(), ks_d.data_ptr(), vs_d.data_ptr(), tq_d.data_ptr(), tk_d.data_ptr(),
+                                  tv_d.data_ptr(), c_sizes, nd, table_len, index.w_sizes.data_ptr(), index.w2n.data_ptr(),
+                                  ident.data_ptr(), n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
+                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16,
+                                  (args.flags | _lib.S3D_ATTN_PLANNED) if planned else args.flags,
+                                  plan.data_ptr() if planned else workspace.data_ptr(),
+                                  plan.numel() if planned else ws_bytes, stream.cuda_stream)
+        if status != 0:
+            _lib.check(status, "s3d_attn_fwd")
+
+    result["kernel_ms"]["window_ordered_rows"] = back_to_back(step_ordered)
+    del qs_d, ks_d, vs_d
 
     # one plain device-to-device copy of known size (64 MiB read + 64 MiB written): the yardstick
     # that the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled against
@@ -348,7 +374,7 @@ def extras_cpu(oracle, synth, scene, ws):
     return out
 
 
-def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=True):
+def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=True, window_ordered=False):
     """Swin3D-L encoder forward, fp16 attention (fp16_mode 2 under autocast),
     random-init weights, a batch of two synthetic rooms of ~300k voxels each; attention, window
     index and KNN on the HIP kernels, the dense layers on torch/hipBLASLt."""
@@ -359,7 +385,8 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     vox = encoder.SparseVoxels(torch.from_numpy(scene.coords).to(dev), torch.from_numpy(feats).to(dev), 1)
     sig = torch.from_numpy(signals).to(dev)
     torch.manual_seed(0)
-    model = encoder.Swin3DEncoder(**encoder.SWIN3D_L, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=2)
+    model = encoder.Swin3DEncoder(**encoder.SWIN3D_L, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=2,
+                                  window_ordered=window_ordered)
     model = model.to(dev).eval()
     times = []
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
@@ -373,6 +400,7 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     result = {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
               "voxels_per_stage": [int(o.coords.shape[0]) for o in outs],
               "finite": bool(all(torch.isfinite(o.feats).all().item() for o in outs)),
+              "window_ordered": bool(window_ordered),
               "config": "Swin3D-L channels [80,160,320,640,640] heads [10,10,20,40,40] depths [2,4,9,4,4] "
                         "windows [5,7,7,7,7] quant 4 cRSE XYZ_RGB_NORM, batch of 2 rooms"}
     if not unet:

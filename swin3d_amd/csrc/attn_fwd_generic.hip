@@ -260,10 +260,12 @@ inline int device_cus()
     return 256;
 }
 
-// workgroups per CU the register budget is set for (one wavefront of each on every SIMD)
+// workgroups per CU the register budget is set for (one wavefront of each on every SIMD): four at head_dim 8 - the
+// two-head fp16 instance fits 128 registers without spills, and the fourth wavefront per SIMD measured -2 to -3 % -
+// three at head_dim 16
 template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
 {
-    return D > 8 || HP == 2 ? 3 : 4;
+    return D > 8 ? 3 : 4;
 }
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side

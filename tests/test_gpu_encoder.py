@@ -52,6 +52,37 @@ def test_encoder_forward_fp16_runs_on_both_kernels(hip_lib):
         assert (o.coords[:, 1:] % o.stride == 0).all()
 
 
+def test_window_ordered_levels_equal_input_ordered_levels(hip_lib):
+    """The encoder keeps every level's voxels in the order of the level's regular windows (window_ordered): same voxel sets and the same features as with the levels in input / cell order, the regular window
+    index of every level is the identity, and the UNet's logits come back in input order."""
+    from swin3d_amd import build_window_index
+    vox, signals = _inputs()
+    ordered, plain = _small_model(fp16_mode=2), _small_model(fp16_mode=2)     # same seed: same weights
+    ordered.window_ordered, plain.window_ordered = True, False
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        outs_o, outs_p = ordered(vox, signals), plain(vox, signals)
+    torch.cuda.synchronize()
+    assert plain.last_input_order is None
+    assert torch.equal(outs_o[0].coords, vox.coords[ordered.last_input_order])
+    for level, (a, b) in enumerate(zip(outs_o, outs_p)):
+        ka, kb = encoder.pack_coords(a.coords), encoder.pack_coords(b.coords)
+        ia, ib = torch.argsort(ka), torch.argsort(kb)
+        assert torch.equal(ka[ia], kb[ib]), level
+        scale = max(1.0, float(b.feats.abs().max()))
+        assert float((a.feats[ia] - b.feats[ib]).abs().max()) < 2e-3 * scale, level
+        index = build_window_index(a.coords, a.stride, ordered.layers[level].window_size, 0)
+        assert torch.equal(index.n2n.long(), torch.arange(a.coords.shape[0], device="cuda")), level
+        assert not torch.equal(build_window_index(b.coords, b.stride, ordered.layers[level].window_size, 0).n2n.long(),
+                               torch.arange(b.coords.shape[0], device="cuda"))
+    unet_o, unet_p = _small_unet(fp16_mode=2), _small_unet(fp16_mode=2)
+    unet_o.eval(), unet_p.eval()
+    unet_o.window_ordered, unet_p.window_ordered = True, False
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        lo, lp = unet_o(vox, signals), unet_p(vox, signals)
+    assert lo.shape == lp.shape
+    assert float((lo - lp).abs().max()) < 2e-3 * max(1.0, float(lp.abs().max()))
+
+
 def test_knn_downsample_matches_oracle_neighbours(oracle_lib, hip_lib):
     vox, signals = _inputs(target=6000, batches=2)
     torch.manual_seed(1)
