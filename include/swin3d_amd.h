@@ -223,6 +223,19 @@ int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t w
                      int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * The same index by a counting sort over the lattice of windows, for scenes whose windows fit a dense lattice of
+ * at most max(4096, 4 N) cells (capped at 2^24): the bounding box of (batch, wx, wy, wz) over the voxels.  Room-sized
+ * scenes do; the call is then five launches of a few microseconds instead of a sort of all voxels.  Same arguments
+ * and outputs as s3d_window_index (the results are identical, rows of equal coordinates in row order); own
+ * workspace size.  When the lattice is too large, counts[3] has bit 1 (value 2) set and NO output is written: call
+ * s3d_window_index instead.  counts[3] bit 0 (value 1): coordinates out of range, as for s3d_window_index.
+ */
+size_t s3d_window_index_grid_workspace_bytes(int64_t N);
+int s3d_window_index_grid(const int32_t *coords, int64_t N, int32_t stride, int32_t window,
+                          int32_t shift, int32_t *n2n, int32_t *w_w_id, int32_t *w_sizes, int32_t *w2n,
+                          int64_t *counts, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Representative voxel of every cell of a window sort: the member whose signal row is nearest (Euclidean, fp32) to
  * the mean of the cell's signal rows; ties go to the lower row.  With a sort at window = 2 a cell is a coarse voxel
  * of the stride-2 downsample (GridCoordsDown, Swin3D/modules/swin3d_layers.py:179-231, a chain of scatter

@@ -40,6 +40,8 @@ SIGNATURES = {
                      [_i64, _i32, _i32, _i64, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_window_index_workspace_bytes": (ctypes.c_size_t, [_i64]),
     "s3d_window_index": (ctypes.c_int, [_vp, _i64, _i32, _i32, _i32] + [_vp] * 6 + [ctypes.c_size_t, _vp]),
+    "s3d_window_index_grid_workspace_bytes": (ctypes.c_size_t, [_i64]),
+    "s3d_window_index_grid": (ctypes.c_int, [_vp, _i64, _i32, _i32, _i32] + [_vp] * 6 + [ctypes.c_size_t, _vp]),
     "s3d_cell_representatives": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp, _i64, _i32, _vp, _vp]),
     "s3d_key_neighbours": (ctypes.c_int, [_vp, _vp, _i64, _vp, _i32, _vp, _vp]),
     "s3d_window_signals": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, ctypes.c_float, ctypes.c_float, _vp,

@@ -22,6 +22,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kMaxBatch = 4096;
+constexpr int kBboxBlocks = 128;   // workgroups of the bounding-box pass = partial boxes the count pass reduces
 
 struct KnnPlan {
     // bounding box of all sources as order-preserving integer images of the floats
@@ -34,7 +35,7 @@ struct KnnPlan {
 };
 
 struct Layout {
-    size_t plan, counts, starts, src_cell, sorted, temp, temp_bytes, total;
+    size_t plan, partials, counts, starts, src_place, sorted, temp, temp_bytes, total;
     int64_t cells_cap;
 };
 
@@ -68,9 +69,10 @@ Layout make_layout(int64_t Ns)
         return at;
     };
     L.plan = take(sizeof(KnnPlan));
+    L.partials = take(sizeof(int32_t) * 6 * kBboxBlocks);
     L.counts = take(cells * sizeof(int32_t));
     L.starts = take(cells * sizeof(int32_t));
-    L.src_cell = take(ns * sizeof(int32_t));
+    L.src_place = take(ns * sizeof(int2));
     L.sorted = take(ns * sizeof(float4));
     L.temp_bytes = scan_temp_bytes(static_cast<int64_t>(cells));
     L.temp = take(L.temp_bytes);
@@ -89,24 +91,15 @@ __device__ __forceinline__ float ordered_to_float(int i)
     return __int_as_float(i >= 0 ? i : i ^ 0x7fffffff);
 }
 
-__global__ __launch_bounds__(kThreads) void knn_init_kernel(KnnPlan *plan, int32_t *counts,
-                                                            int64_t cells)
+// Bounding box of the sources, one partial box per workgroup (no atomics, nothing to initialise), and the cell
+// counters set to zero: a small grid-stride grid.
+__global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restrict__ src, int64_t Ns,
+                                                            int32_t *__restrict__ partials,
+                                                            int32_t *__restrict__ counts, int64_t cells)
 {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-    if (i < cells) counts[i] = 0;
-    if (i < 3) {
-        plan->lo[i] = 0x7fffffff;
-        plan->hi[i] = static_cast<int>(0x80000000u);
-    }
-}
-
-// Bounding box of the sources: a small grid-stride grid so that only a few hundred atomics
-// meet on the six box words (one atomic pair per wavefront and axis).
-constexpr int kBboxBlocks = 128;
-
-__global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restrict__ src,
-                                                            int64_t Ns, KnnPlan *plan)
-{
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < cells;
+         i += static_cast<int64_t>(gridDim.x) * kThreads)
+        counts[i] = 0;
     int lo[3] = {0x7fffffff, 0x7fffffff, 0x7fffffff};
     int hi[3] = {static_cast<int>(0x80000000u), static_cast<int>(0x80000000u),
                  static_cast<int>(0x80000000u)};
@@ -126,7 +119,6 @@ __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restr
             hi[a] = max(hi[a], __shfl_down(hi[a], off));
         }
     }
-    // one set of global atomics per workgroup: they all land on the same six words and serialise
     __shared__ int part[kThreads / 64][6];
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
@@ -140,16 +132,14 @@ __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restr
         int v = part[0][threadIdx.x];
         for (int w = 1; w < kThreads / 64; ++w)
             v = threadIdx.x < 3 ? min(v, part[w][threadIdx.x]) : max(v, part[w][threadIdx.x]);
-        if (threadIdx.x < 3) atomicMin(&plan->lo[threadIdx.x], v);
-        else atomicMax(&plan->hi[threadIdx.x - 3], v);
+        partials[blockIdx.x * 6 + threadIdx.x] = v;
     }
 }
 
-// One thread: turn the bounding box into grid parameters that fit `cells_cap`.
-__global__ void knn_plan_kernel(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B,
-                                int64_t Ns, float cell_hint, int64_t cells_cap)
+// One thread: turn the bounding box (plan->lo / hi) into grid parameters that fit `cells_cap`.
+__device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B, int64_t Ns, float cell_hint,
+                          int64_t cells_cap)
 {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
     int src_end = src_offset[B - 1];
     if (src_end > Ns) src_end = static_cast<int>(Ns);
     if (src_end < 0) src_end = 0;
@@ -207,6 +197,14 @@ __global__ void knn_plan_kernel(KnnPlan *plan, const int32_t *__restrict__ src_o
     plan->cells_per_batch = dim[0] * dim[1] * dim[2];
 }
 
+// the plan of a call without sources (the query kernel pads every slot)
+__global__ void knn_plan_kernel(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B,
+                                int64_t Ns, float cell_hint, int64_t cells_cap)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    make_plan(plan, src_offset, B, Ns, cell_hint, cells_cap);
+}
+
 __device__ __forceinline__ int cell_coord(float p, float origin, float inv_cell)
 {
     const float t = floorf((p - origin) * inv_cell);
@@ -222,40 +220,85 @@ __device__ __forceinline__ int find_batch(const int32_t *__restrict__ offset, in
     return b;  // == B: beyond the last segment
 }
 
+// Every workgroup first reduces the partial boxes and derives the grid from them (the same arithmetic in every
+// workgroup; workgroup 0 leaves the plan for the kernels that follow), then its sources take their places: a
+// source's cell and its slot there, drawn from the cell's counter.  Neighbouring lanes that fall into the same
+// cell (sources usually arrive in lattice order) draw one run of slots with one atomic.
 __global__ __launch_bounds__(kThreads) void knn_count_kernel(
     const float *__restrict__ src, int64_t Ns, const int32_t *__restrict__ src_offset, int B,
-    const KnnPlan *__restrict__ plan, int32_t *__restrict__ counts, int32_t *__restrict__ src_cell)
+    const int32_t *__restrict__ partials, int boxes, float cell_hint, int64_t cells_cap, KnnPlan *__restrict__ plan_out,
+    int32_t *__restrict__ counts, int2 *__restrict__ src_place)
 {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
-    if (i >= Ns) return;
-    const int b = find_batch(src_offset, B, i);
-    if (b >= B) {
-        src_cell[i] = -1;
-        return;
-    }
-    int c[3];
+    __shared__ KnnPlan plan;
+    __shared__ int part[kThreads / 64][6];
+    {
+        int v[6];
 #pragma unroll
-    for (int a = 0; a < 3; ++a) {
-        c[a] = cell_coord(src[i * 3 + a], plan->origin[a], plan->inv_cell);
-        c[a] = min(max(c[a], 0), plan->dim[a] - 1);
+        for (int a = 0; a < 6; ++a) v[a] = a < 3 ? 0x7fffffff : static_cast<int>(0x80000000u);
+        for (int t = threadIdx.x; t < boxes; t += kThreads)
+#pragma unroll
+            for (int a = 0; a < 6; ++a) v[a] = a < 3 ? min(v[a], partials[t * 6 + a]) : max(v[a], partials[t * 6 + a]);
+#pragma unroll
+        for (int a = 0; a < 6; ++a)
+            for (int off = 32; off > 0; off >>= 1) {
+                const int o = __shfl_down(v[a], off);
+                v[a] = a < 3 ? min(v[a], o) : max(v[a], o);
+            }
+        if ((threadIdx.x & 63) == 0)
+#pragma unroll
+            for (int a = 0; a < 6; ++a) part[threadIdx.x >> 6][a] = v[a];
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int a = 0; a < 6; ++a) {
+                int r = part[0][a];
+                for (int w = 1; w < kThreads / 64; ++w) r = a < 3 ? min(r, part[w][a]) : max(r, part[w][a]);
+                if (a < 3) plan.lo[a] = r; else plan.hi[a - 3] = r;
+            }
+            make_plan(&plan, src_offset, B, Ns, cell_hint, cells_cap);
+            if (blockIdx.x == 0) *plan_out = plan;
+        }
+        __syncthreads();
     }
-    const int cell = b * plan->cells_per_batch + (c[2] * plan->dim[1] + c[1]) * plan->dim[0] + c[0];
-    src_cell[i] = cell;
-    atomicAdd(&counts[cell], 1);
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    int cell = -2;                       // beyond the array
+    if (i < Ns) {
+        const int b = find_batch(src_offset, B, i);
+        cell = -1;                       // in no batch segment
+        if (b < B) {
+            int c[3];
+#pragma unroll
+            for (int a = 0; a < 3; ++a) {
+                c[a] = cell_coord(src[i * 3 + a], plan.origin[a], plan.inv_cell);
+                c[a] = min(max(c[a], 0), plan.dim[a] - 1);
+            }
+            cell = b * plan.cells_per_batch + (c[2] * plan.dim[1] + c[1]) * plan.dim[0] + c[0];
+        }
+    }
+    // runs of equal cells along the lanes: the first lane of a run draws the run's slots
+    const int before = __shfl_up(cell, 1);
+    const bool head = lane == 0 || before != cell;
+    const unsigned long long heads = __ballot(head);
+    const unsigned long long upto = heads & (lane == 63 ? ~0ull : ((2ull << lane) - 1));
+    const int my_head = 63 - __clzll(static_cast<long long>(upto));
+    const unsigned long long above = lane == 63 ? 0ull : heads & ~((2ull << lane) - 1);
+    const int next = above ? __ffsll(static_cast<long long>(above)) - 1 : 64;
+    int base = 0;
+    if (head && cell >= 0) base = atomicAdd(&counts[cell], next - lane);
+    base = __shfl(base, my_head);
+    if (i < Ns) src_place[i] = make_int2(cell, base + (lane - my_head));
 }
 
 __global__ __launch_bounds__(kThreads) void knn_scatter_kernel(
-    const float *__restrict__ src, int64_t Ns, const int32_t *__restrict__ src_cell,
-    const int32_t *__restrict__ starts, int32_t *__restrict__ counts, float4 *__restrict__ sorted)
+    const float *__restrict__ src, int64_t Ns, const int2 *__restrict__ src_place,
+    const int32_t *__restrict__ starts, float4 *__restrict__ sorted)
 {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (i >= Ns) return;
-    const int cell = src_cell[i];
-    if (cell < 0) return;
-    const int slot = atomicSub(&counts[cell], 1) - 1;
-    const int pos = starts[cell] + slot;
-    sorted[pos] = make_float4(src[i * 3], src[i * 3 + 1], src[i * 3 + 2],
-                              __int_as_float(static_cast<int>(i)));
+    const int2 place = src_place[i];
+    if (place.x < 0) return;
+    sorted[starts[place.x] + place.y] = make_float4(src[i * 3], src[i * 3 + 1], src[i * 3 + 2],
+                                                    __int_as_float(static_cast<int>(i)));
 }
 
 // ((dx*dx) + (dy*dy)) + (dz*dz) with d = src - query and every operation rounded to fp32 on
@@ -574,31 +617,24 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
     KnnPlan *plan = reinterpret_cast<KnnPlan *>(base + L.plan);
     int32_t *counts = reinterpret_cast<int32_t *>(base + L.counts);
     int32_t *starts = reinterpret_cast<int32_t *>(base + L.starts);
-    int32_t *src_cell = reinterpret_cast<int32_t *>(base + L.src_cell);
+    int2 *src_place = reinterpret_cast<int2 *>(base + L.src_place);
+    int32_t *partials = reinterpret_cast<int32_t *>(base + L.partials);
     float4 *sorted = reinterpret_cast<float4 *>(base + L.sorted);
     void *temp = base + L.temp;
     size_t temp_bytes = L.temp_bytes;
     const int64_t cells = L.cells_cap + 1;
 
-    hipLaunchKernelGGL(knn_init_kernel, dim3(static_cast<unsigned>(ceil_div(cells, kThreads))),
-                       dim3(kThreads), 0, s, plan, counts, cells);
-    S3D_HIP_CHECK(hipGetLastError());
     if (Ns > 0) {
+        // bounding box + zeroed counters, places (grid derived in every workgroup), scan, scatter
         const dim3 sgrid(static_cast<unsigned>(ceil_div(Ns, kThreads)));
-        const int64_t bbox_blocks = ceil_div(Ns, kThreads) < kBboxBlocks ? ceil_div(Ns, kThreads) : kBboxBlocks;
-        hipLaunchKernelGGL(knn_bbox_kernel, dim3(static_cast<unsigned>(bbox_blocks)), dim3(kThreads), 0, s,
-                           src_xyz, Ns, plan);
+        hipLaunchKernelGGL(knn_bbox_kernel, dim3(kBboxBlocks), dim3(kThreads), 0, s, src_xyz, Ns, partials, counts, cells);
         S3D_HIP_CHECK(hipGetLastError());
-        hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,
-                           cell_size, L.cells_cap);
-        S3D_HIP_CHECK(hipGetLastError());
-        hipLaunchKernelGGL(knn_count_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_offset, B,
-                           plan, counts, src_cell);
+        hipLaunchKernelGGL(knn_count_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_offset, B, partials,
+                           kBboxBlocks, cell_size, L.cells_cap, plan, counts, src_place);
         S3D_HIP_CHECK(hipGetLastError());
         S3D_HIP_CHECK(rocprim::exclusive_scan(temp, temp_bytes, counts, starts, 0,
                                               static_cast<size_t>(cells), rocprim::plus<int32_t>(), s));
-        hipLaunchKernelGGL(knn_scatter_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_cell,
-                           starts, counts, sorted);
+        hipLaunchKernelGGL(knn_scatter_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_place, starts, sorted);
         S3D_HIP_CHECK(hipGetLastError());
     } else {
         hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,

@@ -158,6 +158,286 @@ __global__ __launch_bounds__(kThreads) void segment_size_kernel(const int32_t *_
     }
 }
 
+// ---- grid path: the same index without a sort of all voxels ----------------------------------------------
+// When the windows of a scene fit a dense lattice of at most cells_cap cells (they do for room-sized scenes: the
+// lattice is the bounding box of the window coordinates), a window is a lattice cell and the index is a counting
+// sort: every voxel draws a slot in its cell, a scan over the cells gives every non-empty cell its rank (= window
+// number, ascending (batch, wx, wy, wz) because the cell number is) and its first position, the voxels are placed
+// there, and each window's few voxels are put in (local id, row) order by one wavefront.  Five launches of a few
+// microseconds instead of a block sort and eight merge passes.
+constexpr int kGridBoxes = 128;          // workgroups of the bounding-box pass
+constexpr int kSlotBits = 20;            // a voxel's slot in its cell, below its local id in one word
+constexpr int kBadRange = 1, kNoGrid = 2;   // counts[3]: coordinates out of range / lattice too large for the grid path
+
+struct GridPlan {
+    int lo[4], dim[4];   // batch, wx, wy, wz: lowest value and extent of the lattice
+    int ok;              // the lattice fits
+};
+
+struct GridLayout {
+    size_t plan, partials, cells, scan, place, keys, temp, temp_bytes, total;
+    int64_t cells_cap;
+};
+
+int64_t grid_cells_cap(int64_t N)
+{
+    int64_t cap = 4 * N;
+    if (cap < 4096) cap = 4096;
+    if (cap > (1LL << 24)) cap = 1LL << 24;
+    return cap;
+}
+
+// (non-empty << 32 | voxels) of a cell: one scan yields a cell's window number and its first position
+struct CellWord {
+    __host__ __device__ uint64_t operator()(int32_t count) const
+    {
+        return (count > 0 ? (1ULL << 32) : 0ULL) | static_cast<uint32_t>(count);
+    }
+};
+typedef rocprim::transform_iterator<const int32_t *, CellWord, uint64_t> CellWordIterator;
+
+size_t grid_scan_temp_bytes(int64_t n)
+{
+    size_t bytes = 0;
+    const int32_t *p = nullptr;
+    uint64_t *o = nullptr;
+    (void)rocprim::exclusive_scan(nullptr, bytes, CellWordIterator(p, CellWord()), o, uint64_t(0), static_cast<size_t>(n),
+                                  rocprim::plus<uint64_t>(), hipStream_t(0));
+    return bytes;
+}
+
+GridLayout make_grid_layout(int64_t N)
+{
+    GridLayout L{};
+    L.cells_cap = grid_cells_cap(N);
+    const size_t n = static_cast<size_t>(N > 0 ? N : 1), cells = static_cast<size_t>(L.cells_cap) + 1;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 256);
+        return at;
+    };
+    L.plan = take(sizeof(GridPlan));
+    L.partials = take(sizeof(int32_t) * 9 * kGridBoxes);
+    L.cells = take(cells * sizeof(int32_t));
+    L.scan = take(cells * sizeof(uint64_t));
+    L.place = take(n * sizeof(int2));
+    L.keys = take(n * sizeof(uint64_t));
+    L.temp_bytes = grid_scan_temp_bytes(static_cast<int64_t>(cells));
+    L.temp = take(L.temp_bytes);
+    L.total = off;
+    return L;
+}
+
+// window coordinates and local id of a voxel; false when they are outside the supported range
+__device__ __forceinline__ bool window_of(const int4 c, int stride, int window, int shift, int *w, int *local)
+{
+    const int span = window * stride;
+    const int cc[3] = {c.y + shift * stride, c.z + shift * stride, c.w + shift * stride};
+    int lv[3];
+    bool bad = c.x < 0 || c.x >= (1 << kBatchBits);
+    w[0] = min(max(c.x, 0), (1 << kBatchBits) - 1);
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+        const int wv = floordiv(cc[a], span);
+        lv[a] = (cc[a] - wv * span) / stride;
+        bad = bad || wv < -kAxisBias || wv >= kAxisBias;
+        w[1 + a] = min(max(wv, -kAxisBias), kAxisBias - 1);
+    }
+    *local = (lv[0] * window + lv[1]) * window + lv[2];
+    return !bad;
+}
+
+// partial bounding boxes of the window coordinates (one per workgroup, no atomics) and the cell counters at zero
+__global__ __launch_bounds__(kThreads) void grid_bbox_kernel(const int32_t *__restrict__ coords, int64_t N, int stride,
+                                                             int window, int shift, int32_t *__restrict__ partials,
+                                                             int32_t *__restrict__ cells, int64_t num_cells)
+{
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < num_cells;
+         i += static_cast<int64_t>(gridDim.x) * kThreads)
+        cells[i] = 0;
+    int lo[4], hi[4], bad = 0;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) { lo[a] = 0x7fffffff; hi[a] = static_cast<int>(0x80000000u); }
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < N;
+         i += static_cast<int64_t>(gridDim.x) * kThreads) {
+        int w[4], local;
+        if (!window_of(reinterpret_cast<const int4 *>(coords)[i], stride, window, shift, w, &local)) bad = 1;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) { lo[a] = min(lo[a], w[a]); hi[a] = max(hi[a], w[a]); }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            lo[a] = min(lo[a], __shfl_down(lo[a], off));
+            hi[a] = max(hi[a], __shfl_down(hi[a], off));
+        }
+        bad |= __shfl_down(bad, off);
+    }
+    __shared__ int part[kThreads / 64][9];
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) { part[threadIdx.x >> 6][a] = lo[a]; part[threadIdx.x >> 6][4 + a] = hi[a]; }
+        part[threadIdx.x >> 6][8] = bad;
+    }
+    __syncthreads();
+    if (threadIdx.x < 9) {
+        int v = part[0][threadIdx.x];
+        for (int wv = 1; wv < kThreads / 64; ++wv)
+            v = threadIdx.x < 4 ? min(v, part[wv][threadIdx.x]) : max(v, part[wv][threadIdx.x]);   // the flag: max = or
+        partials[blockIdx.x * 9 + threadIdx.x] = v;
+    }
+}
+
+// Every workgroup reduces the partial boxes to the lattice (workgroup 0 records it, the status word and zeroed
+// totals); then every voxel draws a slot in its cell - neighbouring lanes of one cell with one atomic.
+__global__ __launch_bounds__(kThreads) void grid_count_kernel(
+    const int32_t *__restrict__ coords, int64_t N, int stride, int window, int shift,
+    const int32_t *__restrict__ partials, int64_t cells_cap, GridPlan *__restrict__ plan_out,
+    int32_t *__restrict__ cells, int2 *__restrict__ place, int64_t *__restrict__ counts)
+{
+    __shared__ GridPlan plan;
+    __shared__ int part[kThreads / 64][9];
+    {
+        int v[9];
+#pragma unroll
+        for (int a = 0; a < 9; ++a) v[a] = a < 4 ? 0x7fffffff : static_cast<int>(0x80000000u);
+        for (int t = threadIdx.x; t < kGridBoxes; t += kThreads)
+#pragma unroll
+            for (int a = 0; a < 9; ++a) v[a] = a < 4 ? min(v[a], partials[t * 9 + a]) : max(v[a], partials[t * 9 + a]);
+#pragma unroll
+        for (int a = 0; a < 9; ++a)
+            for (int off = 32; off > 0; off >>= 1) {
+                const int o = __shfl_down(v[a], off);
+                v[a] = a < 4 ? min(v[a], o) : max(v[a], o);
+            }
+        if ((threadIdx.x & 63) == 0)
+#pragma unroll
+            for (int a = 0; a < 9; ++a) part[threadIdx.x >> 6][a] = v[a];
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int r[9];
+            for (int a = 0; a < 9; ++a) {
+                r[a] = part[0][a];
+                for (int wv = 1; wv < kThreads / 64; ++wv) r[a] = a < 4 ? min(r[a], part[wv][a]) : max(r[a], part[wv][a]);
+            }
+            double total = 1.0;
+            for (int a = 0; a < 4; ++a) {
+                plan.lo[a] = r[a];
+                plan.dim[a] = r[4 + a] - r[a] + 1;
+                total *= static_cast<double>(plan.dim[a]);
+            }
+            const bool bad = r[8] > 0;
+            plan.ok = !bad && total <= static_cast<double>(cells_cap);
+            if (blockIdx.x == 0) {
+                *plan_out = plan;
+                counts[0] = counts[1] = counts[2] = 0;
+                counts[3] = (bad ? kBadRange : 0) | (plan.ok ? 0 : kNoGrid);
+            }
+        }
+        __syncthreads();
+    }
+    if (!plan.ok) return;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    int cell = -1, local = 0;
+    if (i < N) {
+        int w[4];
+        window_of(reinterpret_cast<const int4 *>(coords)[i], stride, window, shift, w, &local);
+        cell = (((w[0] - plan.lo[0]) * plan.dim[1] + (w[1] - plan.lo[1])) * plan.dim[2] + (w[2] - plan.lo[2])) * plan.dim[3] +
+               (w[3] - plan.lo[3]);
+    }
+    const int before = __shfl_up(cell, 1);
+    const bool head = lane == 0 || before != cell;
+    const unsigned long long heads = __ballot(head);
+    const unsigned long long upto = heads & (lane == 63 ? ~0ull : ((2ull << lane) - 1));
+    const int my_head = 63 - __clzll(static_cast<long long>(upto));
+    const unsigned long long above = lane == 63 ? 0ull : heads & ~((2ull << lane) - 1);
+    const int next = above ? __ffsll(static_cast<long long>(above)) - 1 : 64;
+    int base = 0;
+    if (head && cell >= 0) base = atomicAdd(&cells[cell], next - lane);
+    base = __shfl(base, my_head);
+    if (i < N) {
+        const int slot = base + (lane - my_head);
+        if (slot >= (1 << kSlotBits)) atomicOr(reinterpret_cast<unsigned long long *>(counts + 3), static_cast<unsigned long long>(kNoGrid));
+        place[i] = make_int2(cell, (slot & ((1 << kSlotBits) - 1)) | (local << kSlotBits));
+    }
+}
+
+// every voxel to its window's segment (slot order); the voxel in slot 0 also records the window
+__global__ __launch_bounds__(kThreads) void grid_place_kernel(const int2 *__restrict__ place, int64_t N,
+                                                              const GridPlan *__restrict__ plan,
+                                                              const uint64_t *__restrict__ scan, int64_t cells_cap,
+                                                              uint64_t *__restrict__ keys, int32_t *__restrict__ w2n,
+                                                              int32_t *__restrict__ w_sizes, int64_t *__restrict__ counts)
+{
+    if (!plan->ok) return;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (i == 0) counts[0] = static_cast<int64_t>(scan[cells_cap] >> 32);   // non-empty cells before the end = windows
+    if (i >= N) return;
+    const int2 p = place[i];
+    const uint64_t here = scan[p.x];
+    const int start = static_cast<int>(here & 0xffffffffu), slot = p.y & ((1 << kSlotBits) - 1);
+    keys[start + slot] = (static_cast<uint64_t>(p.y >> kSlotBits) << 32) | static_cast<uint32_t>(i);
+    if (slot == 0) {
+        const int rank = static_cast<int>(here >> 32);
+        w2n[rank] = start;
+        w_sizes[rank] = static_cast<int>(scan[p.x + 1] & 0xffffffffu) - start;
+    }
+}
+
+// One wavefront per window at a time: the window's voxels in (local id, row) order.  The rank of an element is
+// the number of smaller ones, counted against every element of the window (a few dozen to a few hundred voxels).
+// Also the totals: sum of squared sizes and the largest size, one pair of atomics per workgroup.
+__global__ __launch_bounds__(kThreads) void grid_order_kernel(const GridPlan *__restrict__ plan,
+                                                              const uint64_t *__restrict__ keys,
+                                                              const int32_t *__restrict__ w2n,
+                                                              const int32_t *__restrict__ w_sizes,
+                                                              int32_t *__restrict__ n2n, int32_t *__restrict__ w_w_id,
+                                                              int64_t *__restrict__ counts)
+{
+    if (!plan->ok) return;
+    const int lane = threadIdx.x & 63;
+    const int W = static_cast<int>(counts[0]);
+    const int waves = static_cast<int>(gridDim.x) * (kThreads / 64);
+    long long squares = 0, largest = 0;
+    for (int w = static_cast<int>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6); w < W; w += waves) {
+        const int start = w2n[w], n = w_sizes[w];
+        if (lane == 0) {
+            squares += static_cast<long long>(n) * n;
+            largest = max(largest, static_cast<long long>(n));
+        }
+        for (int first = 0; first < n; first += 64) {
+            const int e = first + lane;
+            const uint64_t mine = e < n ? keys[start + e] : ~0ULL;
+            int rank = 0;
+            if (n <= 64) {
+                for (int j = 0; j < n; ++j) {
+                    const uint64_t other = (static_cast<uint64_t>(__builtin_amdgcn_readlane(static_cast<int>(mine >> 32), j)) << 32) |
+                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine), j));
+                    rank += other < mine;
+                }
+            } else {
+                for (int j = 0; j < n; ++j) rank += keys[start + j] < mine;
+            }
+            if (e < n) {
+                n2n[start + rank] = static_cast<int32_t>(mine & 0xffffffffu);
+                w_w_id[start + rank] = static_cast<int32_t>(mine >> 32);
+            }
+        }
+    }
+    __shared__ long long part[kThreads / 64][2];
+    if (lane == 0) { part[threadIdx.x >> 6][0] = squares; part[threadIdx.x >> 6][1] = largest; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int wv = 1; wv < kThreads / 64; ++wv) { squares += part[wv][0]; largest = max(largest, part[wv][1]); }
+        if (largest > 0) {
+            atomicAdd(reinterpret_cast<unsigned long long *>(counts + 1), static_cast<unsigned long long>(squares));
+            atomicMax(reinterpret_cast<unsigned long long *>(counts + 2), static_cast<unsigned long long>(largest));
+        }
+    }
+}
+
 // one thread per (sorted position, column); the add and the multiply stay separate roundings, as in the
 // reference's tensor statement (sum, then scale)
 __global__ __launch_bounds__(kThreads) void window_signals_kernel(
@@ -356,6 +636,66 @@ extern "C" __attribute__((visibility("default"))) int s3d_window_index(const int
     hipLaunchKernelGGL(segment_start_kernel, grid, dim3(kThreads), 0, s, flags, ranks, N, w2n, counts);
     S3D_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(segment_size_kernel, grid, dim3(kThreads), 0, s, w2n, N, w_sizes, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+extern "C" __attribute__((visibility("default"))) size_t s3d_window_index_grid_workspace_bytes(int64_t N)
+{
+    return s3d::make_grid_layout(N).total;
+}
+
+extern "C" __attribute__((visibility("default"))) int s3d_window_index_grid(
+    const int32_t *coords, int64_t N, int32_t stride, int32_t window, int32_t shift, int32_t *n2n, int32_t *w_w_id,
+    int32_t *w_sizes, int32_t *w2n, int64_t *counts, void *workspace, size_t workspace_bytes, void *stream)
+{
+    using namespace s3d;
+    if (N < 0 || N > 0x7fffffffLL)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index_grid: N=%lld out of range", (long long)N);
+    if (stride < 1 || window < 1 || window > 10 || shift < 0 || shift >= window)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index_grid: stride=%d window=%d shift=%d (need stride>=1, "
+                    "1<=window<=10, 0<=shift<window)", stride, window, shift);
+    if (!counts) return fail(S3D_ERR_NULL_POINTER, "s3d_window_index_grid: counts is null");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (N == 0) {
+        hipLaunchKernelGGL(init_counts_kernel, dim3(1), dim3(64), 0, s, counts);
+        S3D_HIP_CHECK(hipGetLastError());
+        return S3D_OK;
+    }
+    if (!coords || !n2n || !w_w_id || !w_sizes || !w2n || !workspace)
+        return fail(S3D_ERR_NULL_POINTER, "s3d_window_index_grid: null device pointer");
+    if (reinterpret_cast<uintptr_t>(coords) % 16 != 0)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_window_index_grid: coords must be 16-byte aligned");
+    const GridLayout L = make_grid_layout(N);
+    if (workspace_bytes < L.total)
+        return fail(S3D_ERR_WORKSPACE, "s3d_window_index_grid: workspace %zu B < required %zu B", workspace_bytes, L.total);
+    char *base = static_cast<char *>(workspace);
+    GridPlan *plan = reinterpret_cast<GridPlan *>(base + L.plan);
+    int32_t *partials = reinterpret_cast<int32_t *>(base + L.partials);
+    int32_t *cells = reinterpret_cast<int32_t *>(base + L.cells);
+    uint64_t *scan = reinterpret_cast<uint64_t *>(base + L.scan);
+    int2 *place = reinterpret_cast<int2 *>(base + L.place);
+    uint64_t *keys = reinterpret_cast<uint64_t *>(base + L.keys);
+    size_t temp_bytes = L.temp_bytes;
+    const int64_t num_cells = L.cells_cap + 1;
+    const dim3 grid(static_cast<unsigned>(ceil_div(N, kThreads)));
+    hipLaunchKernelGGL(grid_bbox_kernel, dim3(kGridBoxes), dim3(kThreads), 0, s, coords, N, stride, window, shift, partials,
+                       cells, num_cells);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(grid_count_kernel, grid, dim3(kThreads), 0, s, coords, N, stride, window, shift, partials,
+                       L.cells_cap, plan, cells, place, counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    S3D_HIP_CHECK(rocprim::exclusive_scan(base + L.temp, temp_bytes, CellWordIterator(cells, CellWord()), scan, uint64_t(0),
+                                          static_cast<size_t>(num_cells), rocprim::plus<uint64_t>(), s));
+    hipLaunchKernelGGL(grid_place_kernel, grid, dim3(kThreads), 0, s, place, N, plan, scan, L.cells_cap, keys, w2n, w_sizes,
+                       counts);
+    S3D_HIP_CHECK(hipGetLastError());
+    // a wavefront takes a few windows in turn; few enough workgroups that their totals (one pair of atomics each)
+    // do not queue up on the two counters
+    int64_t order_blocks = ceil_div(N, 512);
+    order_blocks = order_blocks < 1 ? 1 : (order_blocks > 512 ? 512 : order_blocks);
+    hipLaunchKernelGGL(grid_order_kernel, dim3(static_cast<unsigned>(order_blocks)), dim3(kThreads), 0, s, plan, keys, w2n,
+                       w_sizes, n2n, w_w_id, counts);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }

@@ -13,6 +13,10 @@ import torch
 from . import _lib
 
 
+# s3d_window_index_grid (counting sort over the window lattice) where it applies; False: always the sort of all voxels
+USE_GRID_PATH = True
+
+
 @dataclass
 class WindowIndex:
     n2n: torch.Tensor       # int32 [N]  window-sorted position -> original row
@@ -53,24 +57,37 @@ def build_window_indices(coords, stride, window_size, shifts):
     counts = torch.empty((len(sets), 4), dtype=torch.int64, device=dev)
     lib = _lib.lib()
     outputs = []
+
+    def enqueue(i, window, shift, grid):
+        fn, size_fn = ((lib.s3d_window_index_grid, lib.s3d_window_index_grid_workspace_bytes) if grid else
+                       (lib.s3d_window_index, lib.s3d_window_index_workspace_bytes))
+        ws_bytes = size_fn(n)
+        n2n, wwid, w_sizes, w2n = (torch.empty(n, dtype=torch.int32, device=dev) for _ in range(4))
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        status = fn(coords.data_ptr(), n, int(stride), int(window), int(shift), n2n.data_ptr(), wwid.data_ptr(),
+                    w_sizes.data_ptr(), w2n.data_ptr(), counts[i].data_ptr(), workspace.data_ptr(), ws_bytes,
+                    torch.cuda.current_stream(dev).cuda_stream)
+        _lib.check(status, fn.__name__)
+        return n2n, wwid, w_sizes, w2n
+
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_window_index_workspace_bytes(n)
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        # the counting sort over the window lattice first; a set whose lattice is too large for it (bit 1 of its
+        # status word) is built again by the sort of all voxels, at the price of a second wait
         for i, (window, shift) in enumerate(sets):
-            n2n, wwid, w_sizes, w2n = (torch.empty(n, dtype=torch.int32, device=dev) for _ in range(4))
-            workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            status = lib.s3d_window_index(coords.data_ptr(), n, int(stride), int(window), int(shift),
-                                          n2n.data_ptr(), wwid.data_ptr(), w_sizes.data_ptr(), w2n.data_ptr(),
-                                          counts[i].data_ptr(), workspace.data_ptr(), ws_bytes, stream)
-            _lib.check(status, "s3d_window_index")
-            outputs.append((n2n, wwid, w_sizes, w2n))
+            outputs.append(enqueue(i, window, shift, grid=USE_GRID_PATH))
+        host_counts = counts.tolist()
+        redo = [i for i, c in enumerate(host_counts) if c[3] & 2]
+        if redo:
+            for i in redo:
+                outputs[i] = enqueue(i, sets[i][0], sets[i][1], grid=False)
+            host_counts = counts.tolist()
     result = []
-    for (n2n, wwid, w_sizes, w2n), (num_w, num_m, max_w, err), (window, _) in zip(outputs, counts.tolist(), sets):
-        if err:
+    for (n2n, wwid, w_sizes, w2n), (num_w, num_m, max_w, err), (window, _) in zip(outputs, host_counts, sets):
+        if err & 1:
             raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
                              "-8192..8191)")
         sizes = w_sizes[:num_w]
-        sizes.max_window_voxels = int(max_w)   # read by the attention op (sizes its partial-result workspace)
+        sizes.max_window_voxels = int(max_w)   # read by the attention op (the MFMA kernel sizes its partial results with it)
         result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window)))
     return result
 

@@ -9,6 +9,15 @@ from swin3d_amd import synth
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["grid", "sort"], autouse=True)
+def index_path(request, monkeypatch):
+    """Every test of this file runs on both builders: s3d_window_index_grid (counting sort over the window
+    lattice, the default where it applies) and s3d_window_index (sort of all voxels)."""
+    from swin3d_amd import window_index
+    monkeypatch.setattr(window_index, "USE_GRID_PATH", request.param == "grid")
+    return request.param
+
+
 def _run(coords, stride, ws, shift):
     import swin3d_amd
     index = swin3d_amd.build_window_index(torch.from_numpy(coords).cuda(), stride, ws, shift)
@@ -126,3 +135,27 @@ def test_several_window_sets_in_one_call(oracle_lib, hip_lib):
         np.testing.assert_array_equal(got.n2n.cpu().numpy(), ref["n2n"])
         np.testing.assert_array_equal(got.w_sizes.cpu().numpy(), ref["w_sizes"])
         np.testing.assert_array_equal(got.w2n.cpu().numpy(), ref["w2n"])
+
+
+def test_lattice_too_large_falls_back_to_the_sort(oracle_lib, hip_lib, index_path):
+    """Voxels spread so far apart that the bounding lattice of their windows has more cells than the grid path
+    takes: s3d_window_index_grid reports it (status bit 1, nothing written) and the wrapper builds the set with the
+    sort; the result is the oracle's either way."""
+    import ctypes
+    rng = np.random.default_rng(9)
+    coords = np.concatenate([np.zeros((3000, 1), np.int64), rng.integers(-30000, 30000, size=(3000, 3))], 1).astype(np.int32)
+    coords = np.unique(coords, axis=0)
+    _compare(oracle_lib, coords, 1, 5, 2)
+    if index_path == "grid":
+        n = coords.shape[0]
+        c = torch.from_numpy(coords).cuda()
+        outs = [torch.full((n,), -7, dtype=torch.int32, device="cuda") for _ in range(4)]
+        counts = torch.zeros(4, dtype=torch.int64, device="cuda")
+        ws_bytes = hip_lib.s3d_window_index_grid_workspace_bytes(n)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        status = hip_lib.s3d_window_index_grid(c.data_ptr(), n, 1, 5, 2, *(o.data_ptr() for o in outs), counts.data_ptr(),
+                                               ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream)
+        assert status == 0
+        torch.cuda.synchronize()
+        assert int(counts[3]) & 2
+        assert all(bool((o == -7).all()) for o in outs)
