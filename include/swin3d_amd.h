@@ -224,7 +224,7 @@ int s3d_window_index(const int32_t *coords, int64_t N, int32_t stride, int32_t w
 
 /*
  * The same index by a counting sort over the lattice of windows, for scenes whose windows fit a dense lattice of
- * at most max(4096, 4 N) cells (capped at 2^24): the bounding box of (batch, wx, wy, wz) over the voxels.  Room-sized
+ * at most max(4096, 2 N) cells (capped at 2^24): the bounding box of (batch, wx, wy, wz) over the voxels.  Room-sized
  * scenes do; the call is then five launches of a few microseconds instead of a sort of all voxels.  Same arguments
  * and outputs as s3d_window_index (the results are identical, rows of equal coordinates in row order); own
  * workspace size.  When the lattice is too large, counts[3] has bit 1 (value 2) set and NO output is written: call

@@ -181,7 +181,7 @@ struct GridLayout {
 
 int64_t grid_cells_cap(int64_t N)
 {
-    int64_t cap = 4 * N;
+    int64_t cap = 2 * N;    // the scan over the cells is the longest of the five launches: no more cells than pay
     if (cap < 4096) cap = 4096;
     if (cap > (1LL << 24)) cap = 1LL << 24;
     return cap;
@@ -397,34 +397,69 @@ __global__ __launch_bounds__(kThreads) void grid_order_kernel(const GridPlan *__
                                                               int64_t *__restrict__ counts)
 {
     if (!plan->ok) return;
+    constexpr int kOrderStage = 512;                       // keys of a window staged in LDS at a time, per wavefront
+    constexpr int kTotalGroups = 32;
+    __shared__ uint64_t stage_all[kThreads / 64][kOrderStage];
+    uint64_t *stage = stage_all[threadIdx.x >> 6];
     const int lane = threadIdx.x & 63;
     const int W = static_cast<int>(counts[0]);
     const int waves = static_cast<int>(gridDim.x) * (kThreads / 64);
-    long long squares = 0, largest = 0;
     for (int w = static_cast<int>(blockIdx.x) * (kThreads / 64) + (threadIdx.x >> 6); w < W; w += waves) {
         const int start = w2n[w], n = w_sizes[w];
-        if (lane == 0) {
-            squares += static_cast<long long>(n) * n;
-            largest = max(largest, static_cast<long long>(n));
+        if (n <= 64) {
+            // one element per lane, the others read lane by lane
+            const uint64_t mine = lane < n ? keys[start + lane] : ~0ULL;
+            int rank = 0;
+            for (int j = 0; j < n; ++j) {
+                const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine >> 32), j))) << 32) |
+                                       static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine), j));
+                rank += other < mine;
+            }
+            if (lane < n) {
+                n2n[start + rank] = static_cast<int32_t>(mine & 0xffffffffu);
+                w_w_id[start + rank] = static_cast<int32_t>(mine >> 32);
+            }
+            continue;
         }
+        // larger windows: the keys staged in LDS, every lane ranks its elements against all of them; a window
+        // beyond the staging area (only with many voxels of equal coordinates) is staged piece by piece per chunk
+        auto stage_keys = [&](int base, int m) {
+            __builtin_amdgcn_wave_barrier();
+            for (int t = lane; t < m; t += 64) stage[t] = keys[start + base + t];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+        const bool whole = n <= kOrderStage;
+        if (whole) stage_keys(0, n);
         for (int first = 0; first < n; first += 64) {
             const int e = first + lane;
-            const uint64_t mine = e < n ? keys[start + e] : ~0ULL;
+            const uint64_t mine = e < n ? (whole ? stage[e] : keys[start + e]) : ~0ULL;
             int rank = 0;
-            if (n <= 64) {
-                for (int j = 0; j < n; ++j) {
-                    const uint64_t other = (static_cast<uint64_t>(__builtin_amdgcn_readlane(static_cast<int>(mine >> 32), j)) << 32) |
-                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine), j));
-                    rank += other < mine;
-                }
-            } else {
-                for (int j = 0; j < n; ++j) rank += keys[start + j] < mine;
+            for (int base = 0; base < n; base += kOrderStage) {
+                const int m = min(kOrderStage, n - base);
+                if (!whole) stage_keys(base, m);
+#pragma unroll 4
+                for (int j = 0; j < m; ++j) rank += stage[j] < mine;
             }
             if (e < n) {
                 n2n[start + rank] = static_cast<int32_t>(mine & 0xffffffffu);
                 w_w_id[start + rank] = static_cast<int32_t>(mine >> 32);
             }
         }
+    }
+    // the totals (sum of squared sizes, largest size): the first kTotalGroups workgroups share the windows, one pair
+    // of atomics each
+    if (blockIdx.x >= kTotalGroups) return;
+    long long squares = 0, largest = 0;
+    for (int w = static_cast<int>(blockIdx.x) * kThreads + threadIdx.x; w < W; w += kTotalGroups * kThreads) {
+        const long long n = w_sizes[w];
+        squares += n * n;
+        largest = max(largest, n);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        squares += __shfl_down(squares, off);
+        largest = max(largest, __shfl_down(largest, off));
     }
     __shared__ long long part[kThreads / 64][2];
     if (lane == 0) { part[threadIdx.x >> 6][0] = squares; part[threadIdx.x >> 6][1] = largest; }
@@ -690,10 +725,9 @@ extern "C" __attribute__((visibility("default"))) int s3d_window_index_grid(
     hipLaunchKernelGGL(grid_place_kernel, grid, dim3(kThreads), 0, s, place, N, plan, scan, L.cells_cap, keys, w2n, w_sizes,
                        counts);
     S3D_HIP_CHECK(hipGetLastError());
-    // a wavefront takes a few windows in turn; few enough workgroups that their totals (one pair of atomics each)
-    // do not queue up on the two counters
-    int64_t order_blocks = ceil_div(N, 512);
-    order_blocks = order_blocks < 1 ? 1 : (order_blocks > 512 ? 512 : order_blocks);
+    // about one window per wavefront if the windows hold 16 voxels on average, more in turn otherwise
+    int64_t order_blocks = ceil_div(N, 64);
+    order_blocks = order_blocks < 32 ? 32 : (order_blocks > 4096 ? 4096 : order_blocks);
     hipLaunchKernelGGL(grid_order_kernel, dim3(static_cast<unsigned>(order_blocks)), dim3(kThreads), 0, s, plan, keys, w2n,
                        w_sizes, n2n, w_w_id, counts);
     S3D_HIP_CHECK(hipGetLastError());
