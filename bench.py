@@ -325,7 +325,11 @@ def extras(torch, swin3d_amd, synth, scene, coords_d, ws, dev):
         ns, nq = s.shape[0], q.shape[0]
         alg = 12 * ns + 12 * nq + 8 * k * nq
         out[name] = {"ms": ms, "queries_per_s": nq / (ms * 1e-3), "sources": ns, "queries": nq,
-                     "algorithmic_bytes": alg, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+                     "algorithmic_bytes": alg, "hbm_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     # the candidate distances the reference's kernel evaluates for this call (every source of the
+                     # batch segment for every query, knn_cuda_kernel.cu:174-192) over this call's time; the grid
+                     # search evaluates a few dozen per query
+                     "reference_distance_evals_per_s": float(nq) * float(ns) / (ms * 1e-3)}
     return out
 
 

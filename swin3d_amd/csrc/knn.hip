@@ -137,8 +137,8 @@ __global__ __launch_bounds__(kThreads) void knn_bbox_kernel(const float *__restr
 }
 
 // One thread: turn the bounding box (plan->lo / hi) into grid parameters that fit `cells_cap`.
-__device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B, int64_t Ns, float cell_hint,
-                          int64_t cells_cap)
+__device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B, int64_t Ns, int K,
+                          float cell_hint, int64_t cells_cap)
 {
     int src_end = src_offset[B - 1];
     if (src_end > Ns) src_end = static_cast<int>(Ns);
@@ -162,17 +162,20 @@ __device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset,
         ext[a] = fmaxf(hi - lo, 0.0f);
         max_abs = fmaxf(max_abs, fmaxf(fabsf(lo), fabsf(hi)));
     }
+    const int64_t per_batch_cap = cells_cap / B;  // B <= kMaxBatch <= cells_cap
     float cell = cell_hint;
     if (!(cell > 0.0f)) {
-        // no hint: aim at about one source per cell if the sources filled the box
+        // no hint: about K / 16 sources per cell if the sources filled their box (a query wants its K-th neighbour
+        // inside the first shell of cells; scans of surfaces fill a small part of the box, so the cells hold fewer),
+        // and never more cells than the cell array has
         const float floor_ext = fmaxf(fmaxf(ext[0], ext[1]), ext[2]) * 1e-3f + 1e-12f;
         const float vol = fmaxf(ext[0], floor_ext) * fmaxf(ext[1], floor_ext) * fmaxf(ext[2], floor_ext);
-        cell = cbrtf(vol / static_cast<float>(src_end > 0 ? src_end : 1));
+        cell = cbrtf(vol / static_cast<float>(src_end > 0 ? src_end : 1) * static_cast<float>(K) * (1.0f / 16.0f));
+        cell = fmaxf(cell, cbrtf(vol / static_cast<float>(per_batch_cap > 0 ? per_batch_cap : 1)));
     }
     if (!(cell > 1e-20f)) cell = 1.0f;
-    const int64_t per_batch_cap = cells_cap / B;  // B <= kMaxBatch <= cells_cap
     int dim[3];
-    for (int iter = 0; iter < 200; ++iter) {
+    for (int iter = 0; iter < 400; ++iter) {
         double total = 1.0;
         for (int a = 0; a < 3; ++a) {
             const float cells_f = floorf(ext[a] / cell) + 1.0f;
@@ -180,7 +183,7 @@ __device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset,
             total *= static_cast<double>(dim[a]);
         }
         if (total <= static_cast<double>(per_batch_cap)) break;
-        cell *= 1.25f;
+        cell *= iter < 40 ? 1.03f : 1.25f;
     }
     {
         double total = static_cast<double>(dim[0]) * dim[1] * dim[2];
@@ -199,10 +202,10 @@ __device__ void make_plan(KnnPlan *plan, const int32_t *__restrict__ src_offset,
 
 // the plan of a call without sources (the query kernel pads every slot)
 __global__ void knn_plan_kernel(KnnPlan *plan, const int32_t *__restrict__ src_offset, int B,
-                                int64_t Ns, float cell_hint, int64_t cells_cap)
+                                int64_t Ns, int K, float cell_hint, int64_t cells_cap)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    make_plan(plan, src_offset, B, Ns, cell_hint, cells_cap);
+    make_plan(plan, src_offset, B, Ns, K, cell_hint, cells_cap);
 }
 
 __device__ __forceinline__ int cell_coord(float p, float origin, float inv_cell)
@@ -226,7 +229,8 @@ __device__ __forceinline__ int find_batch(const int32_t *__restrict__ offset, in
 // cell (sources usually arrive in lattice order) draw one run of slots with one atomic.
 __global__ __launch_bounds__(kThreads) void knn_count_kernel(
     const float *__restrict__ src, int64_t Ns, const int32_t *__restrict__ src_offset, int B,
-    const int32_t *__restrict__ partials, int boxes, float cell_hint, int64_t cells_cap, KnnPlan *__restrict__ plan_out,
+    const int32_t *__restrict__ partials, int boxes, int K, float cell_hint, int64_t cells_cap,
+    KnnPlan *__restrict__ plan_out,
     int32_t *__restrict__ counts, int2 *__restrict__ src_place)
 {
     __shared__ KnnPlan plan;
@@ -254,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void knn_count_kernel(
                 for (int w = 1; w < kThreads / 64; ++w) r = a < 3 ? min(r, part[w][a]) : max(r, part[w][a]);
                 if (a < 3) plan.lo[a] = r; else plan.hi[a - 3] = r;
             }
-            make_plan(&plan, src_offset, B, Ns, cell_hint, cells_cap);
+            make_plan(&plan, src_offset, B, Ns, K, cell_hint, cells_cap);
             if (blockIdx.x == 0) *plan_out = plan;
         }
         __syncthreads();
@@ -630,14 +634,14 @@ extern "C" __attribute__((visibility("default"))) int s3d_knn(int32_t K, const f
         hipLaunchKernelGGL(knn_bbox_kernel, dim3(kBboxBlocks), dim3(kThreads), 0, s, src_xyz, Ns, partials, counts, cells);
         S3D_HIP_CHECK(hipGetLastError());
         hipLaunchKernelGGL(knn_count_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_offset, B, partials,
-                           kBboxBlocks, cell_size, L.cells_cap, plan, counts, src_place);
+                           kBboxBlocks, K, cell_size, L.cells_cap, plan, counts, src_place);
         S3D_HIP_CHECK(hipGetLastError());
         S3D_HIP_CHECK(rocprim::exclusive_scan(temp, temp_bytes, counts, starts, 0,
                                               static_cast<size_t>(cells), rocprim::plus<int32_t>(), s));
         hipLaunchKernelGGL(knn_scatter_kernel, sgrid, dim3(kThreads), 0, s, src_xyz, Ns, src_place, starts, sorted);
         S3D_HIP_CHECK(hipGetLastError());
     } else {
-        hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns,
+        hipLaunchKernelGGL(knn_plan_kernel, dim3(1), dim3(64), 0, s, plan, src_offset, B, Ns, K,
                            cell_size, L.cells_cap);
         S3D_HIP_CHECK(hipGetLastError());
     }
