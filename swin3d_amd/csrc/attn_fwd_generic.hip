@@ -24,7 +24,6 @@ namespace {
 
 using namespace sweep;
 
-constexpr int kThreads = 256;
 constexpr int kChunk = 64;   // lanes of a wavefront = lanes of a unit
 constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
 constexpr float kSlack = 10.0f;   // how far a logit may exceed the softmax reference exponent before it moves
@@ -260,12 +259,20 @@ inline int device_cus()
     return 256;
 }
 
-// workgroups per CU the register budget is set for (one wavefront of each on every SIMD): four at head_dim 8 - the
+// workgroups per CU the register budget is set for: four at head_dim 8 (one wavefront of each on every SIMD) - the
 // two-head fp16 instance fits 128 registers without spills, and the fourth wavefront per SIMD measured -2 to -3 % -
-// three at head_dim 16
+// three at head_dim 16 with one head per wavefront, one (of twelve wavefronts) with two heads
 template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
 {
-    return D > 8 ? 3 : 4;
+    return D > 8 ? (HP == 2 ? 1 : 3) : 4;
+}
+
+// threads of a workgroup: four wavefronts, or twelve where one workgroup has the CU to itself (head_dim 16 with two
+// heads per wavefront: 75 KB of tables), which keeps three wavefronts on every SIMD (two workgroups of six wavefronts
+// measured 25 % slower than one of twelve)
+template <typename T, int D, int HP> __host__ __device__ constexpr int group_threads()
+{
+    return D > 8 && HP == 2 ? 768 : 256;
 }
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
@@ -278,11 +285,12 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int table_row
 // LDS addresses of a pair do not depend on the head, so two heads share that part of the work.
 // kSorted: q, k, v and out rows are in window-sorted order already (no n2n).
 template <typename T, int D, int ND, int HP, bool kSorted>
-__global__ __launch_bounds__(kThreads, (groups_per_cu<T, D, HP>())) void attn_fwd_sweep_kernel(AttnArgs a)
+__global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, HP>())) void attn_fwd_sweep_kernel(AttnArgs a)
 {
-    // streamed keys per loop iteration: at head_dim 16 two interleaved chains hide the LDS round trips,
-    // at head_dim 8 the extra registers cost more than they bring
-    constexpr int kKeys = D <= 8 ? 1 : 2;
+    constexpr int kThreads = group_threads<T, D, HP>();
+    // streamed keys per loop iteration: at head_dim 16 with one head two interleaved chains hide the LDS round trips;
+    // with two heads the heads are the two chains
+    constexpr int kKeys = D <= 8 || HP == 2 ? 1 : 2;
     // lazy softmax reference (see the loop): -4 % for fp16; fp32 measured no gain (head_dim 8) or a loss (16)
     constexpr bool kLazy = sizeof(T) == 2;
     // 16-byte aligned like the table rows behind it, which are read 16 bytes at a time
@@ -597,6 +605,7 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
     const int cus = device_cus();
     const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
     AttnArgs b = a;
+    constexpr int kThreads = group_threads<T, D, HP>();
     b.target_items = sets * kQueues * (kThreads / 64);   // wavefronts that serve one head group
     b.block_shift = target_shift_for(a.N, a.W, b.target_items);
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
@@ -613,12 +622,31 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
     return S3D_OK;
 }
 
+// share of the chip's wavefront slots a launch with HP heads per wavefront fills: workgroups come in whole sets of
+// (XCDs x head groups), so that every XCD serves every head group
+template <typename T, int D, int HP> double sweep_coverage(int H, int cus)
+{
+    const int per_cu = groups_per_cu<T, D, HP>();
+    const int set = kQueues * (H / HP);
+    const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
+    return static_cast<double>(sets) * set / (static_cast<double>(per_cu) * cus);
+}
+
 template <typename T, int D, int ND>
 int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
 {
-    // two heads per wavefront where the registers allow it (head_dim 8, fp16) and the heads pair up
-    if constexpr (D <= 8 && sizeof(T) == 2) {
-        if (a.H % 2 == 0)
+    // Two heads per wavefront where the registers allow it (fp16) and the heads pair up: the cRSE rows and LDS
+    // addresses of a pair are spent once for both.  At head_dim 16 that means one workgroup of twelve wavefronts per
+    // CU (75 KB of tables), so the sets of workgroups are coarser: taken when it fills nearly as much of the chip as
+    // one head per wavefront does (it measured -10 % at 6 heads with 240 of 256 CUs in use; at 24 and 40 heads a
+    // single or two sets would leave a quarter or more of the CUs idle).
+    if constexpr (sizeof(T) == 2) {
+        bool pair = a.H % 2 == 0;
+        if constexpr (D > 8) {
+            const int cus = device_cus();
+            pair = pair && sweep_coverage<T, D, 2>(a.H, cus) >= 0.9 * sweep_coverage<T, D, 1>(a.H, cus);
+        }
+        if (pair)
             return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
                          : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
     }
