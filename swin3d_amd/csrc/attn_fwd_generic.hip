@@ -301,7 +301,8 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
     const int H = a.H;
     const int HD = H * D;
     // workgroups go to the XCDs in turn: consecutive runs of eight serve one head group, so every XCD gets every head
-    const int hg = (blockIdx.x / kQueues) % (H / HP);
+    // (or, with many head groups, the head groups take the workgroups in turn: see the launch)
+    const int hg = a.spread_groups ? blockIdx.x % (H / HP) : (blockIdx.x / kQueues) % (H / HP);
     const int h = hg * HP;   // first head of the group
     // table slices of the heads in the I/O type, interleaved per row: [head][q-side | k-side | v-side]
     constexpr int kRowStride = table_row_stride_heads<T, D, HP>();
@@ -597,16 +598,23 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
     auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP, kSorted>;
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    // a workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow,
-    // in whole sets of (XCDs x head groups)
+    // A workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow.
+    // They come in whole sets of (XCDs x head groups) - runs of eight consecutive workgroups, one per XCD, serve one
+    // head group, so every XCD serves every head group and the rows of a unit reach one L2 - unless whole sets
+    // would leave more than a tenth of the slots empty (many head groups): then the head groups take the workgroups
+    // in turn and every slot is used, at the price of that locality (the kernel is not bound by memory traffic).
     int per_cu = groups_per_cu<T, D, HP>();
     while (per_cu > 1 && per_cu * lds > 160 * 1024) --per_cu;
-    const int set = kQueues * (a.H / HP);
+    const int groups = a.H / HP;
     const int cus = device_cus();
-    const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
+    const int slots = per_cu * cus;
+    const int set = kQueues * groups;
+    const int whole = (slots / set) * set;
     AttnArgs b = a;
+    b.spread_groups = 10 * whole < 9 * slots;
+    const int grid = b.spread_groups ? (slots >= groups ? slots / groups * groups : groups) : whole;
     constexpr int kThreads = group_threads<T, D, HP>();
-    b.target_items = sets * kQueues * (kThreads / 64);   // wavefronts that serve one head group
+    b.target_items = grid / groups * (kThreads / 64);   // wavefronts that serve one head group
     b.block_shift = target_shift_for(a.N, a.W, b.target_items);
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
     const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
@@ -616,20 +624,10 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
         S3D_HIP_CHECK(hipGetLastError());
     }
     if (what & 2) {
-        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(sets * set)), dim3(kThreads), lds, stream, b);
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, stream, b);
         S3D_HIP_CHECK(hipGetLastError());
     }
     return S3D_OK;
-}
-
-// share of the chip's wavefront slots a launch with HP heads per wavefront fills: workgroups come in whole sets of
-// (XCDs x head groups), so that every XCD serves every head group
-template <typename T, int D, int HP> double sweep_coverage(int H, int cus)
-{
-    const int per_cu = groups_per_cu<T, D, HP>();
-    const int set = kQueues * (H / HP);
-    const int sets = per_cu * cus / set > 0 ? per_cu * cus / set : 1;
-    return static_cast<double>(sets) * set / (static_cast<double>(per_cu) * cus);
 }
 
 template <typename T, int D, int ND>
@@ -637,16 +635,9 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
 {
     // Two heads per wavefront where the registers allow it (fp16) and the heads pair up: the cRSE rows and LDS
     // addresses of a pair are spent once for both.  At head_dim 16 that means one workgroup of twelve wavefronts per
-    // CU (75 KB of tables), so the sets of workgroups are coarser: taken when it fills nearly as much of the chip as
-    // one head per wavefront does (it measured -10 % at 6 heads with 240 of 256 CUs in use; at 24 and 40 heads a
-    // single or two sets would leave a quarter or more of the CUs idle).
+    // CU (75 KB of tables): it measured -10 % at 6 heads.
     if constexpr (sizeof(T) == 2) {
-        bool pair = a.H % 2 == 0;
-        if constexpr (D > 8) {
-            const int cus = device_cus();
-            pair = pair && sweep_coverage<T, D, 2>(a.H, cus) >= 0.9 * sweep_coverage<T, D, 1>(a.H, cus);
-        }
-        if (pair)
+        if (a.H % 2 == 0)
             return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
                          : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
     }

@@ -22,6 +22,7 @@ struct AttnArgs {
     int32_t max_key_tiles;                 // MFMA path: key tiles of the largest window (stride of `partials`)
     int32_t block_shift;                   // sweep kernel: the step target, a lane streams about 2^block_shift keys
     int32_t target_items;                  // work items the launch wants at least (heads are split to reach it)
+    int32_t spread_groups;                 // sweep kernel: head groups take the workgroups in turn (else in runs of eight)
     int32_t H, D, nd, total_rows;
     int64_t N, W;
     int32_t rows[kMaxAxes];                // rows of each axis table
@@ -41,16 +42,16 @@ int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int wh
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
-// the shapes where it is the faster of the two kernels: head_dim 16 with nearly full windows (256 voxels on
-// average; measured at window 7 with 6 heads: 343-voxel windows 0.88 ms against 0.99 ms, 205 voxels 0.435 against
-// 0.424, 104 voxels 0.165 against 0.145, a room scan with 57 voxels on average 0.43 against 0.35), or with many
-// heads, over which it spreads the row indices of a tile pair, and 60 voxels on average (Swin3D-L, window 7: 20
-// heads and 61 voxels 0.885 against 0.919 ms, 55 voxels 0.853 against 0.718; 40 heads and 69 voxels 0.571 against
-// 0.700, 45 voxels 0.463 against 0.429; 10 heads and 58 voxels 1.57 against 1.37).  At head_dim 8 the sweep
-// kernel's packed fp16 dot products win everywhere.
+// the shapes where it is the faster of the two kernels: head_dim 16 with nearly full windows, 240 voxels or more on
+// average.  Measured at window 7 on a 56 x 56 x 28 lattice filled to 100 / 80 / 60 / 30 % (343 / 274 / 206 / 103
+// voxels per window), sweep against MFMA kernel in ms: 6 heads 2.12 / 1.97, 1.46 / 1.35, 0.90 / 0.83, 0.29 / 0.31;
+// 20 heads 6.92 / 6.18, 4.62 / 4.24, 2.53 / 2.60, 0.80 / 0.86; 40 heads 13.99 / 12.19, 9.21 / 8.39, 5.10 / 5.11,
+// 1.40 / 1.66.  Room scans (50 to 70 voxels per window at every stage of the encoder) are the sweep kernel's: the
+// Swin3D-L encoder takes 28.6 ms on it alone against 29.6 ms with the MFMA kernel on the many-head blocks.  At
+// head_dim 8 the sweep kernel's packed fp16 dot products win everywhere.
 inline bool attn_mfma_preferred(const AttnArgs &a)
 {
-    return a.D > 8 && (a.N >= 256 * a.W || (a.H >= 16 && a.N >= 60 * a.W));
+    return a.D > 8 && a.N >= 240 * a.W;
 }
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
 size_t attn_mfma_items_bytes(int64_t W);
