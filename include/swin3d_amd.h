@@ -66,6 +66,11 @@ const char *s3d_last_error_string(void);
  *   table_sizes    HOST int32 [nd], table_sizes[n] = rows_n * H * D (the values of the
  *                  reference's `table_offsets` tensor, fwd.cu:258,285; read on the host so
  *                  that the row counts travel as kernel arguments)
+ *                  With the flag S3D_ATTN_SIZES_ON_DEVICE the pointer is a DEVICE int32 [nd] array instead - the
+ *                  tensor the reference's caller builds on every call (Swin3D/modules/swin3d_layers.py:511) - and
+ *                  the host never reads it: the sweep kernel takes the row counts from it (clipped so that no
+ *                  access leaves the head's table; sizes that do not add up to table_len give a wrong result, not
+ *                  a fault).  s3d_attn_plan accepts NULL for table_sizes for such callers.
  *   table_len      elements per table = sum_n table_sizes[n]
  *   w_sizes, w2n   device int32 [W]: voxels per window, exclusive prefix sum
  *   n2n            device int32 [N]: window-sorted position -> original row, or NULL when the rows of q, k,
@@ -109,6 +114,7 @@ const char *s3d_last_error_string(void);
 #define S3D_ATTN_FORCE_GENERIC 1
 #define S3D_ATTN_FORCE_MFMA 2
 #define S3D_ATTN_PLANNED 4   /* `workspace` holds a plan written by s3d_attn_plan: see there */
+#define S3D_ATTN_SIZES_ON_DEVICE 8   /* `table_sizes` is a DEVICE int32 [nd] array (sweep kernel; see s3d_attn_fwd) */
 /* 1 if s3d_attn_fwd with flags 0 runs these shapes on the MFMA kernel (fp16, head_dim 16, every axis
  * table <= 64 rows, and windows of at least 256 voxels on average, N >= 256 W, or 60 with 16 heads or more),
  * 0 if on the VALU sweep kernel.  No counterpart in the reference (it has one kernel). */

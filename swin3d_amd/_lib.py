@@ -15,6 +15,7 @@ KNN_KMAX = 64
 S3D_ATTN_FORCE_GENERIC = 1
 S3D_ATTN_FORCE_MFMA = 2
 S3D_ATTN_PLANNED = 4
+S3D_ATTN_SIZES_ON_DEVICE = 8
 
 _lib = None
 

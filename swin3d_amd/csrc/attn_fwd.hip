@@ -103,7 +103,7 @@ int prepare_attn_args(const char *who, AttnArgs &a, bool *empty, const void *q, 
                       const void *table_q, const void *table_k, const void *table_v, const int32_t *table_sizes,
                       int32_t nd, int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
                       const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N, int32_t H,
-                      int32_t D, int64_t W, int64_t qkv_row_stride, int32_t dtype)
+                      int32_t D, int64_t W, int64_t qkv_row_stride, int32_t dtype, bool sizes_on_device = false)
 {
     *empty = true;
     if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
@@ -119,7 +119,19 @@ int prepare_attn_args(const char *who, AttnArgs &a, bool *empty, const void *q, 
     a.nd = nd;
     a.N = N;
     a.W = W;
-    if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
+    if (sizes_on_device) {
+        // the per-axis sizes stay on the device: the host knows the rows of all axes together and nothing more
+        const int64_t hd = static_cast<int64_t>(H) * D;
+        if (table_len % hd != 0 || table_len / hd < nd)
+            return fail(S3D_ERR_BAD_SHAPE, "%s: table_len = %lld is not a multiple of H*D = %lld with a row per axis", who,
+                        (long long)table_len, (long long)hd);
+        for (int n = 0; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = a.pbase[n] = 0;
+        a.total_rows = static_cast<int32_t>(table_len / hd);
+        a.padded_rows = 0;
+        a.sizes_dev = table_sizes;
+    } else if (int rc = fill_axes(a, table_sizes, nd, table_len)) {
+        return rc;
+    }
     if (N == 0 || W == 0) return S3D_OK;
     if (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n_coords || !out)
         return fail(S3D_ERR_NULL_POINTER, "%s: null device pointer", who);
@@ -181,15 +193,17 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     using namespace s3d;
     AttnArgs a{};
     bool empty = true;
+    const bool sizes_on_device = (flags & S3D_ATTN_SIZES_ON_DEVICE) != 0;
     if (int rc = prepare_attn_args("s3d_attn_fwd", a, &empty, q, k, v, table_q, table_k, table_v, table_sizes, nd,
                                    table_len, w_sizes, w2n, n2n, n_coords, out, out_max, out_sum, N, H, D, W,
-                                   qkv_row_stride, dtype))
+                                   qkv_row_stride, dtype, sizes_on_device))
         return rc;
     if (empty) return S3D_OK;
     a.workspace = workspace;
     hipStream_t s = static_cast<hipStream_t>(stream);
     // the MFMA kernel needs the window bound (it sizes partial results with it) and the row map
-    const bool want_mfma = !(flags & (S3D_ATTN_FORCE_GENERIC | S3D_ATTN_PLANNED)) && max_window_voxels >= 1 && n2n &&
+    const bool want_mfma = !(flags & (S3D_ATTN_FORCE_GENERIC | S3D_ATTN_PLANNED | S3D_ATTN_SIZES_ON_DEVICE)) &&
+                           max_window_voxels >= 1 && n2n &&
                            attn_mfma_supported(a, dtype) && (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
     if (want_mfma) {
         const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
@@ -223,14 +237,20 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_plan(
     if (int rc = check_shape(N, W, H, D, nd, table_len)) return rc;
     if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
         return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_plan: dtype %d (0 = fp32, 1 = fp16)", dtype);
-    if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_plan: table_sizes (host) is null");
     AttnArgs a{};
     a.H = H;
     a.D = D;
     a.nd = nd;
     a.N = N;
     a.W = W;
-    if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
+    if (table_sizes) {
+        if (int rc = fill_axes(a, table_sizes, nd, table_len)) return rc;
+    } else {
+        // the list depends on the tables through their total size only (how many workgroups share a CU)
+        const int64_t hd = static_cast<int64_t>(H) * D;
+        if (table_len % hd != 0) return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_plan: table_len is not a multiple of H*D");
+        a.total_rows = static_cast<int32_t>(table_len / hd);
+    }
     if (N == 0 || W == 0) return S3D_OK;
     if (!w_sizes || !w2n) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_plan: null device pointer");
     const size_t need = attn_generic_workspace_bytes(H, W, N);

@@ -25,7 +25,7 @@ namespace {
 using namespace sweep;
 
 constexpr int kChunk = 64;   // lanes of a wavefront = lanes of a unit
-constexpr int kListThreads = 256, kListGroups = 128;   // the list builder's workgroups: size, and how many at most
+constexpr int kListThreads = 256, kListGroups = 32;   // the list builder's workgroups: size, and how many at most
 constexpr float kSlack = 10.0f;   // how far a logit may exceed the softmax reference exponent before it moves
 // A window of n voxels belongs to class g (0..kMaxSplit): each of its queries is served by 2^g adjacent lanes that
 // take alternate keys, g the smallest value for which a lane streams at most `target` keys (the launch's step
@@ -86,7 +86,7 @@ __host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N)
 }
 __host__ __device__ inline size_t ws_end_offset(int H, int64_t W, int64_t N)
 {
-    return ws_bins_offset(H, W, N) + ws_round(sizeof(unsigned long long) * kListGroups * kBins);
+    return ws_bins_offset(H, W, N) + ws_round(sizeof(unsigned long long) * kListGroups * (kListThreads / 64) * kBins);
 }
 
 // How the queries of class 0 (sorted by steps, longest first) are cut into units.  A unit is one pass of a
@@ -121,42 +121,82 @@ __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 // lane of a unit runs (almost) the same number of steps, a query's keys never leave its wavefront (the lanes
 // that share a query merge their softmax states by shuffles), and the launch ends on its shortest units.
 //
-// generic_count_kernel: every workgroup takes a run of windows; a window takes a place in the workgroup's bin
-// of its (class, steps) - its rank there and the queries before it (one 64-bit LDS atomic returns both, so the
-// two orders agree; the order inside a bin does not affect results) - and the workgroup leaves its bin totals.
+// generic_count_kernel: every wavefront takes a run of consecutive windows, 64 at a time.  A window's place in the
+// bin of its (class, steps) - its rank there and the queries before it - follows the window numbers: the lanes
+// of each bin present among the 64 are ranked by their lane numbers on top of the bin's running totals, which
+// the wavefront keeps in registers (lane b % 64 holds bin b), and the wavefront leaves its bin totals.  No
+// atomics: the list, and with it the cut of the queries into units and so every bit of the result, is the same
+// on every run.
 __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
 {
-    __shared__ unsigned long long bin[kBins];   // per bin: windows << 32 | queries
-    for (int t = threadIdx.x; t < kBins; t += kListThreads) bin[t] = 0;
-    __syncthreads();
+    constexpr int kWaves = kListThreads / 64;
+    const int lane = threadIdx.x & 63;
+    const int table = static_cast<int>(blockIdx.x) * kWaves + static_cast<int>(threadIdx.x >> 6);
+    const int tables = static_cast<int>(gridDim.x) * kWaves;
     char *ws = static_cast<char *>(a.workspace);
     int2 *place = reinterpret_cast<int2 *>(ws + ws_place_offset(a.H, a.W, a.N));
     unsigned long long *group_bins = reinterpret_cast<unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N));
     const int W = static_cast<int>(a.W);
-    const int per = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
-    const int begin = min(static_cast<int>(blockIdx.x) * per, W), end = min(begin + per, W);
-    for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
-        const int n = a.w_sizes[w];
+    const int per = (W + tables - 1) / tables;
+    const int begin = min(table * per, W), end = min(begin + per, W);
+    uint32_t held_c[kBins / 64], held_s[kBins / 64];   // bins lane, lane + 64, ...: windows and queries so far
+#pragma unroll
+    for (int j = 0; j < kBins / 64; ++j) held_c[j] = held_s[j] = 0;
+    for (int w0 = begin; w0 < end; w0 += 64) {
+        const int w = w0 + lane;
+        const int n = w < end ? a.w_sizes[w] : 0;
+        const int b = n > 0 ? window_bin(n, window_class(n, a.block_shift)) : -1;
         int2 got = make_int2(-1, 0);
-        if (n > 0) {
-            const unsigned long long before =
-                atomicAdd(&bin[window_bin(n, window_class(n, a.block_shift))], (1ull << 32) | static_cast<unsigned>(n));
-            got = make_int2(static_cast<int>(before >> 32), static_cast<int>(before & 0xffffffffu));
+        unsigned long long todo = __ballot(b >= 0);
+        while (todo != 0) {
+            const int leader = __ffsll(todo) - 1;
+            const int cb = __shfl(b, leader), n_lead = __shfl(n, leader);
+            const bool in = b == cb;
+            const unsigned long long same = __ballot(in);
+            const int below = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(same >> 32),
+                                                        __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(same), 0u));
+            int before_n, all_n;
+            if (__ballot(in && n != n_lead) == 0) {   // the usual case: a bin of class 0 is one window size
+                before_n = below * n_lead;
+                all_n = __popcll(same) * n_lead;
+            } else {
+                int incl = in ? n : 0;
+                for (int off = 1; off < 64; off <<= 1) {
+                    const int up = __shfl_up(incl, off);
+                    if (lane >= off) incl += up;
+                }
+                before_n = incl - (in ? n : 0);
+                all_n = __shfl(incl, 63);
+            }
+            uint32_t c = 0, q = 0;
+#pragma unroll
+            for (int j = 0; j < kBins / 64; ++j)
+                if ((cb >> 6) == j) { c = held_c[j]; q = held_s[j]; }
+            c = __shfl(c, cb & 63);
+            q = __shfl(q, cb & 63);
+            if (in) got = make_int2(static_cast<int>(c) + below, static_cast<int>(q) + before_n);
+#pragma unroll
+            for (int j = 0; j < kBins / 64; ++j)
+                if ((cb >> 6) == j && lane == (cb & 63)) { held_c[j] += __popcll(same); held_s[j] += all_n; }
+            todo &= ~same;
         }
-        place[w] = got;
+        if (w < end) place[w] = got;
     }
-    __syncthreads();
-    for (int t = threadIdx.x; t < kBins; t += kListThreads) group_bins[blockIdx.x * kBins + t] = bin[t];
+#pragma unroll
+    for (int j = 0; j < kBins / 64; ++j)
+        group_bins[static_cast<size_t>(table) * kBins + j * 64 + lane] =
+            (static_cast<unsigned long long>(held_c[j]) << 32) | held_s[j];
 }
 
-// generic_place_kernel (same grid): bins in order, workgroups in order inside a bin.  Writes one entry (first
+// generic_place_kernel (same grid): bins in order, wavefronts in order inside a bin.  Writes one entry (first
 // query of its class, voxels, first sorted position, class) per window in sorted order, one record per unit
 // (the entry that holds its first query, lanes per query as a shift, first query, queries), the totals, and
 // the queue counters at zero.
 __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
 {
-    __shared__ int bin_entry[kBins], bin_slot[kBins];
-    __shared__ int wave_c[kListThreads / 64], wave_s[kListThreads / 64];
+    constexpr int kWaves = kListThreads / 64;
+    __shared__ int bin_entry[kWaves][kBins], bin_slot[kWaves][kBins];
+    __shared__ int wave_c[kWaves], wave_s[kWaves];
     __shared__ int class_base[kClasses + 1];       // queries before each class (index = kMaxSplit - g), and all
     __shared__ int total_entries_s;
     char *ws = static_cast<char *>(a.workspace);
@@ -167,16 +207,18 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
     const int2 *place = reinterpret_cast<const int2 *>(ws + ws_place_offset(a.H, a.W, a.N));
     const unsigned long long *group_bins =
         reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N));
-    // thread t holds bin t: the launch's total, and what the workgroups before this one put there; an exclusive
-    // scan over the threads gives the bins their places (entries over all bins, queries restarting per class)
+    const int tables = static_cast<int>(gridDim.x) * kWaves, first_table = static_cast<int>(blockIdx.x) * kWaves;
+    // thread t holds bin t: the launch's total, and what the wavefronts before this workgroup's put there; an
+    // exclusive scan over the threads gives the bins their places (entries over all bins, queries restarting per
+    // class)
     {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         unsigned long long all = 0, before = 0;
 #pragma unroll 8
-        for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
-            const unsigned long long v = group_bins[g * kBins + threadIdx.x];
+        for (int g = 0; g < tables; ++g) {
+            const unsigned long long v = group_bins[static_cast<size_t>(g) * kBins + threadIdx.x];
             all += v;
-            before += g < static_cast<int>(blockIdx.x) ? v : 0;
+            before += g < first_table ? v : 0;
         }
         const int cnt = static_cast<int>(all >> 32), slots = static_cast<int>(all & 0xffffffffu);
         int incl_c = cnt, incl_s = slots;
@@ -190,8 +232,12 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
         for (int v = 0; v < wave; ++v) { base_c += wave_c[v]; base_s += wave_s[v]; }
         static_assert(kMaxSteps == 64, "a class is the bins of one wavefront of the scan");
         // queries are numbered per class: the class's bins are this wavefront's, so drop the earlier wavefronts' sum
-        bin_entry[threadIdx.x] = base_c + incl_c - cnt + static_cast<int>(before >> 32);
-        bin_slot[threadIdx.x] = incl_s - slots + static_cast<int>(before & 0xffffffffu);
+#pragma unroll
+        for (int v = 0; v < kWaves; ++v) {
+            bin_entry[v][threadIdx.x] = base_c + incl_c - cnt + static_cast<int>(before >> 32);
+            bin_slot[v][threadIdx.x] = incl_s - slots + static_cast<int>(before & 0xffffffffu);
+            before += group_bins[static_cast<size_t>(first_table + v) * kBins + threadIdx.x];
+        }
         if (lane == 0) class_base[wave] = base_s;
         if (threadIdx.x == kListThreads - 1) { class_base[kClasses] = base_s + incl_s; total_entries_s = base_c + incl_c; }
     }
@@ -211,15 +257,16 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
 #pragma unroll
     for (int k = 0; k < 3; ++k) sec_unit[kMaxSplit + k + 1] = sec_unit[kMaxSplit + k] + plan.units[k];
     const int W = static_cast<int>(a.W);
-    const int per_group = (W + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
-    const int begin = min(static_cast<int>(blockIdx.x) * per_group, W), end = min(begin + per_group, W);
-    for (int w = begin + threadIdx.x; w < end; w += kListThreads) {
+    const int my_wave = threadIdx.x >> 6;
+    const int per_wave = (W + tables - 1) / tables;     // the count kernel's runs
+    const int begin = min((first_table + my_wave) * per_wave, W), end = min(begin + per_wave, W);
+    for (int w = begin + (threadIdx.x & 63); w < end; w += 64) {
         const int2 got = place[w];
         if (got.x < 0) continue;
         const int n = a.w_sizes[w];
         const int g = window_class(n, a.block_shift), b = window_bin(n, g);
-        const int e = bin_entry[b] + got.x;
-        const int s = bin_slot[b] + got.y;               // first query of the window inside its class
+        const int e = bin_entry[my_wave][b] + got.x;
+        const int s = bin_slot[my_wave][b] + got.y;      // first query of the window inside its class
         entries[e] = make_int4(s, n, a.w2n[w], g);
         const int s_end = s + n;
         if (g > 0) {
@@ -341,12 +388,24 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
     const uint32_t row_bytes = kRowBytes;
     float half_rows[ND], upper[ND];
     uint32_t base_off[ND];
+    {
+        // rows of every axis table: kernel arguments, or (sizes_dev) read from the caller's device tensor of table
+        // sizes, which the host has not seen - clipped so that every axis keeps a row inside the head's table
+        int run = 0;
 #pragma unroll
-    for (int n = 0; n < ND; ++n) {
-        half_rows[n] = static_cast<float>(a.rows[n] / 2);
-        upper[n] = crse_upper(a.rows[n]);
-        // LDS byte address of the axis table's first row
-        base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + a.base[n] * kRowBytes);
+        for (int n = 0; n < ND; ++n) {
+            int rows = a.rows[n], first = a.base[n];
+            if (a.sizes_dev) {
+                rows = __builtin_amdgcn_readfirstlane(a.sizes_dev[n]) / HD;
+                rows = max(1, min(rows, a.total_rows - run - (ND - 1 - n)));
+                first = run;
+                run += rows;
+            }
+            half_rows[n] = static_cast<float>(rows / 2);
+            upper[n] = crse_upper(rows);
+            // LDS byte address of the axis table's first row
+            base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + first * kRowBytes);
+        }
     }
 
     int queue = xcd_id() % kQueues;
@@ -484,7 +543,7 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
                 }
             } else {
                 // Online softmax against a reference exponent m that follows the running maximum lazily: it moves
-                // (and the sums are rescaled) only when some lane's logit exceeds it by more than kSlack, which
+                // (and the sums are rescaled) only when the lane's logit exceeds it by more than kSlack, which
                 // after the first keys of a unit is rare, so most steps skip the rescaling of l and the D outputs;
                 // weights stay below e^kSlack.  `top` is the true running maximum.
                 float hi[HP];
@@ -499,17 +558,17 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
                     }
                     moved = moved || hi[hh] > m[hh] + kSlack;
                 }
-                if (__builtin_amdgcn_ballot_w64(valid[0] && moved) != 0) {   // uniform: all lanes move their reference
-                    if (valid[0]) {
+                // each lane decides for itself, so the bits of a query's result do not depend on which other queries
+                // share its wavefront
+                if (valid[0] && moved) {
 #pragma unroll
-                        for (int hh = 0; hh < HP; ++hh) {
-                            const float m_new = fmaxf(m[hh], hi[hh]);
-                            const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
-                            l[hh] *= scale;
+                    for (int hh = 0; hh < HP; ++hh) {
+                        const float m_new = fmaxf(m[hh], hi[hh]);
+                        const float scale = __expf(m[hh] - m_new);   // exp(-inf) = 0 on the first key
+                        l[hh] *= scale;
 #pragma unroll
-                            for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
-                            m[hh] = m_new;
-                        }
+                        for (int c = 0; c < D; ++c) acc[hh][c] *= scale;
+                        m[hh] = m_new;
                     }
                 }
                 if (valid[0]) {   // the lowest key of the iteration; lanes whose block has ended sit the step out

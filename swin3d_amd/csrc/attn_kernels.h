@@ -13,6 +13,7 @@ struct AttnArgs {
     int64_t row_stride;
     const void *table_q, *table_k, *table_v;  // flat [sum rows][H][D]
     const int32_t *w_sizes, *w2n, *n2n;
+    const int32_t *sizes_dev;              // sweep kernel: per-axis table sizes on the device (rows[] / base[] unset), or null
     const float *n_coords;                 // [N,nd], window-sorted
     void *out;                             // [N,H,D]
     float *out_max, *out_sum;              // [N,H] or null

@@ -92,11 +92,9 @@ def _as_int32(name, t, device):
 
 
 def _host_table_sizes(table_sizes):
-    """The op reads the per-axis table sizes on the host.  A CUDA tensor costs one synchronising
-    device-to-host copy; the values are then kept on the tensor object (with its version counter), so a
-    module that keeps its table_offsets tensor pays the copy once.  The reference's caller builds a new
-    tensor from a Python list on every call (Swin3D/modules/swin3d_layers.py:511): pass the list, or a CPU
-    tensor, to avoid the copy altogether."""
+    """The per-axis table sizes as a host list (the backward and the MFMA kernel need them there).  A CUDA
+    tensor costs one synchronising device-to-host copy; the values are then kept on the tensor object (with
+    its version counter), so a module that keeps its table_offsets tensor pays the copy once."""
     if isinstance(table_sizes, torch.Tensor):
         if not table_sizes.is_cuda:
             return [int(x) for x in table_sizes.reshape(-1).tolist()]
@@ -111,8 +109,21 @@ def _host_table_sizes(table_sizes):
 # keep the sweep kernel's work list ("plan") on the w_sizes tensor between calls (False: build it in every call)
 REUSE_PLANS = True
 
+# a CUDA table_sizes tensor whose values the host has not seen yet goes to the sweep kernel as it is, and the
+# host never waits for it (False: always copy it to the host, which also lets the MFMA kernel be chosen)
+DEVICE_TABLE_SIZES = True
 
-def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, table_len, n, h, d, code, stream):
+
+def _sizes_stay_on_device(table_sizes):
+    """True for the reference caller's table_offsets (a new CUDA tensor on every call, Swin3D/modules/
+    swin3d_layers.py:511) in a forward that does not need the values on the host."""
+    if not DEVICE_TABLE_SIZES or not isinstance(table_sizes, torch.Tensor) or not table_sizes.is_cuda:
+        return False
+    kept = getattr(table_sizes, "_s3d_host_sizes", None)
+    return kept is None or kept[0] != table_sizes._version
+
+
+def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, nd, table_len, n, h, d, code, stream):
     """The plan buffer (s3d_attn_plan) of this window set and shape, built on first use and kept as an attribute
     of the caller's w_sizes tensor; None when there is no tensor object to keep it on.  A plan is valid for the
     contents it was built from (the tensors' version counters are checked) and for one stream (it holds the work
@@ -122,7 +133,7 @@ def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, table_len, 
     plans = getattr(w_sizes_in, "_s3d_attn_plans", None)
     if plans is None:
         plans = w_sizes_in._s3d_attn_plans = {}
-    key = (h, d, code, tuple(sizes), n, stream)
+    key = (h, d, code, tuple(sizes) if sizes is not None else None, n, stream)
     stamp = (w_sizes_in._version, w2n_in._version, w2n_in.data_ptr())
     kept = plans.get(key)
     if kept is not None and kept[0] == stamp:
@@ -130,8 +141,10 @@ def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, table_len, 
     num_w = w_sizes.numel()
     nbytes = lib.s3d_attn_plan_bytes(h, n, num_w)
     plan = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=w_sizes.device)
-    status = lib.s3d_attn_plan(c_sizes, len(sizes), table_len, w_sizes.data_ptr(), w2n.data_ptr(), n, h, d, num_w, code,
-                               plan.data_ptr(), nbytes, stream)
+    # the work list depends on the tables through their total length only: no sizes are passed when they are
+    # on the device
+    status = lib.s3d_attn_plan(c_sizes if sizes is not None else None, nd, table_len, w_sizes.data_ptr(),
+                               w2n.data_ptr(), n, h, d, num_w, code, plan.data_ptr(), nbytes, stream)
     _lib.check(status, "s3d_attn_plan")
     plans[key] = (stamp, plan)
     return plan
@@ -145,7 +158,10 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5); dense, or views with
                    a dense (H,D) block and one common row stride (slices of a [N,3*H*D] projection output)
     table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
-    table_sizes    int tensor / list [nd], per-axis element counts rows*H*D (read on the host)
+    table_sizes    int tensor / list [nd], per-axis element counts rows*H*D.  A list or CPU tensor is read on
+                   the host; a CUDA tensor stays on the device and the sweep kernel reads it (no host wait, no
+                   check of the values beyond clipping them to the table; the MFMA kernel is then not chosen)
+                   unless force_mfma or DEVICE_TABLE_SIZES = False ask for the host copy
     w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
     n2n            [N] window-sorted position -> row of q/k/v, or None when the rows are in window-sorted
                    order already (the sweep kernel then reads and writes them without the indirection)
@@ -177,14 +193,21 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     row_stride = _row_stride(q)
     if d not in (8, 16):
         raise ValueError(f"head_dim must be 8 or 16, got {d}")
-    sizes = _host_table_sizes(table_sizes)
-    nd = len(sizes)
+    if not force_mfma and _sizes_stay_on_device(table_sizes):
+        sizes = None
+        sizes_dev = _as_int32("table_sizes", table_sizes.reshape(-1), dev)
+        nd = sizes_dev.numel()
+        c_sizes = sizes_dev.data_ptr()
+    else:
+        sizes = _host_table_sizes(table_sizes)
+        nd = len(sizes)
     if nd not in (3, 6, 9):
         raise ValueError(f"table_sizes must have 3, 6 or 9 entries, got {nd}")
-    if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_q.numel():
-        raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
-                         f"to the table length {table_q.numel()}")
-    c_sizes = (ctypes.c_int32 * nd)(*sizes)
+    if sizes is not None:
+        if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_q.numel():
+            raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
+                             f"to the table length {table_q.numel()}")
+        c_sizes = (ctypes.c_int32 * nd)(*sizes)
     table_len = table_q.numel()
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
@@ -222,17 +245,22 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     code = _DTYPE_CODE[q.dtype]
     num_w = w_sizes.numel()
     flags = ((_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |
-             (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0))
+             (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0) |
+             (_lib.S3D_ATTN_SIZES_ON_DEVICE if sizes is None else 0))
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
         # the sweep kernel's work list depends on the window set only: it is built once and kept on the
         # caller's w_sizes tensor, so the blocks that share a window set share it
-        mfma = (not flags & _lib.S3D_ATTN_FORCE_GENERIC and n2n is not None and max_window_voxels >= 1 and
+        mfma = (sizes is not None and not flags & _lib.S3D_ATTN_FORCE_GENERIC and n2n is not None and
+                max_window_voxels >= 1 and
                 (force_mfma or lib.s3d_attn_fwd_uses_mfma(c_sizes, nd, h, d, code, n, num_w)))
         plan = None if mfma or not REUSE_PLANS else _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes,
-                                                              table_len, n, h, d, code, stream)
+                                                              nd, table_len, n, h, d, code, stream)
         if plan is not None:
             workspace, ws_bytes, flags = plan, plan.numel(), flags | _lib.S3D_ATTN_PLANNED
+        elif sizes is None:
+            ws_bytes = lib.s3d_attn_plan_bytes(h, n, num_w)   # the sweep kernel's work list
+            workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         else:
             ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, num_w, max_window_voxels)
             workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)

@@ -16,6 +16,8 @@ def _check(oracle_lib, case, dtype):
     ref = oracle_lib.attn_fwd(*case.oracle_args())
     got = run_attention(case, dtype)
     assert_attn_close(got, ref, dtype)
+    # per-axis table sizes read by the kernel from device memory: the bits of the sweep kernel with host sizes
+    assert np.array_equal(run_attention(case, dtype, device_sizes=True), run_attention(case, dtype, force_generic=True))
     if dtype == torch.float16:
         # fp16: the library picks the sweep or the MFMA kernel by head_dim; both must agree with the oracle
         assert_attn_close(run_attention(case, dtype, force_generic=True), ref, dtype)
@@ -161,8 +163,8 @@ def test_single_voxel_windows_and_one_head(oracle_lib, hip_lib):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_more_windows_than_list_builder_threads(oracle_lib, hip_lib, dtype):
     """40 000 windows of one to four voxels (a sparse 3-D lattice of window cells): the work-list kernels of the
-    sweep kernel run at most 128 workgroups of 256 threads, so here every thread places several windows, and
-    all units are of the small kinds."""
+    sweep kernel run at most 32 workgroups of 256 threads, so here every wavefront ranks several rounds of 64
+    windows, and all units are of the small kinds."""
     ws, quant, heads, dim = 5, 4, 6, 8
     rng = np.random.default_rng(61)
     cells = np.stack(np.meshgrid(np.arange(50), np.arange(40), np.arange(20), indexing="ij"), -1).reshape(-1, 3)
@@ -315,6 +317,51 @@ def test_random_shapes(oracle_lib, hip_lib, seed):
     if dtype == torch.float16:
         _sharp16(case)
     _check(oracle_lib, case, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_table_sizes_on_the_device_need_no_host_read(oracle_lib, hip_lib, dtype):
+    """The reference's caller hands table_offsets over as a new CUDA tensor on every call (Swin3D/modules/
+    swin3d_layers.py:511).  The forward leaves it on the device (flag S3D_ATTN_SIZES_ON_DEVICE): same bits as with
+    host sizes, axis tables of different lengths (40 rows for the position axes, 32 for colour and normal), no
+    host copy of the values kept on the tensor; a forward that needs gradients reads them once for its backward."""
+    import swin3d_amd
+    from swin3d_amd.sparse_dl.attn import attn_coff
+    case = make_attn_case(oracle_lib, seed=83, n=3000, ws=5, quant=4, heads=6, dim=8, cRSE="XYZ_RGB_NORM",
+                          extent=(12, 12, 5), recipe="layer")
+    assert len(set(int(x) for x in case.table_sizes)) > 1
+    if dtype == torch.float16:
+        to_half_and_back(case)
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    f = lambda a: t(a).to(dtype)
+    i = case.index
+    feats = [f(x) for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
+    index = [t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)]
+    host_sizes = [int(x) for x in case.table_sizes]
+    ref = swin3d_amd.window_attention_forward(*feats, host_sizes, *index, force_generic=True)
+    for sizes_dtype in (torch.int32, torch.int64):
+        sizes = torch.tensor(host_sizes, dtype=sizes_dtype).cuda()
+        got = swin3d_amd.window_attention_forward(*feats, sizes, *index)
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref)
+        assert not hasattr(sizes, "_s3d_host_sizes")
+    from gpu_helpers import assert_attn_close
+    assert_attn_close(got.double().cpu().numpy(), oracle_lib.attn_fwd(*case.oracle_args()), dtype)
+    # the autograd surface: without gradients the sizes stay on the device, with them the host reads them once
+    fn = attn_coff.SelfAttnAIOFunction
+    args = (None, index[0], None, index[1], index[2], index[3])
+    modes = (attn_coff.PosEmb.SEPARATE, attn_coff.TableDims.D0, attn_coff.IndexMode.INDIRECT,
+             attn_coff.PrecisionMode.HALF_NONE)
+    sizes = torch.tensor(host_sizes, dtype=torch.int32).cuda()
+    with torch.no_grad():
+        out = fn.apply(*[x.float() for x in feats], sizes, args, *modes)
+    assert not hasattr(sizes, "_s3d_host_sizes")
+    if dtype == torch.float32:
+        assert torch.equal(out, ref)
+    leaves = [x.float().requires_grad_() for x in feats]
+    fn.apply(*leaves, sizes, args, *modes).sum().backward()
+    assert sizes._s3d_host_sizes[1] == host_sizes and all(x.grad is not None for x in leaves)
 
 
 def test_fp32_elementwise_bound_report(oracle_lib, hip_lib, capsys):
