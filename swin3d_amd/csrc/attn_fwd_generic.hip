@@ -86,7 +86,7 @@ __host__ __device__ inline size_t ws_bins_offset(int H, int64_t W, int64_t N)
 }
 __host__ __device__ inline size_t ws_end_offset(int H, int64_t W, int64_t N)
 {
-    return ws_bins_offset(H, W, N) + ws_round(sizeof(unsigned long long) * kListGroups * (kListThreads / 64) * kBins);
+    return ws_bins_offset(H, W, N) + ws_round(sizeof(unsigned long long) * kListGroups * (kListThreads / 64 + 1) * kBins);
 }
 
 // How the queries of class 0 (sorted by steps, longest first) are cut into units.  A unit is one pass of a
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
         unsigned long long todo = __ballot(b >= 0);
         while (todo != 0) {
             const int leader = __ffsll(todo) - 1;
-            const int cb = __shfl(b, leader), n_lead = __shfl(n, leader);
+            const int cb = __builtin_amdgcn_readlane(b, leader), n_lead = __builtin_amdgcn_readlane(n, leader);
             const bool in = b == cb;
             const unsigned long long same = __ballot(in);
             const int below = __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(same >> 32),
@@ -166,14 +166,14 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
                     if (lane >= off) incl += up;
                 }
                 before_n = incl - (in ? n : 0);
-                all_n = __shfl(incl, 63);
+                all_n = __builtin_amdgcn_readlane(incl, 63);
             }
             uint32_t c = 0, q = 0;
 #pragma unroll
             for (int j = 0; j < kBins / 64; ++j)
                 if ((cb >> 6) == j) { c = held_c[j]; q = held_s[j]; }
-            c = __shfl(c, cb & 63);
-            q = __shfl(q, cb & 63);
+            c = __builtin_amdgcn_readlane(c, cb & 63);
+            q = __builtin_amdgcn_readlane(q, cb & 63);
             if (in) got = make_int2(static_cast<int>(c) + below, static_cast<int>(q) + before_n);
 #pragma unroll
             for (int j = 0; j < kBins / 64; ++j)
@@ -182,10 +182,20 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
         }
         if (w < end) place[w] = got;
     }
+    // the wavefront's totals, and the workgroup's (what the place kernel sums over the launch)
+    __shared__ unsigned long long wave_bins[kWaves][kBins];
+    unsigned long long *sum_bins = group_bins + static_cast<size_t>(kListGroups) * kWaves * kBins;
 #pragma unroll
-    for (int j = 0; j < kBins / 64; ++j)
-        group_bins[static_cast<size_t>(table) * kBins + j * 64 + lane] =
-            (static_cast<unsigned long long>(held_c[j]) << 32) | held_s[j];
+    for (int j = 0; j < kBins / 64; ++j) {
+        const unsigned long long v = (static_cast<unsigned long long>(held_c[j]) << 32) | held_s[j];
+        group_bins[static_cast<size_t>(table) * kBins + j * 64 + lane] = v;
+        wave_bins[threadIdx.x >> 6][j * 64 + lane] = v;
+    }
+    __syncthreads();
+    unsigned long long sum = 0;
+#pragma unroll
+    for (int v = 0; v < kWaves; ++v) sum += wave_bins[v][threadIdx.x];
+    sum_bins[static_cast<size_t>(blockIdx.x) * kBins + threadIdx.x] = sum;
 }
 
 // generic_place_kernel (same grid): bins in order, wavefronts in order inside a bin.  Writes one entry (first
@@ -208,17 +218,17 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
     const unsigned long long *group_bins =
         reinterpret_cast<const unsigned long long *>(ws + ws_bins_offset(a.H, a.W, a.N));
     const int tables = static_cast<int>(gridDim.x) * kWaves, first_table = static_cast<int>(blockIdx.x) * kWaves;
-    // thread t holds bin t: the launch's total, and what the wavefronts before this workgroup's put there; an
-    // exclusive scan over the threads gives the bins their places (entries over all bins, queries restarting per
-    // class)
+    const unsigned long long *sum_bins = group_bins + static_cast<size_t>(kListGroups) * kWaves * kBins;
+    // thread t holds bin t: the launch's total, and what the workgroups before this one put there; an exclusive
+    // scan over the threads gives the bins their places (entries over all bins, queries restarting per class)
     {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         unsigned long long all = 0, before = 0;
 #pragma unroll 8
-        for (int g = 0; g < tables; ++g) {
-            const unsigned long long v = group_bins[static_cast<size_t>(g) * kBins + threadIdx.x];
+        for (int g = 0; g < static_cast<int>(gridDim.x); ++g) {
+            const unsigned long long v = sum_bins[static_cast<size_t>(g) * kBins + threadIdx.x];
             all += v;
-            before += g < first_table ? v : 0;
+            before += g < static_cast<int>(blockIdx.x) ? v : 0;
         }
         const int cnt = static_cast<int>(all >> 32), slots = static_cast<int>(all & 0xffffffffu);
         int incl_c = cnt, incl_s = slots;
@@ -580,12 +590,21 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
                             const float p = __expf(logit[u][hh] - m[hh]);
                             l[hh] += p;
                             v_in[u][hh].fma_to(acc[hh], p);
+                            // The pair's value-table rows are summed in packed fp16 (two short chains), two channels
+                            // per instruction, and enter the fp32 sums once: 4 (ND - 1) + D instructions per pair
+                            // and head at head_dim 8 instead of D * ND mixed-precision FMAs.  The reference's half
+                            // path adds these rows, and the value, in half2 (self_attn_aio_fwd.cu:147); adding the
+                            // value here as well measured -4 % and left too little of the 2e-3 error budget.
+                            Slice<T, D> tv_sum[2];
 #pragma unroll
                             for (int n = 0; n < ND; ++n) {
                                 Slice<T, D> tv_r;
                                 tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
-                                tv_r.fma_to(acc[hh], p);
+                                if (n < 2) tv_sum[n] = tv_r;
+                                else tv_sum[n & 1].add(tv_r);
                             }
+                            tv_sum[0].add(tv_sum[1]);
+                            tv_sum[0].fma_to(acc[hh], p);
                         }
                     }
                 }

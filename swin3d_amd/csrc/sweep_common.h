@@ -172,6 +172,12 @@ template <int D> struct Slice<__half, D> {
             acc[2 * e + 1] = __builtin_fmaf(static_cast<float>(x[e][1]), p, acc[2 * e + 1]);
         }
     }
+    // x += o in packed fp16 (two channels per instruction)
+    __device__ __forceinline__ void add(const Slice &o)
+    {
+#pragma unroll
+        for (int e = 0; e < D / 2; ++e) x[e] = x[e] + o.x[e];
+    }
     // acc + sum_c x[c] * y[c], x widened inside the FMAs
     __device__ __forceinline__ float dot_f32(const float *y, float acc) const
     {
