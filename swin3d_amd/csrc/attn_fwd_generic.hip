@@ -590,21 +590,27 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
                             const float p = __expf(logit[u][hh] - m[hh]);
                             l[hh] += p;
                             v_in[u][hh].fma_to(acc[hh], p);
-                            // The pair's value-table rows are summed in packed fp16 (two short chains), two channels
-                            // per instruction, and enter the fp32 sums once: 4 (ND - 1) + D instructions per pair
-                            // and head at head_dim 8 instead of D * ND mixed-precision FMAs.  The reference's half
-                            // path adds these rows, and the value, in half2 (self_attn_aio_fwd.cu:147); adding the
-                            // value here as well measured -4 % and left too little of the 2e-3 error budget.
-                            Slice<T, D> tv_sum[2];
+                            // The pair's value-table rows are added three at a time in packed fp16, two channels per
+                            // instruction, before they enter the fp32 sums: 56 instructions per pair and head at
+                            // head_dim 8 instead of 80 mixed-precision FMAs.  Groups of three keep the fp16 roundings
+                            // at two per element, on sums of three rows (one chain over all nine rows saves eight
+                            // more instructions, measured 13 % slower - eight dependent adds - and used up the 2e-3
+                            // error budget on tables of magnitude 0.1); adding the value here as well measured -4 %
+                            // for the same reason not to.  The reference's half path adds all rows and the value in
+                            // half2 (self_attn_aio_fwd.cu:147).
+                            constexpr int kGroup = 3;
 #pragma unroll
-                            for (int n = 0; n < ND; ++n) {
-                                Slice<T, D> tv_r;
-                                tv_r.load_lds(off[u][n] + hh * kHeadBytes + 2 * D * sizeof(T));
-                                if (n < 2) tv_sum[n] = tv_r;
-                                else tv_sum[n & 1].add(tv_r);
+                            for (int n0 = 0; n0 < ND; n0 += kGroup) {
+                                Slice<T, D> tv_sum;
+                                tv_sum.load_lds(off[u][n0] + hh * kHeadBytes + 2 * D * sizeof(T));
+#pragma unroll
+                                for (int g = 1; g < kGroup && n0 + g < ND; ++g) {
+                                    Slice<T, D> tv_r;
+                                    tv_r.load_lds(off[u][n0 + g] + hh * kHeadBytes + 2 * D * sizeof(T));
+                                    tv_sum.add(tv_r);
+                                }
+                                tv_sum.fma_to(acc[hh], p);
                             }
-                            tv_sum[0].add(tv_sum[1]);
-                            tv_sum[0].fma_to(acc[hh], p);
                         }
                     }
                 }
