@@ -109,7 +109,10 @@ const char *s3d_last_error_string(void);
  * the axis table when the clamped value equals rows_n, this library folds that
  * case onto the last row).
  *
- * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.
+ * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.  The sweep kernel adds the
+ * value-table rows of a pair three at a time in fp16 before they enter the fp32 sums (the reference's half path
+ * adds all of them and the value in half2, Swin3D/src/attn/self_attn_aio_fwd.cu:147).  Every call gives the
+ * same bits for the same inputs (no atomics on data, work list in window order).
  */
 #define S3D_ATTN_FORCE_GENERIC 1
 #define S3D_ATTN_FORCE_MFMA 2

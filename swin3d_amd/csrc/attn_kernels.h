@@ -43,16 +43,15 @@ int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int wh
 
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
-// the shapes where it is the faster of the two kernels: head_dim 16 with nearly full windows, 240 voxels or more on
+// the shapes where it is the faster of the two kernels: head_dim 16 with full windows, 300 voxels or more on
 // average.  Measured at window 7 on a 56 x 56 x 28 lattice filled to 100 / 80 / 60 / 30 % (343 / 274 / 206 / 103
-// voxels per window), sweep against MFMA kernel in ms: 6 heads 2.12 / 1.97, 1.46 / 1.35, 0.90 / 0.83, 0.29 / 0.31;
-// 20 heads 6.92 / 6.18, 4.62 / 4.24, 2.53 / 2.60, 0.80 / 0.86; 40 heads 13.99 / 12.19, 9.21 / 8.39, 5.10 / 5.11,
-// 1.40 / 1.66.  Room scans (50 to 70 voxels per window at every stage of the encoder) are the sweep kernel's: the
-// Swin3D-L encoder takes 28.6 ms on it alone against 29.6 ms with the MFMA kernel on the many-head blocks.  At
-// head_dim 8 the sweep kernel's packed fp16 dot products win everywhere.
+// voxels per window), sweep against MFMA kernel in ms: 6 heads 2.01 / 1.96, 1.36 / 1.34, 0.83 / 0.83, 0.26 / 0.31;
+// 20 heads 6.39 / 6.14, 4.24 / 4.22, 2.38 / 2.58, 0.76 / 0.85; 40 heads 12.86 / 12.15, 8.43 / 8.36, 4.68 / 5.08,
+// 1.36 / 1.65.  Room scans (50 to 70 voxels per window at every stage of the encoder) are the sweep kernel's.  At
+// head_dim 8 the sweep kernel's packed fp16 arithmetic wins everywhere.
 inline bool attn_mfma_preferred(const AttnArgs &a)
 {
-    return a.D > 8 && a.N >= 240 * a.W;
+    return a.D > 8 && a.N >= 300 * a.W;
 }
 size_t attn_mfma_table_bytes(int H, int D, int padded_rows);
 size_t attn_mfma_items_bytes(int64_t W);

@@ -85,19 +85,19 @@ def test_more_argument_errors_without_a_device(hip_lib):
 
 def test_kernel_choice_is_reported(hip_lib):
     """fp16 Swin3D shapes with head_dim 16 (S and L, stages 2-5) go to the MFMA kernel when the windows hold
-    240 voxels or more on average; sparser scenes, head_dim 8 and fp32 go to the sweep kernel."""
+    300 voxels or more on average; sparser scenes, head_dim 8 and fp32 go to the sweep kernel."""
     import ctypes
     from swin3d_amd import crse
     for ws, heads, dim in [(5, 6, 8), (7, 6, 16), (7, 12, 16), (7, 24, 16), (5, 10, 8), (7, 40, 16)]:
         sizes = crse.crse_table_sizes(ws, 4, heads, dim, "XYZ_RGB_NORM")
         c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 240000, 1000) == (1 if dim == 16 else 0)
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 239999, 1000) == 0
+        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 300000, 1000) == (1 if dim == 16 else 0)
+        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 299999, 1000) == 0
         assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 60000, 1000) == 0
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 0, 256000, 1000) == 0
+        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 0, 320000, 1000) == 0
     sizes = crse.crse_table_sizes(10, 4, 6, 8, "XYZ")          # 80-row tables: generic kernel
     c_sizes = (ctypes.c_int32 * 3)(*sizes)
-    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, 3, 6, 8, 1, 256000, 1000) == 0
+    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, 3, 6, 8, 1, 320000, 1000) == 0
 
 
 def test_window_signals_rejects_bad_arguments(hip_lib):
