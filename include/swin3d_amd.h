@@ -100,7 +100,7 @@ const char *s3d_last_error_string(void);
  *                  max_window_voxels > 32.  The size function returns the larger of the two.
  *   w2n must be ascending (the exclusive prefix sum of w_sizes, as the reference builds it:
  *   Swin3D/modules/swin3d_layers.py:100-103).
- *   D in {8,16}, nd in {3,6,9}, H >= 1.
+ *   D in {8,16,32}, nd in {3,6,9}, H >= 1 (the reference takes head_dim up to 32: self_attn_aio_fwd.cu:486).
  *
  * Row index of axis n for the pair (query i, key j), all in fp32:
  *   rel = (n_coords[i][n] - n_coords[j][n]) + float(rows_n / 2)

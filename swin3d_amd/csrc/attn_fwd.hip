@@ -39,8 +39,8 @@ int check_shape(int64_t N, int64_t W, int32_t H, int32_t D, int32_t nd, int64_t 
                     (long long)N, (long long)W, H, D, nd, (long long)table_len);
     if (nd != 3 && nd != 6 && nd != 9)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d cRSE axes (3, 6 or 9)", nd);
-    if (D != 8 && D != 16)
-        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: head_dim %d (8 or 16)", D);
+    if (D != 8 && D != 16 && D != 32)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: head_dim %d (8, 16 or 32)", D);
     if (W > 0x7fffffffLL || N > 0x7fffffffLL || H > 65535)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: N, W must fit 31 bits and H 16 bits");
     if (table_len / (static_cast<int64_t>(H) * D) > 65536)

@@ -318,10 +318,11 @@ inline int device_cus()
 
 // workgroups per CU the register budget is set for: four at head_dim 8 (one wavefront of each on every SIMD) - the
 // two-head fp16 instance fits 128 registers without spills, and the fourth wavefront per SIMD measured -2 to -3 % -
-// three at head_dim 16 with one head per wavefront, one (of twelve wavefronts) with two heads
+// three at head_dim 16 with one head per wavefront, one (of twelve wavefronts) with two heads, two at head_dim 32
+// (an fp32 query, key, value and output row are 128 registers)
 template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
 {
-    return D > 8 ? (HP == 2 ? 1 : 3) : 4;
+    return D > 16 ? 2 : D > 8 ? (HP == 2 ? 1 : 3) : 4;
 }
 
 // threads of a workgroup: four wavefronts, or twelve where one workgroup has the CU to itself (head_dim 16 with two
@@ -347,7 +348,7 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
     constexpr int kThreads = group_threads<T, D, HP>();
     // streamed keys per loop iteration: at head_dim 16 with one head two interleaved chains hide the LDS round trips;
     // with two heads the heads are the two chains
-    constexpr int kKeys = D <= 8 || HP == 2 ? 1 : 2;
+    constexpr int kKeys = D == 16 && HP == 1 ? 2 : 1;
     // lazy softmax reference (see the loop): -4 % for fp16; fp32 measured no gain (head_dim 8) or a loss (16)
     constexpr bool kLazy = sizeof(T) == 2;
     // 16-byte aligned like the table rows behind it, which are read 16 bytes at a time
@@ -720,7 +721,7 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
     // Two heads per wavefront where the registers allow it (fp16) and the heads pair up: the cRSE rows and LDS
     // addresses of a pair are spent once for both.  At head_dim 16 that means one workgroup of twelve wavefronts per
     // CU (75 KB of tables): it measured -10 % at 6 heads.
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (sizeof(T) == 2 && D <= 16) {
         if (a.H % 2 == 0)
             return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
                          : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
@@ -736,9 +737,10 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream, int what)
     if (a.D == DD && a.nd == NN) return launch_sweep<T, DD, NN>(a, stream, what);
     S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
     S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
+    S3D_CASE(32, 3) S3D_CASE(32, 6) S3D_CASE(32, 9)
 #undef S3D_CASE
     return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: unsupported head_dim %d / cRSE axes %d "
-                "(head_dim in {8,16}, axes in {3,6,9})", a.D, a.nd);
+                "(head_dim in {8,16,32}, axes in {3,6,9})", a.D, a.nd);
 }
 
 }  // namespace

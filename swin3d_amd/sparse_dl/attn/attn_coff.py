@@ -43,8 +43,10 @@ class PrecisionMode(enum.Enum):
 
 _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_F16}
 
-# s3d_attn_bwd keeps a head's table gradients in registers: at most 64 rows per axis on average
+# s3d_attn_bwd keeps a head's table gradients in registers: at most 64 rows per axis on average, head_dim 8 or 16
+# (the forward also takes head_dim 32)
 BWD_MAX_ROWS_PER_AXIS = 64
+BWD_HEAD_DIMS = (8, 16)
 
 # debugging / ablation switch: run the generic VALU kernel even where the MFMA kernel applies
 FORCE_GENERIC = False
@@ -168,8 +170,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
     force_generic  run the VALU sweep kernel for every case
-    force_mfma     run the MFMA kernel wherever it applies (fp16, axis tables of at most 64 rows); by default
-                   it serves head_dim 16 only
+    force_mfma     run the MFMA kernel wherever it applies (fp16, head_dim 8 or 16, axis tables of at most 64
+                   rows); by default it serves head_dim 16 with full windows only
     max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
                    (set by build_window_index) when not given.  Without a bound the sweep kernel serves the
                    call (it takes windows of any size); the host waits for the device to find one only under
@@ -191,8 +193,8 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     if len(strides) != 1 or None in strides:
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     row_stride = _row_stride(q)
-    if d not in (8, 16):
-        raise ValueError(f"head_dim must be 8 or 16, got {d}")
+    if d not in (8, 16, 32):
+        raise ValueError(f"head_dim must be 8, 16 or 32, got {d}")
     if not force_mfma and _sizes_stay_on_device(table_sizes):
         sizes = None
         sizes_dev = _as_int32("table_sizes", table_sizes.reshape(-1), dev)
@@ -292,8 +294,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
         _require_cuda(name, t, dev)
         if t.shape != q.shape or t.dtype != q.dtype:
             raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
-    if d not in (8, 16):
-        raise ValueError(f"head_dim must be 8 or 16, got {d}")
+    if d not in BWD_HEAD_DIMS:
+        raise NotImplementedError(f"attention backward supports head_dim 8 and 16, got {d}")
     sizes = _host_table_sizes(table_sizes)
     nd = len(sizes)
     if nd not in (3, 6, 9):
@@ -368,7 +370,11 @@ class SelfAttnAIOFunction(Function):
         n_coords = n_coords.to(torch.float32).contiguous()
         needs_grad = any(ctx.needs_input_grad[:6])
         if needs_grad:
-            # the backward's limit, reported where the op is called and not from inside autograd
+            # the backward's limits, reported where the op is called and not from inside autograd
+            if raw_query_feats.shape[2] not in BWD_HEAD_DIMS:
+                raise NotImplementedError(
+                    f"attention backward supports head_dim 8 and 16, got {raw_query_feats.shape[2]}; run the forward "
+                    "under torch.no_grad()")
             sizes = _host_table_sizes(table_offsets)
             rows = sum(sizes) // max(raw_query_feats.shape[1] * raw_query_feats.shape[2], 1)
             if rows > BWD_MAX_ROWS_PER_AXIS * len(sizes):
