@@ -189,9 +189,11 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W) bytes
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
- * Every output is a sum in a fixed order (deterministic, no global atomics): dq, dk, dv have one owning
- * lane per row; the table gradients are accumulated per wavefront, left in a slot of the workspace and
- * summed per head by a reduction kernel.
+ * No global atomics.  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on
+ * every call.  The table gradients are accumulated per wavefront over the units it draws from the work queues,
+ * left in a slot of the workspace and summed per head, slots in order, by a reduction kernel: which units a
+ * wavefront draws varies from call to call, so these sums are regrouped and agree between calls to fp32 rounding
+ * (about 1e-6 of the largest element), not bit for bit.
  */
 size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W);
 int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
