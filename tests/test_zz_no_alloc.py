@@ -74,10 +74,12 @@ def test_noalloc_forward_equals_workspace_forward_on_two_calls(oracle_lib, hip_l
 def test_noalloc_forward_rejects_inputs_beyond_its_scratch(hip_lib):
     """More windows than the built-in work list holds: a clear error before anything is launched."""
     from swin3d_amd import _lib
-    n = w = 400000      # one voxel per window: 24 bytes of work list per window
+    # the pointers below are placeholders, so the call must not get as far as a launch: sizes that no built-in
+    # scratch of any plausible size holds (one voxel per window, 24 bytes of work list per window: 26 GB)
+    n = w = 1 << 30
     sizes = [40 * 48] * 3
     c_sizes = (ctypes.c_int32 * 3)(*sizes)
-    assert hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, 3, 6, 8, n, w, 0) > (8 << 20)
+    assert hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, 3, 6, 8, n, w, 0) > (1 << 34)
     one = torch.zeros(16, dtype=torch.float16, device="cuda")
     p = one.data_ptr()
     status = hip_lib.s3d_attn_fwd_noalloc(p, p, p, p, p, p, c_sizes, 3, sum(sizes), p, p, p, p, p, None, None,
