@@ -318,11 +318,12 @@ inline int device_cus()
 
 // workgroups per CU the register budget is set for: four at head_dim 8 (one wavefront of each on every SIMD) - the
 // two-head fp16 instance fits 128 registers without spills, and the fourth wavefront per SIMD measured -2 to -3 % -
+// or three with three heads per wavefront (168 registers);
 // three at head_dim 16 with one head per wavefront, one (of twelve wavefronts) with two heads, two at head_dim 32
 // (an fp32 query, key, value and output row are 128 registers)
 template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
 {
-    return D > 16 ? 2 : D > 8 ? (HP == 2 ? 1 : 3) : 4;
+    return D > 16 ? 2 : D > 8 ? (HP == 2 ? 1 : 3) : (HP == 3 ? 3 : 4);
 }
 
 // threads of a workgroup: four wavefronts, or twelve where one workgroup has the CU to itself (head_dim 16 with two
@@ -340,7 +341,7 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int table_row
 }
 
 // HP: heads a wavefront carries through a unit (adjacent heads HP * g .. HP * g + HP - 1).  The cRSE rows and
-// LDS addresses of a pair do not depend on the head, so two heads share that part of the work.
+// LDS addresses of a pair do not depend on the head, so two or three heads share that part of the work.
 // kSorted: q, k, v and out rows are in window-sorted order already (no n2n).
 template <typename T, int D, int ND, int HP, bool kSorted>
 __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, HP>())) void attn_fwd_sweep_kernel(AttnArgs a)
@@ -722,6 +723,13 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
     // addresses of a pair are spent once for both.  At head_dim 16 that means one workgroup of twelve wavefronts per
     // CU (75 KB of tables): it measured -10 % at 6 heads.
     if constexpr (sizeof(T) == 2 && D <= 16) {
+        // three heads where they go in threes and fit (head_dim 8: 168 registers, three workgroups of 45 KB of
+        // tables per CU): -2 % against pairs at 6 and 12 heads
+        if constexpr (D == 8) {
+            if (a.H % 3 == 0)
+                return a.n2n ? launch_sweep_heads<T, D, ND, 3, false>(a, stream, what)
+                             : launch_sweep_heads<T, D, ND, 3, true>(a, stream, what);
+        }
         if (a.H % 2 == 0)
             return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
                          : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
