@@ -316,22 +316,23 @@ inline int device_cus()
     return 256;
 }
 
-// workgroups per CU the register budget is set for: four at head_dim 8 (one wavefront of each on every SIMD) - the
-// two-head fp16 instance fits 128 registers without spills, and the fourth wavefront per SIMD measured -2 to -3 % -
-// or three with three heads per wavefront (168 registers);
-// three at head_dim 16 with one head per wavefront, one (of twelve wavefronts) with two heads, two at head_dim 32
-// (an fp32 query, key, value and output row are 128 registers)
-template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
-{
-    return D > 16 ? 2 : D > 8 ? (HP == 2 ? 1 : 3) : (HP == 3 ? 3 : 4);
-}
-
-// threads of a workgroup: four wavefronts, or twelve where one workgroup has the CU to itself (head_dim 16 with two
-// heads per wavefront: 75 KB of tables), which keeps three wavefronts on every SIMD (two workgroups of six wavefronts
-// measured 25 % slower than one of twelve)
+// Workgroup shapes.  A workgroup holds its heads' table slices once, so what fits a CU is set by registers and LDS:
+//   one head per wavefront: four workgroups of four wavefronts per CU at head_dim 8 (one wavefront of each on every
+//     SIMD), three at head_dim 16, two at head_dim 32 (an fp32 query, key, value and output row are 128 registers);
+//   fp16, head_dim 8, two heads: four of four (128 registers without spills; the fourth wavefront per SIMD measured
+//     -2 to -3 %); three heads: three of four (168 registers, 45 KB of tables each);
+//   fp32, head_dim 8, two heads: two workgroups of eight wavefronts (126 registers, 65 KB of tables each: four
+//     wavefronts per SIMD; one workgroup of twelve measured 17 % slower than one head per wavefront, this -4 %);
+//   fp16, head_dim 16, two heads: one workgroup of twelve wavefronts (75 KB of tables, three wavefronts per SIMD; two
+//     workgroups of six measured 25 % slower than one of twelve).
 template <typename T, int D, int HP> __host__ __device__ constexpr int group_threads()
 {
-    return D > 8 && HP == 2 ? 768 : 256;
+    return HP == 2 && sizeof(T) == 4 && D == 8 ? 512 : HP == 2 && D == 16 ? 768 : 256;
+}
+template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
+{
+    return group_threads<T, D, HP>() == 512 ? 2 : group_threads<T, D, HP>() == 768 ? 1
+           : D > 16 ? 2 : D > 8 ? 3 : (HP == 3 ? 3 : 4);
 }
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
@@ -730,6 +731,12 @@ int launch_sweep(const AttnArgs &a, hipStream_t stream, int what)
                 return a.n2n ? launch_sweep_heads<T, D, ND, 3, false>(a, stream, what)
                              : launch_sweep_heads<T, D, ND, 3, true>(a, stream, what);
         }
+        if (a.H % 2 == 0)
+            return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
+                         : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
+    }
+    // fp32 at head_dim 8: pairs of heads as well
+    if constexpr (sizeof(T) == 4 && D == 8) {
         if (a.H % 2 == 0)
             return a.n2n ? launch_sweep_heads<T, D, ND, 2, false>(a, stream, what)
                          : launch_sweep_heads<T, D, ND, 2, true>(a, stream, what);
