@@ -279,6 +279,11 @@ def main():
         result["extras"]["attn_bwd"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3),
                                         "vs_forward": ms / kernel_ms, "dtype": "f16 I/O, f32 arithmetic"}
         result["extras"]["other_shapes"] = other_shapes(torch, swin3d_amd, synth, crse, scene, dev)
+        # the headline layer in fp32, the compute type of the operator when autocast is off (PrecisionMode.HALF_NONE)
+        f32_args = tuple(x.float() for x in fwd_args[:6]) + fwd_args[6:]
+        ms = _time_gpu(torch, lambda: swin3d_amd.window_attention_forward(*f32_args), reps=10)
+        result["extras"]["attn_fwd_fp32"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3)}
+        del f32_args
 
     if not args.no_extras and not args.no_encoder:
         result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)
