@@ -231,6 +231,22 @@ class StemConv(nn.Module):
         return voxels.with_feats(F.relu(self.conv_layers[1](out.float())))
 
 
+def _linear(layer, x):
+    """layer(x) for an nn.Linear.  Inference under autocast keeps the parameters' copies in the autocast dtype on
+    the layer (per parameter version) instead of casting them in every forward: autocast's own cache lives only as
+    long as its context, and the encoder has about seventy such layers."""
+    if torch.is_grad_enabled() or not torch.is_autocast_enabled() or not x.is_cuda:
+        return layer(x)
+    dtype = torch.get_autocast_dtype("cuda")
+    w, b = layer.weight, layer.bias
+    key = (dtype, w.data_ptr(), w._version, None if b is None else (b.data_ptr(), b._version))
+    kept = getattr(layer, "_s3d_cast", None)
+    if kept is None or kept[0] != key:
+        kept = (key, w.detach().to(dtype), None if b is None else b.detach().to(dtype))
+        layer._s3d_cast = kept
+    return F.linear(x, kept[1], kept[2])
+
+
 class Mlp(nn.Module):
     """fc1 -> GELU -> fc2 with the reference's attribute names (Swin3D/modules/swin3d_layers.py:153-176);
     dropout is 0 in every shipped configuration and left out."""
@@ -242,7 +258,7 @@ class Mlp(nn.Module):
         self.fc2 = nn.Linear(hidden_features, in_features)
 
     def forward(self, x):
-        return self.fc2(self.act(self.fc1(x)))
+        return _linear(self.fc2, self.act(_linear(self.fc1, x)))
 
 
 def _fused_norm_applies(feats):
@@ -288,7 +304,7 @@ class GridKNNDownsample(nn.Module):
             if pending is not None:
                 voxels.feats += pending
             normed = self.norm(voxels.feats)
-        projected = self.linear(normed)
+        projected = _linear(self.linear, normed)
         if not torch.is_grad_enabled() and projected.is_cuda and projected.dtype in (torch.float16, torch.float32):
             feats = knn_max_pool(idx, projected)      # one kernel, no [Nq, K, C] intermediate
         else:
@@ -359,7 +375,7 @@ class WindowAttention(nn.Module):
             query, key, value, *tables, self.table_sizes, [m2w, w_sizes, w2m, w2n, n2n, n_crse], PosEmb.SEPARATE,
             TableDims.D0, IndexMode.INDIRECT, precision)
         out = out.reshape(n, self.dim)
-        return self.proj(out if torch.is_autocast_enabled() else out.to(feats.dtype))
+        return _linear(self.proj, out if torch.is_autocast_enabled() else out.to(feats.dtype))
 
 
 class SwinBlock(nn.Module):
