@@ -324,14 +324,19 @@ inline int device_cus()
 //   fp32, head_dim 8, two heads: two workgroups of eight wavefronts (126 registers, 65 KB of tables each: four
 //     wavefronts per SIMD; one workgroup of twelve measured 17 % slower than one head per wavefront, this -4 %);
 //   fp16, head_dim 16, two heads: one workgroup of twelve wavefronts (75 KB of tables, three wavefronts per SIMD; two
-//     workgroups of six measured 25 % slower than one of twelve).
+//     workgroups of six measured 25 % slower than one of twelve);
+//   fp32, head_dim 16: one workgroup of twelve wavefronts as well (75 KB of tables, 160 registers: -19 % against two
+//     workgroups of four, which is all that LDS held); fp32, head_dim 32: one workgroup of eight (125 KB of tables).
 template <typename T, int D, int HP> __host__ __device__ constexpr int group_threads()
 {
-    return HP == 2 && sizeof(T) == 4 && D == 8 ? 512 : HP == 2 && D == 16 ? 768 : 256;
+    return sizeof(T) == 4 && D == 32 ? 512
+           : HP == 2 && sizeof(T) == 4 && D == 8 ? 512
+           : (HP == 2 || sizeof(T) == 4) && D == 16 ? 768 : 256;
 }
 template <typename T, int D, int HP> __host__ __device__ constexpr int groups_per_cu()
 {
-    return group_threads<T, D, HP>() == 512 ? 2 : group_threads<T, D, HP>() == 768 ? 1
+    return sizeof(T) == 4 && D == 32 ? 1
+           : group_threads<T, D, HP>() == 512 ? 2 : group_threads<T, D, HP>() == 768 ? 1
            : D > 16 ? 2 : D > 8 ? 3 : (HP == 3 ? 3 : 4);
 }
 
