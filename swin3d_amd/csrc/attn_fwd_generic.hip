@@ -320,7 +320,8 @@ inline int device_cus()
 //   one head per wavefront: four workgroups of four wavefronts per CU at head_dim 8 (one wavefront of each on every
 //     SIMD), three at head_dim 16, two at head_dim 32 (an fp32 query, key, value and output row are 128 registers);
 //   fp16, head_dim 8, two heads: four of four (128 registers without spills; the fourth wavefront per SIMD measured
-//     -2 to -3 %); three heads: three of four (168 registers, 45 KB of tables each);
+//     -2 to -3 %); three heads: one workgroup of twelve wavefronts (168 registers, 45 KB of tables: -4 % against
+//     three workgroups of four; sixteen-wavefront workgroups for the one- and two-head instances measured +-2 %);
 //   fp32, head_dim 8, two heads: two workgroups of eight wavefronts (126 registers, 65 KB of tables each: four
 //     wavefronts per SIMD; one workgroup of twelve measured 17 % slower than one head per wavefront, this -4 %);
 //   fp16, head_dim 16, two heads: one workgroup of twelve wavefronts (75 KB of tables, three wavefronts per SIMD; two
@@ -330,6 +331,7 @@ inline int device_cus()
 template <typename T, int D, int HP> __host__ __device__ constexpr int group_threads()
 {
     return sizeof(T) == 4 && D == 32 ? 512
+           : HP == 3 ? 768
            : HP == 2 && sizeof(T) == 4 && D == 8 ? 512
            : (HP == 2 || sizeof(T) == 4) && D == 16 ? 768 : 256;
 }
@@ -337,7 +339,7 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int groups_pe
 {
     return sizeof(T) == 4 && D == 32 ? 1
            : group_threads<T, D, HP>() == 512 ? 2 : group_threads<T, D, HP>() == 768 ? 1
-           : D > 16 ? 2 : D > 8 ? 3 : (HP == 3 ? 3 : 4);
+           : D > 16 ? 2 : D > 8 ? 3 : 4;
 }
 
 // elements of T between table rows in LDS when a workgroup holds the slices of HP heads side by side
