@@ -23,6 +23,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
+SETTLE_MS = 80.0         # untimed, continuous launches before every timed region (see _settle)
+SETTLE = {"ms": SETTLE_MS}
 HEADLINE_PROFILE = os.path.join("profiles", "attn_fwd_headline.txt")
 # the sources of the headline kernel: counter figures taken from a profile are only quoted while these are unchanged
 KERNEL_SOURCES = ["attn_fwd.hip", "attn_fwd_generic.hip", "attn_kernels.h", "sweep_common.h", "s3d_common.h"]
@@ -65,6 +67,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed launches after the warm-up steps until the card has been busy this long (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (0 = the library picks, 1 = sweep kernel, 2 = MFMA kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
@@ -78,6 +82,7 @@ def main():
                     help="run only the Swin3D-L encoder forward (1 warm-up + 3 timed passes, no UNet) and print its "
                          "figures: the command the encoder's kernel trace is taken with")
     args = ap.parse_args()
+    SETTLE["ms"] = args.settle_ms   # the side figures' helpers read it
     if args.sources_hash:
         print(kernel_sources_sha256())
         return 0
@@ -154,6 +159,8 @@ def main():
 
     for _ in range(args.warmup):
         step()
+    # ... and further untimed launches until the card has been busy for args.settle_ms (its clocks settle)
+    settle_launches = _settle(torch, step)
     torch.cuda.synchronize()
     # per-launch kernel time from events on the launch stream (torch's current stream)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
@@ -180,6 +187,9 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle": {"ms": args.settle_ms, "untimed_launches": settle_launches,
+                   "note": "after the warm-up steps, untimed launches of the same call until the card has been busy "
+                           "this long; every side figure does the same"},
         "ms_per_step": wall_ms,
         "higher_is_better": True,
         "scaling": "weak",
@@ -232,7 +242,7 @@ def main():
         """median launch time as in the timed region above: all calls enqueued, one wait at the end"""
         for _ in range(warm):
             fn()
-        torch.cuda.synchronize()
+        _settle(torch, fn)
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for s_ev, e_ev in evs:
             s_ev.record(stream)
@@ -298,9 +308,25 @@ def main():
     return 0
 
 
-def _time_gpu(torch, fn, reps=20, warm=3):
+def _settle(torch, fn, ms=None, batch=20):
+    """Untimed launches of `fn`, back to back, for at least `ms` of wall clock: the card reaches its steady clocks only
+    after some tens of milliseconds of continuous work (the headline kernel measures 0.24 ms per launch in the first
+    10 ms after an idle period and 0.205 ms from about 40 ms on), and a training or serving loop runs there.  Returns
+    the number of launches."""
+    done = 0
+    t_end = time.perf_counter() + (SETTLE["ms"] if ms is None else ms) * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(batch):
+            fn()
+        done += batch
+        torch.cuda.synchronize()
+    return done
+
+
+def _time_gpu(torch, fn, reps=20, warm=3, settle_ms=None):
     for _ in range(warm):
         fn()
+    _settle(torch, fn, settle_ms, batch=max(1, min(20, reps)))
     torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
@@ -400,7 +426,7 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     times = []
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
         outs = model(vox, sig)          # warm-up (allocator, hipBLASLt heuristics)
-        torch.cuda.synchronize()
+        _settle(torch, lambda: model(vox, sig), 2 * SETTLE["ms"], batch=1)
         for _ in range(reps):
             t0 = time.perf_counter()
             outs = model(vox, sig)
@@ -423,7 +449,7 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     times = []
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
         logits = unet(vox, sig)
-        torch.cuda.synchronize()
+        _settle(torch, lambda: unet(vox, sig), 2 * SETTLE["ms"], batch=1)
         for _ in range(reps):
             t0 = time.perf_counter()
             logits = unet(vox, sig)

@@ -51,13 +51,17 @@ __host__ __device__ inline int window_bin(int n, int g)
 // The step target of a launch, as a shift.  The launch ends when its last wavefront does, so a unit must stay
 // short against what a wavefront does in the whole launch: N^2 / W pairs at least, per head group, over the
 // lanes of `waves` wavefronts that serve the group.  64 steps unless that leaves fewer than about six units per
-// wavefront.
+// wavefront; not below 32 where the mean window has at most 32 voxels: a target of 16 would give the typical
+// window two lanes per query, whose softmax states are merged at the end of the unit, where one lane per query
+// serves it in 32 steps without a merge (-3.5 % on 26-voxel windows; on window-7 levels, 57 voxels a window and
+// most pairs in windows of more than 64, the target of 32 measured +4 %: longer units, the same merges).
 __host__ inline int target_shift_for(int64_t N, int64_t W, int waves)
 {
     if (N <= 0 || W <= 0) return 6;
     const double lane_steps = static_cast<double>(N) * static_cast<double>(N) / static_cast<double>(W);
+    const int least = N <= 32 * W ? 5 : 4;
     int shift = 6;
-    while (shift > 4 && lane_steps / (64.0 * (1 << shift)) < 6.0 * (waves > 0 ? waves : 1)) --shift;
+    while (shift > least && lane_steps / (64.0 * (1 << shift)) < 6.0 * (waves > 0 ? waves : 1)) --shift;
     return shift;
 }
 
