@@ -186,7 +186,13 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *   dout           device [N,H,D] of `dtype`: gradient of the loss w.r.t. `out`
  *   dq, dk, dv     device [N,H,D] of `dtype`, overwritten (every row belongs to exactly one window)
  *   dtable_q/k/v   device FP32 [table_len], overwritten; layout of the tables
- *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W) bytes
+ *   pairs          M = sum of w_sizes^2, the pairs of the window set (counts[1] of s3d_window_index; the length
+ *                  of the reference's index arrays), or 0.  With M the call runs two pair sweeps on the forward's
+ *                  kind of work list (dq; dk and dv), which leave dL and P of every (pair, head) in the workspace
+ *                  - 12 * H * pairs bytes -, and two table-gradient sweeps that read them.  With 0 it runs two fused
+ *                  sweeps that recompute the logits for the table gradients and need no such store (about twice
+ *                  the time).  A value below M leaves the gradients of the windows beyond it unwritten.
+ *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs) bytes
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
  * No global atomics.  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on
@@ -195,14 +201,14 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  * wavefront draws varies from call to call, so these sums are regrouped and agree between calls to fp32 rounding
  * (about 1e-6 of the largest element), not bit for bit.
  */
-size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W);
+size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W, int64_t pairs);
 int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
                  const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
                  const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords,
                  const void *out, const float *out_max, const float *out_sum, const void *dout, void *dq,
                  void *dk, void *dv, float *dtable_q, float *dtable_k, float *dtable_v, int64_t N,
-                 int32_t H, int32_t D, int64_t W, int32_t dtype, void *workspace, size_t workspace_bytes,
-                 void *stream);
+                 int32_t H, int32_t D, int64_t W, int64_t pairs, int32_t dtype, void *workspace,
+                 size_t workspace_bytes, void *stream);
 
 /*
  * Window sort + segment offsets.

@@ -46,6 +46,10 @@ struct BwdArgs {
     float *dtq, *dtk, *dtv;
     float *delta;     // [N,H] dout_i . o_i
     float *tgrad;     // per-wavefront table gradients of a sweep: [wavefront][kind][64 * BLK rows][D]
+    int64_t *pos_base;   // [N]: at a window's first sorted position, the pairs (n^2) of the windows before it
+    const float2 *pd;    // [H][pairs]: (dL, P) of the pair sweeps at base + i n + j
+    const float *dl_t;   // [H][pairs]: dL at base + j n + i
+    int64_t pairs;       // capacity of pd and dl_t per head
     int32_t *units;   // H * kQueues work counters (kCounterStride apart), the unit count, (window, chunk) per unit
     int32_t H, D, nd, total_rows;
     int64_t N, W, table_len;
@@ -119,18 +123,22 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
     auto class_of = [](int n) { return n > 256 ? 0 : n > 128 ? 1 : n > 64 ? 2 : n > 32 ? 3 : n > 16 ? 4 : 5; };
     __shared__ int wave_sum[16][kClasses];
     __shared__ int class_start[kClasses + 1];
+    __shared__ long long pairs_before[1024];   // pairs (n^2) of the windows of the threads before this one
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
     const int begin = min(static_cast<int>(threadIdx.x) * per, W), end = min(begin + per, W);
     int mine[kClasses];
 #pragma unroll
     for (int c = 0; c < kClasses; ++c) mine[c] = 0;
+    long long pairs_mine = 0;
     for (int w = begin; w < end; ++w) {
         const int n = a.w_sizes[w];
         const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
 #pragma unroll
         for (int c = 0; c < kClasses; ++c) mine[c] += c == cls ? chunks : 0;
+        pairs_mine += static_cast<long long>(n) * n;
     }
+    pairs_before[threadIdx.x] = pairs_mine;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int incl[kClasses];
 #pragma unroll
@@ -154,8 +162,23 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
             }
         }
         class_start[kClasses] = run;
+        long long before = 0;
+        for (int t = 0; t < 1024; ++t) {
+            const long long add = pairs_before[t];
+            pairs_before[t] = before;
+            before += add;
+        }
     }
     __syncthreads();
+    {
+        // where the (pair, head) records of a window start in the pair store: written at the window's first position
+        long long before = pairs_before[threadIdx.x];
+        for (int w = begin; w < end; ++w) {
+            const int n = a.w_sizes[w];
+            if (n > 0) a.pos_base[a.w2n[w]] = before;
+            before += static_cast<long long>(n) * n;
+        }
+    }
     int run[kClasses];
 #pragma unroll
     for (int c = 0; c < kClasses; ++c) run[c] = wave_sum[wave][c] + incl[c] - mine[c];
@@ -537,6 +560,242 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
     }
 }
 
+// Table gradients from the dL and P that the pair sweeps left for every (pair, head): the histogram and rank-1
+// machinery of the sweeps above without their logits, table rows and owned gradients.
+//   KEY_OWNED: lanes = keys j of a 64-key chunk, the window's queries stream:  dTq += hist(dL) x q_i,  dTv += hist(P) x dout_i
+//   else:      lanes = queries i, the keys stream:                              dTk += hist(dL) x k_j
+// A step's inputs - the lane's record, the streamed rows and coordinates - are fetched one step ahead: the records
+// come from HBM and a step is a short dependent chain (rows, histogram atomics, read-back), so their latency would
+// be most of it.
+template <typename T, int D, int ND, bool KEY_OWNED, int BLK>
+__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) void attn_bwd_tables_kernel(BwdArgs a)
+{
+    constexpr bool kAccB = KEY_OWNED;                          // dTv
+    constexpr int kHistKinds = 1 + (kAccB ? 1 : 0);
+    constexpr int kFlat = BLK * 64;
+    // A histogram cell exists in kCopies copies, chosen by the low bits of the lane number: lanes that hit the
+    // same table row - neighbouring voxels share colours and normals - serialise on a cell, and the copies divide
+    // that by up to kCopies; the copies of a row lie side by side, 16 bytes that the read-back fetches at once.
+    constexpr int kCopies = kAccB ? 2 : 4;
+    constexpr int kHistWords = kHistKinds * 2 * kFlat * kCopies;   // [group][flat row][copy] of 32- or 64-bit cells
+    extern __shared__ float smem[];
+    const int H = a.H;
+    const int HD = H * D;
+    const int h = (blockIdx.x / kQueues) % H;
+    int *hist_all = reinterpret_cast<int *>(smem);
+    for (int t = threadIdx.x; t < kBwdWaves * kHistWords; t += kBwdThreads) hist_all[t] = 0;
+    __syncthreads();   // the only workgroup barrier
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    int *hist_a = hist_all + wave * kHistWords;
+    unsigned long long *hist_ab = reinterpret_cast<unsigned long long *>(hist_a);
+    const T *gx = static_cast<const T *>(KEY_OWNED ? a.q : a.k);      // the streamed row of the first rank-1 update
+    const T *gy = static_cast<const T *>(a.dout);                     // ... of the second (key-owned)
+
+    // The rank-1 updates as 4x4x1 MFMAs wherever the VALU form would not fit the registers: the accumulators may
+    // then live in accumulation registers.  Measured at head_dim 8 (us, VALU / MFMA form): fp16 with five 64-row
+    // blocks 658 / 1017 key-owned and 387 / 510 query-owned; six blocks 1804 / 817 and 843 / 508 (the VALU form
+    // spills); fp32 with five blocks 1256 / 644 and 384 / 380.
+    constexpr bool kMfmaUpdate = D > 8 || BLK > 5 || (KEY_OWNED && sizeof(T) == 4);
+    float acc_a[BLK][D], acc_b[kAccB ? BLK : 1][D];
+#pragma unroll
+    for (int m = 0; m < BLK; ++m)
+#pragma unroll
+        for (int c = 0; c < D; ++c) {
+            acc_a[m][c] = 0.0f;
+            if (kAccB) acc_b[m][c] = 0.0f;
+        }
+    auto mfma_update = [](float (&acc)[D], float row_sum, const float (&b)[D / 4]) {
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            f32x4_t r = {acc[4 * c], acc[4 * c + 1], acc[4 * c + 2], acc[4 * c + 3]};
+            r = __builtin_amdgcn_mfma_f32_4x4x1f32(row_sum, b[c], r, 0, 0, 0);
+            acc[4 * c] = r[0]; acc[4 * c + 1] = r[1]; acc[4 * c + 2] = r[2]; acc[4 * c + 3] = r[3];
+        }
+    };
+    // per-axis constants, kept in scalar registers
+    float half_rows[ND], upper[ND];
+#pragma unroll
+    for (int n = 0; n < ND; ++n) {
+        half_rows[n] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(static_cast<float>(a.rows[n] / 2))));
+        upper[n] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(crse_upper(a.rows[n]))));
+    }
+    const int copy = lane & (kCopies - 1);
+
+    const int2 *unit_list = reinterpret_cast<const int2 *>(a.units + units_list_index(H));
+    const int total_units = __builtin_amdgcn_readfirstlane(a.units[units_total_index(H)]);
+    int *counters = a.units + h * kQueues * kCounterStride;
+
+    int queue = xcd_id() % kQueues;
+    int tried = 0;
+    int drawn = 0;
+    if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+    for (;;) {
+        int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        while (unit >= total_units && ++tried < kQueues) {
+            queue = (queue + 1) % kQueues;
+            if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+            unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        }
+        if (unit >= total_units) break;
+        const int2 desc = unit_list[unit];
+        const int w = __builtin_amdgcn_readfirstlane(desc.x);
+        const int chunk = __builtin_amdgcn_readfirstlane(desc.y);
+        const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
+        const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
+        const int gs = n_w <= 32 ? 32 : 64;
+        const int ng = 64 / gs;
+        const int grp = lane / gs;
+        const int own = chunk * kChunk + (lane - grp * gs);
+        const bool own_valid = own < n_w;
+        const int own_in = min(own, n_w - 1);
+        // records of this window and head in the pair store; a window beyond the store contributes nothing
+        const int64_t before = a.pos_base[s0];
+        const int64_t before_u = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(before >> 32))) << 32) |
+                                 static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(before)));
+        const bool fits = before_u + static_cast<int64_t>(n_w) * n_w <= a.pairs;
+        const int64_t stored_at = static_cast<int64_t>(h) * a.pairs + before_u + own_in;
+        float own_c[ND];
+#pragma unroll
+        for (int n = 0; n < ND; ++n) own_c[n] = a.n_coords[static_cast<int64_t>(s0 + own_in) * ND + n];
+
+        const int steps = (n_w + ng - 1) / ng;
+        // The inputs of step `it` for this lane's group (streamed element st = it ng + grp): the streamed rows and
+        // coordinates are fetched one step ahead, the lane's records kPrefetch steps ahead.  Every load of the loop is
+        // unconditional (clamped positions; what lies past the end is masked where it is used), so the waits count
+        // loads statically and a step waits for the oldest record only.
+        constexpr int kPrefetch = 4;
+        struct StepIn {
+            Slice<T, D> x, y;
+            float c[ND];
+        };
+        auto fetch = [&](int it, int st_row, StepIn &in) {
+            const int st = min(it * ng + grp, n_w - 1);
+            in.x.load(gx + static_cast<int64_t>(st_row) * HD + h * D);
+            if constexpr (KEY_OWNED) in.y.load(gy + static_cast<int64_t>(st_row) * HD + h * D);
+#pragma unroll
+            for (int n = 0; n < ND; ++n) in.c[n] = a.n_coords[static_cast<int64_t>(s0 + st) * ND + n];
+        };
+        // a window beyond the store reads the first record of the head instead (never used: `fits` masks it)
+        const int64_t rec_base = fits ? stored_at : static_cast<int64_t>(h) * a.pairs;
+        const int rec_stride = fits ? n_w : 0;
+        auto fetch_record = [&](int it) {
+            const int st = min(it * ng + grp, n_w - 1);
+            const int64_t rec_at = rec_base + static_cast<int64_t>(st) * rec_stride;
+            float2 rec = make_float2(0.0f, 0.0f);
+            if constexpr (KEY_OWNED) rec = a.pd[rec_at];
+            else rec.x = a.dl_t[rec_at];
+            return rec;
+        };
+        // the next unit's ticket, drawn here: its round trip overlaps the unit's first loads
+        if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+        StepIn next;
+        float2 rec_ahead[kPrefetch];
+#pragma unroll
+        for (int e = 0; e < kPrefetch; ++e) rec_ahead[e] = fetch_record(e);
+        int row_after = a.n2n[s0 + min(ng + grp, n_w - 1)];   // row of step 1's element
+        fetch(0, a.n2n[s0 + min(grp, n_w - 1)], next);
+        for (int it = 0; it < steps; ++it) {
+            const StepIn cur = next;
+            const bool have = own_valid && fits && it * ng + grp < n_w;
+            const float2 rec = rec_ahead[0];
+#pragma unroll
+            for (int e = 0; e + 1 < kPrefetch; ++e) rec_ahead[e] = rec_ahead[e + 1];
+            rec_ahead[kPrefetch - 1] = fetch_record(it + kPrefetch);
+            {
+                const int row_next = row_after;
+                row_after = a.n2n[s0 + min((it + 2) * ng + grp, n_w - 1)];
+                fetch(it + 1, row_next, next);
+            }
+            const float dl = have ? rec.x : 0.0f, p = have ? rec.y : 0.0f;
+            const float amax = group_max_nonneg(fabsf(dl), ng == 2, grp);
+            const int qd = __float2int_rn(dl * (amax > 0.0f ? kFixL * __builtin_amdgcn_rcpf(amax) : 0.0f));
+            if constexpr (kAccB) {
+                const int qp = __float2int_rn(p * kFixP);
+                const unsigned long long both =
+                    (static_cast<unsigned long long>(static_cast<unsigned>(qd)) << 32) + static_cast<unsigned>(qp);
+                if (both != 0) {
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) {
+                        const float ci = KEY_OWNED ? cur.c[n] : own_c[n], cj = KEY_OWNED ? own_c[n] : cur.c[n];
+                        atomicAdd(hist_ab + (grp * kFlat + a.base[n] + crse_row(ci, cj, half_rows[n], upper[n])) * kCopies + copy, both);
+                    }
+                }
+            } else {
+                if (qd != 0) {
+#pragma unroll
+                    for (int n = 0; n < ND; ++n) {
+                        const float ci = KEY_OWNED ? cur.c[n] : own_c[n], cj = KEY_OWNED ? own_c[n] : cur.c[n];
+                        atomicAdd(hist_a + (grp * kFlat + a.base[n] + crse_row(ci, cj, half_rows[n], upper[n])) * kCopies + copy, qd);
+                    }
+                }
+            }
+            wave_lds_fence();
+            for (int g = 0; g < ng; ++g) {
+                const int src = __builtin_amdgcn_readfirstlane(g * gs);
+                const float sc = lane_value(amax, src) * (1.0f / kFixL);
+                const Slice<T, D> sx = cur.x.lane(src);
+                float bx[D / 4], by[D / 4];
+                if constexpr (kMfmaUpdate) sx.quad_channels(lane, bx);
+                if constexpr (kAccB) {
+                    const Slice<T, D> sy = cur.y.lane(src);
+                    if constexpr (kMfmaUpdate) sy.quad_channels(lane, by);
+#pragma unroll
+                    for (int m = 0; m < BLK; ++m) {
+                        // both copies of the row in one 16-byte read; the halves add without carry (see above)
+                        uint4 *cell = reinterpret_cast<uint4 *>(hist_ab + (g * kFlat + m * 64 + lane) * kCopies);
+                        const uint4 two = *cell;
+                        *cell = make_uint4(0, 0, 0, 0);
+                        const unsigned long long both = ((static_cast<unsigned long long>(two.y) << 32) | two.x) +
+                                                        ((static_cast<unsigned long long>(two.w) << 32) | two.z);
+                        const float gsum = static_cast<float>(static_cast<int>(both >> 32)) * sc;
+                        const float psum = static_cast<float>(static_cast<unsigned>(both)) * (1.0f / kFixP);
+                        if constexpr (kMfmaUpdate) {
+                            mfma_update(acc_a[m], gsum, bx);
+                            mfma_update(acc_b[m], psum, by);
+                        } else {
+                            sx.fma_to(acc_a[m], gsum);
+                            sy.fma_to(acc_b[m], psum);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int m = 0; m < BLK; ++m) {
+                        int4 *cell = reinterpret_cast<int4 *>(hist_a + (g * kFlat + m * 64 + lane) * kCopies);
+                        const int4 four = *cell;
+                        *cell = make_int4(0, 0, 0, 0);
+                        const float gsum = static_cast<float>(four.x + four.y + four.z + four.w) * sc;
+                        if constexpr (kMfmaUpdate) mfma_update(acc_a[m], gsum, bx);
+                        else sx.fma_to(acc_a[m], gsum);
+                    }
+                }
+            }
+            wave_lds_fence();
+        }
+    }
+
+    float *slot = a.tgrad + (static_cast<size_t>(blockIdx.x) * kBwdWaves + wave) * (2 * kFlat * D);
+#pragma unroll
+    for (int m = 0; m < BLK; ++m) {
+        if constexpr (kMfmaUpdate) {
+#pragma unroll
+            for (int c = 0; c < D / 4; ++c) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const size_t at = static_cast<size_t>(m * 64 + (lane & ~3) + i) * D + 4 * c + (lane & 3);
+                    slot[at] = acc_a[m][4 * c + i];
+                    if constexpr (kAccB) slot[static_cast<size_t>(kFlat) * D + at] = acc_b[m][4 * c + i];
+                }
+            }
+        } else {
+            const int row = m * 64 + lane;
+            store_row<D>(slot + static_cast<size_t>(row) * D, acc_a[m]);
+            if constexpr (kAccB) store_row<D>(slot + static_cast<size_t>(kFlat + row) * D, acc_b[m]);
+        }
+    }
+}
+
 // Sums the per-wavefront table gradients of a sweep over the wavefronts of each head: one thread per
 // (kind, flat row, head, channel).  dst_a / dst_b: the gradient tables of kind 0 / 1 (null = not produced).
 __global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float *dst_a, float *dst_b, int flat_rows,
@@ -592,6 +851,58 @@ int launch_sweep_blk(const BwdArgs &a, int grid, hipStream_t stream)
     return S3D_OK;
 }
 
+// workgroups of a sweep: whole sets of (XCDs x heads), about two per CU (a workgroup serves one head for its
+// whole life).  At head_dim 16 only one fits a CU at a time; the others start as the first heads run out of
+// units and go to the heads that still have some, which measured 5 % faster than a grid of one per CU (whole
+// sets leave 16 of 256 CUs without a workgroup at six heads).
+constexpr int kTablesPerCu = 4;   // workgroups per CU of the table-gradient kernels, at most
+int bwd_grid(int H, int per_cu = 2)
+{
+    int device = 0, cus = 256;
+    if (hipGetDevice(&device) == hipSuccess) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
+    }
+    const int set = kQueues * H;
+    return (per_cu * cus / set > 0 ? per_cu * cus / set : 1) * set;
+}
+
+template <typename T, int D, int ND, bool KEY_OWNED, int BLK>
+int launch_tables_blk(const BwdArgs &a, int grid, hipStream_t stream)
+{
+    constexpr int kinds = KEY_OWNED ? 2 : 1;
+    auto kernel = attn_bwd_tables_kernel<T, D, ND, KEY_OWNED, BLK>;
+    constexpr int copies = KEY_OWNED ? 2 : 4;
+    const size_t lds = sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(BLK) * 64 * copies;
+    S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    // as many workgroups per CU as registers and histograms allow (at most kTablesPerCu: the slots of the
+    // workspace), in whole sets of (XCDs x heads)
+    int fit = 0;
+    S3D_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reinterpret_cast<const void *>(kernel), kBwdThreads, lds));
+    grid = bwd_grid(a.H, fit < 1 ? 1 : fit > kTablesPerCu ? kTablesPerCu : fit);
+    hipLaunchKernelGGL(bwd_reset_counters_kernel, dim3(1), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
+    S3D_HIP_CHECK(hipGetLastError());
+    const int threads = 2 * a.total_rows * a.H * a.D;
+    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
+                       a, KEY_OWNED ? a.dtq : a.dtk, KEY_OWNED ? a.dtv : nullptr, BLK * 64, grid);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+template <typename T, int D, int ND, bool KEY_OWNED>
+int launch_tables(const BwdArgs &a, int grid, hipStream_t stream)
+{
+    const int blocks = (a.total_rows + 63) / 64;
+    constexpr int kSmall = 2 * ND / 3;
+    if constexpr (ND == 9) {
+        if (blocks <= 5) return launch_tables_blk<T, D, ND, KEY_OWNED, 5>(a, grid, stream);
+    }
+    if (blocks <= kSmall) return launch_tables_blk<T, D, ND, KEY_OWNED, kSmall>(a, grid, stream);
+    return launch_tables_blk<T, D, ND, KEY_OWNED, ND>(a, grid, stream);
+}
+
 // table-gradient registers for as many 64-row blocks as the head's flat table has: 5 for window 5 at four steps
 // per cell with all nine axes (312 rows), 6 for window 7 (360 rows); every block costs 2 * D registers and a
 // share of the per-step histogram flush
@@ -607,23 +918,8 @@ int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
     return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, ND>(a, grid, stream);
 }
 
-// workgroups of a sweep: whole sets of (XCDs x heads), about two per CU (a workgroup serves one head for its
-// whole life).  At head_dim 16 only one fits a CU at a time; the others start as the first heads run out of
-// units and go to the heads that still have some, which measured 5 % faster than a grid of one per CU (whole
-// sets leave 16 of 256 CUs without a workgroup at six heads).
-int bwd_grid(int H)
-{
-    int device = 0, cus = 256;
-    if (hipGetDevice(&device) == hipSuccess) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) cus = v;
-    }
-    const int set = kQueues * H;
-    return (2 * cus / set > 0 ? 2 * cus / set : 1) * set;
-}
-
 template <typename T, int D, int ND>
-int launch_bwd(const BwdArgs &a, hipStream_t stream)
+int launch_bwd(const BwdArgs &a, const BwdPairArgs &pairs, int dtype, hipStream_t stream)
 {
     const int64_t work = a.N * a.H + a.table_len;
     const int prep_grid = static_cast<int>(ceil_div(work > 0 ? work : 1, 256) < 4096 ? ceil_div(work > 0 ? work : 1, 256) : 4096);
@@ -632,6 +928,12 @@ int launch_bwd(const BwdArgs &a, hipStream_t stream)
     hipLaunchKernelGGL(bwd_units_kernel, dim3(1), dim3(1024), 0, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     const int grid = bwd_grid(a.H);
+    if (a.pairs > 0) {
+        // dq, dk, dv by the pair sweeps, which leave dL and P of every (pair, head); the table gradients from those
+        if (int rc = launch_attn_bwd_pairs(pairs, dtype, stream)) return rc;
+        if (int rc = launch_tables<T, D, ND, true>(a, grid, stream)) return rc;
+        return launch_tables<T, D, ND, false>(a, grid, stream);
+    }
     // one key-owned sweep for dk, dv and both of its table gradients; at head_dim 16 with more than six 64-row
     // blocks of table rows (quant 8) the two sets of accumulation registers no longer fit one wavefront
     // (250-320 registers spilled) and the sweep runs as its two halves
@@ -680,19 +982,28 @@ size_t bwd_delta_bytes(int64_t N, int H) { return align_up(sizeof(float) * stati
 // one slot per wavefront of a sweep: two kinds x (64 rows per axis at most) x D floats
 size_t bwd_tgrad_bytes(int H, int D, int nd)
 {
-    return align_up(sizeof(float) * static_cast<size_t>(bwd_grid(H)) * kBwdWaves * 2 * (64 * nd) * D, 256);
+    return align_up(sizeof(float) * static_cast<size_t>(bwd_grid(H, kTablesPerCu)) * kBwdWaves * 2 * (64 * nd) * D, 256);
 }
+
+// the pair path's part of the workspace: window pair offsets, (dL, P) and transposed dL of every (pair, head), and
+// the pair sweeps' work list
+size_t bwd_pos_base_bytes(int64_t N) { return align_up(sizeof(int64_t) * static_cast<size_t>(N > 0 ? N : 1), 256); }
+size_t bwd_pd_bytes(int H, int64_t pairs) { return align_up(sizeof(float2) * static_cast<size_t>(H) * pairs, 256); }
+size_t bwd_dlt_bytes(int H, int64_t pairs) { return align_up(sizeof(float) * static_cast<size_t>(H) * pairs, 256); }
 
 }  // namespace
 }  // namespace s3d
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D,
                                                                                       int32_t nd, int64_t N,
-                                                                                      int64_t W)
+                                                                                      int64_t W, int64_t pairs)
 {
     using namespace s3d;
-    if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || N < 0 || W < 0) return 0;
-    return bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd);
+    if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || N < 0 || W < 0 || pairs < 0) return 0;
+    size_t need = bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
+    if (pairs > 0)
+        need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_generic_workspace_bytes(H, W, N), 256);
+    return need;
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
@@ -701,12 +1012,12 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, const void *out,
     const float *out_max, const float *out_sum, const void *dout, void *dq, void *dk, void *dv,
     float *dtable_q, float *dtable_k, float *dtable_v, int64_t N, int32_t H, int32_t D, int64_t W,
-    int32_t dtype, void *workspace, size_t workspace_bytes, void *stream)
+    int64_t pairs, int32_t dtype, void *workspace, size_t workspace_bytes, void *stream)
 {
     using namespace s3d;
-    if (N < 0 || W < 0 || H < 1 || D < 1 || nd < 1 || table_len < 1)
-        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: bad sizes N=%lld W=%lld H=%d D=%d nd=%d table_len=%lld",
-                    (long long)N, (long long)W, H, D, nd, (long long)table_len);
+    if (N < 0 || W < 0 || H < 1 || D < 1 || nd < 1 || table_len < 1 || pairs < 0)
+        return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: bad sizes N=%lld W=%lld H=%d D=%d nd=%d table_len=%lld pairs=%lld",
+                    (long long)N, (long long)W, H, D, nd, (long long)table_len, (long long)pairs);
     if (nd != 3 && nd != 6 && nd != 9)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d cRSE axes (3, 6 or 9)", nd);
     if (D != 8 && D != 16) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8 or 16)", D);
@@ -725,7 +1036,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     if (int rc = fill_bwd_axes(a, table_sizes, nd, table_len)) return rc;
     if (!dtable_q || !dtable_k || !dtable_v)
         return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null table-gradient pointer");
-    const size_t need = s3d_attn_bwd_workspace_bytes(H, D, nd, N, W);
+    const size_t need = s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_bwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
@@ -741,7 +1052,35 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
     a.units = static_cast<int32_t *>(workspace);
     a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H));
-    a.tgrad = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H));
+    char *at = static_cast<char *>(workspace) + bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H);
+    a.tgrad = reinterpret_cast<float *>(at);
+    at += bwd_tgrad_bytes(H, D, nd);
+    a.pos_base = reinterpret_cast<int64_t *>(at);
+    at += bwd_pos_base_bytes(N);
+    a.pairs = pairs;
+    BwdPairArgs pr{};
+    if (pairs > 0) {
+        float2 *pd = reinterpret_cast<float2 *>(at);
+        at += bwd_pd_bytes(H, pairs);
+        float *dl_t = reinterpret_cast<float *>(at);
+        at += bwd_dlt_bytes(H, pairs);
+        a.pd = pd;
+        a.dl_t = dl_t;
+        pr.f.q = q; pr.f.k = k; pr.f.v = v;
+        pr.f.row_stride = static_cast<int64_t>(H) * D;
+        pr.f.table_q = table_q; pr.f.table_k = table_k; pr.f.table_v = table_v;
+        pr.f.w_sizes = w_sizes; pr.f.w2n = w2n; pr.f.n2n = n2n;
+        pr.f.n_coords = n_coords;
+        pr.f.workspace = at;
+        pr.f.H = H; pr.f.D = D; pr.f.nd = nd; pr.f.total_rows = a.total_rows;
+        pr.f.N = N; pr.f.W = W;
+        for (int n = 0; n < kMaxAxes; ++n) { pr.f.rows[n] = a.rows[n]; pr.f.base[n] = a.base[n]; }
+        pr.dout = dout;
+        pr.stat_max = out_max; pr.stat_sum = out_sum; pr.delta = a.delta;
+        pr.dq = dq; pr.dk = dk; pr.dv = dv;
+        pr.pos_base = a.pos_base;
+        pr.pd = pd; pr.dl_t = dl_t; pr.pairs = pairs;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (N == 0 || W == 0) {
         // nothing to differentiate: the table gradients are zero
@@ -752,7 +1091,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     }
 #define S3D_BWD_CASE(DD, NN)                                                              \
     if (D == DD && nd == NN)                                                              \
-        return dtype == S3D_DTYPE_F16 ? launch_bwd<__half, DD, NN>(a, s) : launch_bwd<float, DD, NN>(a, s);
+        return dtype == S3D_DTYPE_F16 ? launch_bwd<__half, DD, NN>(a, pr, dtype, s) : launch_bwd<float, DD, NN>(a, pr, dtype, s);
     S3D_BWD_CASE(8, 3) S3D_BWD_CASE(8, 6) S3D_BWD_CASE(8, 9)
     S3D_BWD_CASE(16, 3) S3D_BWD_CASE(16, 6) S3D_BWD_CASE(16, 9)
 #undef S3D_BWD_CASE

@@ -686,6 +686,264 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
     }
 }
 
+// ---- backward: the pair sweeps ------------------------------------------------------------------------------
+// dq, dk, dv of the attention backward (Swin3D/src/attn/self_attn_aio_bwd.cu:197-509 adds every term with a global
+// atomic) on the forward's work list: a lane owns one voxel of some window and streams the window's other side,
+//   kKeyOwned = false: lane = query i, streams the keys j:    dq_i += dL (k_j + Tq(i,j))
+//   kKeyOwned = true:  lane = key j, streams the queries i:   dk_j += dL (q_i + Tk(i,j)),  dv_j += P dout_i
+// with P = exp(L - max_i) / sum_i from the forward's saved statistics, dP = dout_i . (v_j + Tv(i,j)) and
+// dL = P (dP - dout_i . o_i).  Every gradient row has one owner and is stored once.  The sweeps also leave dL and
+// P of every (pair, head) for the table-gradient kernels, each in the order its reader wants: the key-owned sweep
+// writes (dL, P) at [head][pairs before the window + i n + j], the query-owned sweep dL at [.. + j n + i] - in both
+// the lanes of a window write consecutive addresses.
+template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_threads() { return 256; }
+
+template <typename T, int D, int ND, int HP, bool kKeyOwned>
+__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>())) void attn_bwd_pairs_kernel(BwdPairArgs b)
+{
+    const AttnArgs &a = b.f;
+    constexpr int kThreads = bwd_pair_threads<T, D, HP>();
+    extern __shared__ __align__(16) float smem[];
+    __shared__ __align__(16) int group_exit_counter[4];
+    int &group_exited = group_exit_counter[0];
+    if (threadIdx.x == 0) group_exited = 0;
+    const int H = a.H;
+    const int HD = H * D;
+    const int hg = a.spread_groups ? blockIdx.x % (H / HP) : (blockIdx.x / kQueues) % (H / HP);
+    const int h = hg * HP;
+    constexpr int kRowStride = table_row_stride_heads<T, D, HP>();
+    T *tab = reinterpret_cast<T *>(smem);
+    {
+        const T *gq = static_cast<const T *>(a.table_q);
+        const T *gk = static_cast<const T *>(a.table_k);
+        const T *gv = static_cast<const T *>(a.table_v);
+        constexpr int kPieces = D * static_cast<int>(sizeof(T)) / 16;
+        constexpr int kPerPiece = 16 / static_cast<int>(sizeof(T));
+        for (int t = threadIdx.x; t < a.total_rows * HP * kPieces; t += kThreads) {
+            const int r = t / (HP * kPieces), hp = t - r * (HP * kPieces);
+            const int hh = hp / kPieces, c = (hp - hh * kPieces) * kPerPiece;
+            const int64_t g = static_cast<int64_t>(r) * HD + (h + hh) * D + c;
+            T *row = tab + r * kRowStride + hh * 3 * D + c;
+            *reinterpret_cast<uint4 *>(row) = *reinterpret_cast<const uint4 *>(gq + g);
+            *reinterpret_cast<uint4 *>(row + D) = *reinterpret_cast<const uint4 *>(gk + g);
+            *reinterpret_cast<uint4 *>(row + 2 * D) = *reinterpret_cast<const uint4 *>(gv + g);
+        }
+    }
+    __syncthreads();   // the only workgroup barrier
+
+    const int lane = threadIdx.x & 63;
+    const T *gq = static_cast<const T *>(a.q);
+    const T *gk = static_cast<const T *>(a.k);
+    const T *gv = static_cast<const T *>(a.v);
+    const T *ggo = static_cast<const T *>(b.dout);
+    const char *ws = static_cast<const char *>(a.workspace);
+    const int4 *unit_info = reinterpret_cast<const int4 *>(ws + ws_units_offset(H));
+    const int4 *entries = reinterpret_cast<const int4 *>(ws + ws_entries_offset(H, a.N));
+    const int total_units = __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(ws + ws_total_offset(H))[0]);
+    int *counters = static_cast<int *>(a.workspace) + hg * kQueues * kCounterStride;
+    constexpr int kRowBytes = kRowStride * static_cast<int>(sizeof(T));
+    constexpr uint32_t kHeadBytes = 3 * D * sizeof(T);
+    const uint32_t tab_addr = __builtin_amdgcn_readfirstlane(lds_address(tab));
+    const uint32_t row_bytes = kRowBytes;
+    float half_rows[ND], upper[ND];
+    uint32_t base_off[ND];
+#pragma unroll
+    for (int n = 0; n < ND; ++n) {
+        half_rows[n] = static_cast<float>(a.rows[n] / 2);
+        upper[n] = crse_upper(a.rows[n]);
+        base_off[n] = __builtin_amdgcn_readfirstlane(tab_addr + a.base[n] * kRowBytes);
+    }
+    // the one table-row sum that enters the owned gradient as a vector (Tq for dq_i, Tk for dk_j) sits behind the
+    // q-side slice in the query-owned sweep and behind the k-side slice in the key-owned one
+    constexpr uint32_t kVecSlice = kKeyOwned ? D * sizeof(T) : 0;
+
+    int queue = xcd_id() % kQueues;
+    int tried = 0;
+    int drawn = 0;
+    if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+    for (;;) {
+        int unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        while (unit >= total_units && ++tried < kQueues) {
+            queue = (queue + 1) % kQueues;
+            if (lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+            unit = __builtin_amdgcn_readfirstlane(drawn) * kQueues + queue;
+        }
+        if (unit >= total_units) break;
+        // the unit, as in the forward sweep: 64 >> gshift owned voxels, each on 2^gshift adjacent lanes that take
+        // alternate elements of the streamed side
+        const int4 info = unit_info[unit];
+        const int first = __builtin_amdgcn_readfirstlane(info.x);
+        const int gshift = __builtin_amdgcn_readfirstlane(info.y);
+        const int owners = __builtin_amdgcn_readfirstlane(info.w);
+        const int sub = lane & ((1 << gshift) - 1);
+        const bool own_valid = (lane >> gshift) < owners;
+        const int slot = __builtin_amdgcn_readfirstlane(info.z) + min(lane >> gshift, owners - 1);
+        const int4 seen = entries[first + lane];
+        const int seen_from = seen.w == __builtin_amdgcn_readfirstlane(seen.w) ? seen.x : 0x7fffffff;
+        int at = 0;
+#pragma unroll
+        for (int half = 32; half > 0; half >>= 1)
+            if (__shfl(seen_from, at + half) <= slot) at += half;
+        const int n_w = __shfl(seen.y, at), s0 = __shfl(seen.z, at);
+        const int own_in = slot - __shfl(seen.x, at);     // position inside the window
+        const int own_pos = s0 + own_in;
+        const int own_row = a.n2n[own_pos];
+        int max_steps = (n_w + (1 << gshift) - 1) >> gshift;
+#pragma unroll
+        for (int other = 32; other > 0; other >>= 1) max_steps = max(max_steps, __shfl_xor(max_steps, other));
+        max_steps = __builtin_amdgcn_readfirstlane(max_steps);
+        // pairs before the window; a window that does not fit the caller's pair store is skipped as a whole
+        const int64_t pair_base = b.pos_base[s0];
+        const bool fits = pair_base + static_cast<int64_t>(n_w) * n_w <= b.pairs;
+
+        Slice<T, D> own_x[HP], own_y[HP];     // q_i, dout_i  or  k_j, v_j
+        float own_m[HP], own_inv[HP], own_delta[HP];
+        float ci[ND], res_x[HP][D], res_y[kKeyOwned ? HP : 1][D];
+#pragma unroll
+        for (int hh = 0; hh < HP; ++hh) {
+            const int64_t at_row = static_cast<int64_t>(own_row) * HD + (h + hh) * D;
+            if constexpr (kKeyOwned) {
+                own_x[hh].load(gk + at_row);
+                own_y[hh].load(gv + at_row);
+            } else {
+                own_x[hh].load(gq + at_row);
+                own_y[hh].load(ggo + at_row);
+                own_m[hh] = b.stat_max[static_cast<int64_t>(own_row) * H + h + hh];
+                own_inv[hh] = 1.0f / b.stat_sum[static_cast<int64_t>(own_row) * H + h + hh];
+                own_delta[hh] = b.delta[static_cast<int64_t>(own_row) * H + h + hh];
+            }
+#pragma unroll
+            for (int c = 0; c < D; ++c) res_x[hh][c] = 0.0f;
+            if constexpr (kKeyOwned) {
+#pragma unroll
+                for (int c = 0; c < D; ++c) res_y[hh][c] = 0.0f;
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < ND; ++n) ci[n] = a.n_coords[static_cast<int64_t>(own_pos) * ND + n];
+
+        int row_next = a.n2n[s0 + min(sub, n_w - 1)];
+        for (int it = 0; it < max_steps; ++it) {
+            if (it + 1 >= max_steps && lane == 0) drawn = atomicAdd(counters + queue * kCounterStride, 1);
+            const int st = (it << gshift) + sub;
+            const bool valid = st < n_w && own_valid && fits;
+            const int st_in = min(st, n_w - 1);
+            const int st_pos = s0 + st_in;
+            const int st_row = row_next;
+            row_next = a.n2n[s0 + min(st + (1 << gshift), n_w - 1)];
+            Slice<T, D> st_x[HP], st_y[HP];   // k_j, v_j  or  q_i, dout_i
+            float st_m[HP], st_inv[HP], st_delta[HP];
+#pragma unroll
+            for (int hh = 0; hh < HP; ++hh) {
+                const int64_t at_row = static_cast<int64_t>(st_row) * HD + (h + hh) * D;
+                if constexpr (kKeyOwned) {
+                    st_x[hh].load(gq + at_row);
+                    st_y[hh].load(ggo + at_row);
+                    st_m[hh] = b.stat_max[static_cast<int64_t>(st_row) * H + h + hh];
+                    st_inv[hh] = b.stat_sum[static_cast<int64_t>(st_row) * H + h + hh];
+                    st_delta[hh] = b.delta[static_cast<int64_t>(st_row) * H + h + hh];
+                } else {
+                    st_x[hh].load(gk + at_row);
+                    st_y[hh].load(gv + at_row);
+                }
+            }
+            uint32_t off[ND];
+            {
+                float cj[ND];
+#pragma unroll
+                for (int n = 0; n < ND; ++n) cj[n] = a.n_coords[static_cast<int64_t>(st_pos) * ND + n];
+#pragma unroll
+                for (int n = 0; n < ND; ++n) {
+                    // row_n(i, j): the query's coordinate first
+                    const float c_i = kKeyOwned ? cj[n] : ci[n], c_j = kKeyOwned ? ci[n] : cj[n];
+                    off[n] = mad_u24(static_cast<uint32_t>(crse_row(c_i, c_j, half_rows[n], upper[n])), row_bytes, base_off[n]);
+                }
+            }
+#pragma unroll
+            for (int hh = 0; hh < HP; ++hh) {
+                const Slice<T, D> &qv = kKeyOwned ? st_x[hh] : own_x[hh];
+                const Slice<T, D> &kv = kKeyOwned ? own_x[hh] : st_x[hh];
+                const Slice<T, D> &vv = kKeyOwned ? own_y[hh] : st_y[hh];
+                const Slice<T, D> &gov = kKeyOwned ? st_y[hh] : own_y[hh];
+                float logit = qv.dot(kv, 0.0f);
+                float dp = gov.dot(vv, 0.0f);
+                // sums of three rows of the table that enters the owned gradient as a vector (packed fp16 adds for
+                // fp16 I/O, as the forward adds its value-table rows)
+                constexpr int kGroup = 3;
+                Slice<T, D> vec_sum[(ND + kGroup - 1) / kGroup];
+#pragma unroll
+                for (int n = 0; n < ND; ++n) {
+                    Slice<T, D> tq_r, tk_r, tv_r;
+                    tq_r.load_lds(off[n] + hh * kHeadBytes);
+                    tk_r.load_lds(off[n] + hh * kHeadBytes + D * sizeof(T));
+                    tv_r.load_lds(off[n] + hh * kHeadBytes + 2 * D * sizeof(T));
+                    if (Slice<T, D>::kChainLogit) logit = kv.dot(tk_r, qv.dot(tq_r, logit));
+                    else logit += kv.dot(tk_r, qv.dot(tq_r, 0.0f));
+                    if (Slice<T, D>::kChainLogit) dp = gov.dot(tv_r, dp);
+                    else dp += gov.dot(tv_r, 0.0f);
+                    const Slice<T, D> &vec_r = kKeyOwned ? tk_r : tq_r;
+                    if (n % kGroup == 0) vec_sum[n / kGroup] = vec_r;
+                    else vec_sum[n / kGroup].add(vec_r);
+                }
+                const float m_i = kKeyOwned ? st_m[hh] : own_m[hh];
+                const float inv_i = kKeyOwned ? 1.0f / st_inv[hh] : own_inv[hh];
+                const float delta_i = kKeyOwned ? st_delta[hh] : own_delta[hh];
+                const float p = valid ? __expf(logit - m_i) * inv_i : 0.0f;
+                const float dl = p * (dp - delta_i);
+                // dq_i += dL (k_j + Tq)   or   dk_j += dL (q_i + Tk)
+                st_x[hh].fma_to(res_x[hh], dl);
+#pragma unroll
+                for (int g = 0; g < (ND + kGroup - 1) / kGroup; ++g) vec_sum[g].fma_to(res_x[hh], dl);
+                if constexpr (kKeyOwned) st_y[hh].fma_to(res_y[hh], p);     // dv_j += P dout_i
+                if (valid) {
+                    const int64_t head_at = static_cast<int64_t>(h + hh) * b.pairs + pair_base;
+                    if constexpr (kKeyOwned) b.pd[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = make_float2(dl, p);
+                    else b.dl_t[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = dl;
+                }
+            }
+        }
+#pragma unroll
+        for (int hh = 0; hh < HP; ++hh) {
+            // lanes that share an owned voxel saw alternate elements of the stream
+            for (int other = 1; other < (1 << gshift); other <<= 1) {
+#pragma unroll
+                for (int c = 0; c < D; ++c) res_x[hh][c] += __shfl_xor(res_x[hh][c], other);
+                if constexpr (kKeyOwned) {
+#pragma unroll
+                    for (int c = 0; c < D; ++c) res_y[hh][c] += __shfl_xor(res_y[hh][c], other);
+                }
+            }
+            if (own_valid && sub == 0 && fits) {
+                const int64_t at_row = static_cast<int64_t>(own_row) * HD + (h + hh) * D;
+                if constexpr (kKeyOwned) {
+                    store_row<D>(static_cast<T *>(b.dk) + at_row, res_x[hh]);
+                    store_row<D>(static_cast<T *>(b.dv) + at_row, res_y[hh]);
+                } else {
+                    store_row<D>(static_cast<T *>(b.dq) + at_row, res_x[hh]);
+                }
+            }
+        }
+    }
+    // the last wavefront of the launch to leave puts the queue counters back to zero (as in the forward sweep):
+    // the next sweep runs on the same list
+    if (lane == 0 && atomicAdd(&group_exited, 1) == kThreads / 64 - 1) {
+        __threadfence();
+        int *total = static_cast<int *>(a.workspace) + ws_total_offset(H) / sizeof(int);
+        const int groups = static_cast<int>(gridDim.x), line = static_cast<int>(blockIdx.x) % kQueues;
+        const int on_line = (groups - line + kQueues - 1) / kQueues;
+        int *line_counter = total + (1 + line) * kCounterStride;
+        if (atomicAdd(line_counter, 1) == on_line - 1) {
+            *line_counter = 0;
+            if (atomicAdd(total + 1, 1) == min(groups, kQueues) - 1) {
+                total[1] = 0;
+                int *all_counters = static_cast<int *>(a.workspace);
+                for (int t = 0; t < H * kQueues; ++t) all_counters[t * kCounterStride] = 0;
+                __threadfence();
+            }
+        }
+    }
+}
+
 template <typename T, int D, int ND, int HP, bool kSorted>
 int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
 {
@@ -770,6 +1028,87 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream, int what)
 }
 
 }  // namespace
+
+namespace {
+
+template <typename T, int D, int ND, int HP>
+int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
+{
+    const AttnArgs &a = b0.f;
+    const size_t lds = align_up(sizeof(T) * static_cast<size_t>(a.total_rows) * table_row_stride_heads<T, D, HP>(), 16);
+    if (lds > 160 * 1024)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
+                    a.total_rows, D, lds);
+    auto q_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, false>;
+    auto k_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, true>;
+    constexpr int kThreads = bwd_pair_threads<T, D, HP>();
+    int per_cu = 1;
+    for (auto kernel : {q_sweep, k_sweep}) {
+        S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    }
+    {
+        // workgroups per CU: what the registers of the heavier sweep and the tables in LDS allow
+        int fit_q = 0, fit_k = 0;
+        S3D_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit_q, reinterpret_cast<const void *>(q_sweep), kThreads, lds));
+        S3D_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit_k, reinterpret_cast<const void *>(k_sweep), kThreads, lds));
+        per_cu = fit_q < fit_k ? fit_q : fit_k;
+        if (per_cu < 1) per_cu = 1;
+    }
+    const int groups = a.H / HP;
+    const int cus = device_cus();
+    const int slots = per_cu * cus;
+    const int set = kQueues * groups;
+    const int whole = (slots / set) * set;
+    BwdPairArgs b = b0;
+    b.f.spread_groups = 10 * whole < 9 * slots;
+    const int grid = b.f.spread_groups ? (slots >= groups ? slots / groups * groups : groups) : whole;
+    b.f.target_items = grid / groups * (kThreads / 64);
+    b.f.block_shift = target_shift_for(a.N, a.W, b.f.target_items);
+    const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
+    const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
+    hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
+    hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
+    S3D_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(q_sweep, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, stream, b);
+    hipLaunchKernelGGL(k_sweep, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, stream, b);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+template <typename T, int D, int ND>
+int launch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
+{
+    // two heads per wavefront where the registers allow it: fp16 at head_dim 8
+#ifdef S3D_BWD_PAIR_HEADS2
+    if constexpr (sizeof(T) == 2 && D == 8) {
+        if (b.f.H % 2 == 0) return launch_bwd_pairs_heads<T, D, ND, 2>(b, stream);
+    }
+#endif
+    return launch_bwd_pairs_heads<T, D, ND, 1>(b, stream);
+}
+
+template <typename T>
+int dispatch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
+{
+#define S3D_CASE(DD, NN) \
+    if (b.f.D == DD && b.f.nd == NN) return launch_bwd_pairs<T, DD, NN>(b, stream);
+    S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
+    S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
+#undef S3D_CASE
+    return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: unsupported head_dim %d / cRSE axes %d", b.f.D, b.f.nd);
+}
+
+}  // namespace
+
+int launch_attn_bwd_pairs(const BwdPairArgs &b, int dtype, hipStream_t stream)
+{
+    switch (dtype) {
+    case S3D_DTYPE_F32: return dispatch_bwd_pairs<float>(b, stream);
+    case S3D_DTYPE_F16: return dispatch_bwd_pairs<__half>(b, stream);
+    default: return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    }
+}
 
 size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N)
 {

@@ -41,6 +41,20 @@ size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N);
 constexpr int kAttnBuildList = 1, kAttnSweep = 2;
 int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int what = kAttnBuildList | kAttnSweep);
 
+// The pair sweeps of the backward on the sweep kernel's work list (built here, in b.f.workspace, which needs
+// attn_generic_workspace_bytes): dq, dk, dv, and dL, P of every (pair, head) for the table-gradient kernels.
+struct BwdPairArgs {
+    AttnArgs f;                  // shape, q, k, v, tables, index arrays (n2n required), rows[] / base[], workspace
+    const void *dout;            // [N,H,D]
+    const float *stat_max, *stat_sum, *delta;   // [N,H]: the forward's statistics, dout_i . o_i
+    void *dq, *dk, *dv;          // [N,H,D]
+    const int64_t *pos_base;     // [N]: at a window's first sorted position, the pairs of the windows before it
+    float2 *pd;                  // [H][pairs]: (dL, P) at base + i n + j  (i, j: query, key position inside the window)
+    float *dl_t;                 // [H][pairs]: dL at base + j n + i
+    int64_t pairs;               // capacity of pd and dl_t per head; windows beyond it are skipped
+};
+int launch_attn_bwd_pairs(const BwdPairArgs &b, int dtype, hipStream_t stream);
+
 // One wavefront per window, MFMA products + LDS gathers; fp16 only.
 bool attn_mfma_supported(const AttnArgs &a, int dtype);
 // the shapes where it is the faster of the two kernels: head_dim 16 with full windows, 300 voxels or more on

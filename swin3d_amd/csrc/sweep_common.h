@@ -116,6 +116,12 @@ template <int D> struct Slice<float, D> {
 #pragma unroll
         for (int c = 0; c < D; ++c) acc[c] += p * x[c];
     }
+    // x += o
+    __device__ __forceinline__ void add(const Slice &o)
+    {
+#pragma unroll
+        for (int c = 0; c < D; ++c) x[c] += o.x[c];
+    }
     // acc + sum_c x[c] * y[c]
     __device__ __forceinline__ float dot_f32(const float *y, float acc) const
     {

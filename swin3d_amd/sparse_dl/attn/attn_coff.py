@@ -43,6 +43,10 @@ class PrecisionMode(enum.Enum):
 
 _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_F16}
 
+# the backward keeps dL and P of every (pair, head) in its workspace when the window set's pair count is known
+# (window_attention_backward): switch, and the size above which it runs the fused sweeps instead
+BWD_PAIR_STORE = True
+BWD_PAIR_STORE_MAX_BYTES = 32 << 30
 # s3d_attn_bwd keeps a head's table gradients in registers: at most 64 rows per axis on average, head_dim 8 or 16
 # (the forward also takes head_dim 32)
 BWD_MAX_ROWS_PER_AXIS = 64
@@ -278,11 +282,30 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     return out
 
 
+def _pairs_of(w_sizes_in, w_sizes):
+    """M = sum of w_sizes^2, the pairs of the window set (one host read, kept on the caller's tensor)."""
+    if isinstance(w_sizes_in, torch.Tensor):
+        kept = getattr(w_sizes_in, "_s3d_pairs", None)
+        if kept is not None and kept[0] == w_sizes_in._version:
+            return kept[1]
+    pairs = int((w_sizes.long() ** 2).sum().item()) if w_sizes.numel() else 0
+    if isinstance(w_sizes_in, torch.Tensor):
+        w_sizes_in._s3d_pairs = (w_sizes_in._version, pairs)
+    return pairs
+
+
 def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n, n_coords,
-                              out, out_max, out_sum, dout):
+                              out, out_max, out_sum, dout, pairs=None):
     """Gradients of window_attention_forward -> (dq, dk, dv [N,H,D] in the dtype of q,
     dtable_q, dtable_k, dtable_v flat fp32).  out / out_max / out_sum are the forward's results
-    (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes."""
+    (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes.
+
+    pairs: M = sum(w_sizes^2) of the window set (the reference's index arrays have this length,
+    swin3d_layers.py:96-103); None = read it from w_sizes once and keep it on that tensor.  With it the library
+    runs the pair sweeps, which keep dL and P of every (pair, head) in the workspace (12 bytes each); 0, or a
+    store above BWD_PAIR_STORE_MAX_BYTES, selects the fused sweeps, which need no such store and take about
+    twice as long."""
+    w_sizes_in = w_sizes
     _require_cuda("query", q)
     dev = q.device
     if q.dim() != 3:
@@ -326,15 +349,22 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     lib = _lib.lib()
     tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
     out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
+    if pairs is None:
+        pairs = _pairs_of(w_sizes_in, w_sizes) if BWD_PAIR_STORE else 0
+    pairs = int(pairs)
+    if pairs < 0:
+        raise ValueError(f"pairs = {pairs}")
+    if 12 * pairs * h > BWD_PAIR_STORE_MAX_BYTES:
+        pairs = 0
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, n, w_sizes.numel())
+        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, n, w_sizes.numel(), pairs)
         workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
         status = lib.s3d_attn_bwd(
             *(t.data_ptr() for t in tensors), c_sizes, nd, table_len, w_sizes.data_ptr(), w2n.data_ptr(),
             n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(), out_max.data_ptr(), out_sum.data_ptr(),
             dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dtq.data_ptr(), dtk.data_ptr(),
-            dtv.data_ptr(), n, h, d, w_sizes.numel(), _DTYPE_CODE[q.dtype], workspace.data_ptr(), ws_bytes,
+            dtv.data_ptr(), n, h, d, w_sizes.numel(), pairs, _DTYPE_CODE[q.dtype], workspace.data_ptr(), ws_bytes,
             stream)
     _lib.check(status, "s3d_attn_bwd")
     return dq, dk, dv, dtq, dtk, dtv

@@ -1,4 +1,5 @@
-"""GPU parity of the window attention backward (HIP through the C ABI) against the float64 CPU oracle.
+"""GPU parity of the window attention backward (HIP through the C ABI) against the float64 CPU oracle, on both
+of its paths (with and without the window set's pair count).
 
 Tolerance: |got - ref| <= rel * scale with rel = 2e-5 for fp32 and 3e-3 for fp16 (fp16: the forward output
 o that enters dout.o, and dq / dk / dv themselves, are rounded to fp16); scale = largest |ref| over
@@ -15,7 +16,7 @@ pytestmark = pytest.mark.gpu
 NAMES = ("dq", "dk", "dv", "dtable_q", "dtable_k", "dtable_v")
 
 
-def _run(case, dout, dtype):
+def _run(case, dout, dtype, pairs=None):
     import swin3d_amd
     dev = torch.device("cuda")
     t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
@@ -24,7 +25,7 @@ def _run(case, dout, dtype):
     args = (f(case.q), f(case.k), f(case.v), f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
             t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
     out, omax, osum = swin3d_amd.window_attention_forward(*args, return_stats=True)
-    grads = swin3d_amd.window_attention_backward(*args, out, omax, osum, f(dout))
+    grads = swin3d_amd.window_attention_backward(*args, out, omax, osum, f(dout), pairs=pairs)
     torch.cuda.synchronize()
     return [g.double().cpu().numpy() for g in grads]
 
@@ -50,7 +51,10 @@ def _check(oracle_lib, case, dtype, seed=0, dout_scale=1.0):
     if dtype == torch.float16:
         dout = dout.astype(np.float16).astype(np.float32)
     ref = oracle_lib.attn_bwd(*case.oracle_args(), dout)
+    # both ways through s3d_attn_bwd: the pair sweeps with their store of dL and P (the pair count from w_sizes),
+    # and the fused sweeps that run when the caller gives no pair count
     _assert_close(_run(case, dout, dtype), ref, dtype)
+    _assert_close(_run(case, dout, dtype, pairs=0), ref, dtype)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
@@ -264,3 +268,24 @@ def test_repeated_calls(oracle_lib, hip_lib, dtype):
             assert torch.equal(a, b)
         for a, b in zip(first[3:], again[3:]):
             assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max())
+
+
+def test_pair_count_larger_than_needed(oracle_lib, hip_lib):
+    """pairs is a capacity: a store larger than the window set's sum of squares gives the same gradients."""
+    import swin3d_amd
+    case = make_attn_case(oracle_lib, seed=78, n=3000, ws=5, quant=4, heads=6, dim=8, extent=(16, 16, 8), recipe="layer")
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    feats = [t(x).half() for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
+    idx = [t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)]
+    sizes = [int(x) for x in case.table_sizes]
+    out, mx, sm = swin3d_amd.window_attention_forward(*feats, sizes, *idx, return_stats=True)
+    dout = torch.randn_like(out)
+    m = int((idx[0].long() ** 2).sum())
+    exact = swin3d_amd.window_attention_backward(*feats, sizes, *idx, out, mx, sm, dout, pairs=m)
+    roomy = swin3d_amd.window_attention_backward(*feats, sizes, *idx, out, mx, sm, dout, pairs=m + 12345)
+    for a, b in zip(exact[:3], roomy[:3]):
+        assert torch.equal(a, b)
+    for a, b in zip(exact[3:], roomy[3:]):
+        assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max())
