@@ -123,7 +123,7 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
     auto class_of = [](int n) { return n > 256 ? 0 : n > 128 ? 1 : n > 64 ? 2 : n > 32 ? 3 : n > 16 ? 4 : 5; };
     __shared__ int wave_sum[16][kClasses];
     __shared__ int class_start[kClasses + 1];
-    __shared__ long long pairs_before[1024];   // pairs (n^2) of the windows of the threads before this one
+    __shared__ long long wave_pairs[16];       // pairs (n^2) of the windows of each wavefront's threads
     const int W = static_cast<int>(a.W);
     const int per = (W + 1023) / 1024;
     const int begin = min(static_cast<int>(threadIdx.x) * per, W), end = min(begin + per, W);
@@ -138,8 +138,13 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
         for (int c = 0; c < kClasses; ++c) mine[c] += c == cls ? chunks : 0;
         pairs_mine += static_cast<long long>(n) * n;
     }
-    pairs_before[threadIdx.x] = pairs_mine;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    long long pairs_incl = pairs_mine;
+    for (int off = 1; off < 64; off <<= 1) {
+        const long long up = __shfl_up(pairs_incl, off);
+        if (lane >= off) pairs_incl += up;
+    }
+    if (lane == 63) wave_pairs[wave] = pairs_incl;
     int incl[kClasses];
 #pragma unroll
     for (int c = 0; c < kClasses; ++c) {
@@ -163,16 +168,16 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
         }
         class_start[kClasses] = run;
         long long before = 0;
-        for (int t = 0; t < 1024; ++t) {
-            const long long add = pairs_before[t];
-            pairs_before[t] = before;
+        for (int v = 0; v < 16; ++v) {
+            const long long add = wave_pairs[v];
+            wave_pairs[v] = before;
             before += add;
         }
     }
     __syncthreads();
     {
         // where the (pair, head) records of a window start in the pair store: written at the window's first position
-        long long before = pairs_before[threadIdx.x];
+        long long before = wave_pairs[wave] + pairs_incl - pairs_mine;
         for (int w = begin; w < end; ++w) {
             const int n = a.w_sizes[w];
             if (n > 0) a.pos_base[a.w2n[w]] = before;
@@ -562,15 +567,21 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 
 // Table gradients from the dL and P that the pair sweeps left for every (pair, head): the histogram and rank-1
 // machinery of the sweeps above without their logits, table rows and owned gradients.
-//   KEY_OWNED: lanes = keys j of a 64-key chunk, the window's queries stream:  dTq += hist(dL) x q_i,  dTv += hist(P) x dout_i
-//   else:      lanes = queries i, the keys stream:                              dTk += hist(dL) x k_j
+//   KIND 0: lanes = queries i of a 64-voxel chunk, the window's keys stream:   dTk += hist(dL) x k_j
+//   KIND 1: lanes = keys j, the queries stream:   dTq += hist(dL) x q_i  and  dTv += hist(P) x dout_i
+//   KIND 2, 3: the two halves of KIND 1 as kernels of their own (dTq; dTv), for the shapes where both sets of
+//           accumulators leave one wavefront per SIMD
 // A step's inputs - the lane's record, the streamed rows and coordinates - are fetched one step ahead: the records
 // come from HBM and a step is a short dependent chain (rows, histogram atomics, read-back), so their latency would
 // be most of it.
-template <typename T, int D, int ND, bool KEY_OWNED, int BLK>
-__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) void attn_bwd_tables_kernel(BwdArgs a)
+// Wavefronts per SIMD: two for KIND 1 at head_dim 8 (80 accumulators; capped at 168 registers for three it spills
+// and measured 1.7x the time), three for the one-table kinds; at head_dim 16 one, and two for the halves.
+template <typename T, int D, int ND, int KIND, int BLK>
+__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND >= 2 ? 2 : 1))) void attn_bwd_tables_kernel(BwdArgs a)
 {
-    constexpr bool kAccB = KEY_OWNED;                          // dTv
+    constexpr bool KEY_OWNED = KIND != 0;
+    constexpr bool kAccB = KIND == 1;                          // two histograms and two sets of accumulators
+    constexpr bool kFromP = KIND == 3;                         // the one histogram is of P, the vector dout_i
     constexpr int kHistKinds = 1 + (kAccB ? 1 : 0);
     constexpr int kFlat = BLK * 64;
     // A histogram cell exists in kCopies copies, chosen by the low bits of the lane number: lanes that hit the
@@ -590,14 +601,15 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
     const int lane = threadIdx.x & 63;
     int *hist_a = hist_all + wave * kHistWords;
     unsigned long long *hist_ab = reinterpret_cast<unsigned long long *>(hist_a);
-    const T *gx = static_cast<const T *>(KEY_OWNED ? a.q : a.k);      // the streamed row of the first rank-1 update
-    const T *gy = static_cast<const T *>(a.dout);                     // ... of the second (key-owned)
+    // the streamed row of the first rank-1 update (k_j, q_i or, for the dTv half, dout_i) and of the second (KIND 1)
+    const T *gx = static_cast<const T *>(KIND == 0 ? a.k : KIND == 3 ? a.dout : a.q);
+    const T *gy = static_cast<const T *>(a.dout);
 
     // The rank-1 updates as 4x4x1 MFMAs wherever the VALU form would not fit the registers: the accumulators may
     // then live in accumulation registers.  Measured at head_dim 8 (us, VALU / MFMA form): fp16 with five 64-row
     // blocks 658 / 1017 key-owned and 387 / 510 query-owned; six blocks 1804 / 817 and 843 / 508 (the VALU form
     // spills); fp32 with five blocks 1256 / 644 and 384 / 380.
-    constexpr bool kMfmaUpdate = D > 8 || BLK > 5 || (KEY_OWNED && sizeof(T) == 4);
+    constexpr bool kMfmaUpdate = D > 8 || BLK > 5 || (KIND == 1 && sizeof(T) == 4);
     float acc_a[BLK][D], acc_b[kAccB ? BLK : 1][D];
 #pragma unroll
     for (int m = 0; m < BLK; ++m)
@@ -673,7 +685,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
         auto fetch = [&](int it, int st_row, StepIn &in) {
             const int st = min(it * ng + grp, n_w - 1);
             in.x.load(gx + static_cast<int64_t>(st_row) * HD + h * D);
-            if constexpr (KEY_OWNED) in.y.load(gy + static_cast<int64_t>(st_row) * HD + h * D);
+            if constexpr (kAccB) in.y.load(gy + static_cast<int64_t>(st_row) * HD + h * D);
 #pragma unroll
             for (int n = 0; n < ND; ++n) in.c[n] = a.n_coords[static_cast<int64_t>(s0 + st) * ND + n];
         };
@@ -684,7 +696,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
             const int st = min(it * ng + grp, n_w - 1);
             const int64_t rec_at = rec_base + static_cast<int64_t>(st) * rec_stride;
             float2 rec = make_float2(0.0f, 0.0f);
-            if constexpr (KEY_OWNED) rec = a.pd[rec_at];
+            if constexpr (KIND == 1) rec = a.pd[rec_at];
+            else if constexpr (KIND == 2) rec.x = a.pd[rec_at].x;
+            else if constexpr (KIND == 3) rec.x = a.pd[rec_at].y;
             else rec.x = a.dl_t[rec_at];
             return rec;
         };
@@ -708,9 +722,11 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
                 row_after = a.n2n[s0 + min((it + 2) * ng + grp, n_w - 1)];
                 fetch(it + 1, row_next, next);
             }
+            // dl: the value of the first histogram (P for the dTv half, whose fixed-point scale is constant)
             const float dl = have ? rec.x : 0.0f, p = have ? rec.y : 0.0f;
-            const float amax = group_max_nonneg(fabsf(dl), ng == 2, grp);
-            const int qd = __float2int_rn(dl * (amax > 0.0f ? kFixL * __builtin_amdgcn_rcpf(amax) : 0.0f));
+            const float amax = kFromP ? 1.0f : group_max_nonneg(fabsf(dl), ng == 2, grp);
+            const int qd = kFromP ? __float2int_rn(dl * kFixP)
+                                  : __float2int_rn(dl * (amax > 0.0f ? kFixL * __builtin_amdgcn_rcpf(amax) : 0.0f));
             if constexpr (kAccB) {
                 const int qp = __float2int_rn(p * kFixP);
                 const unsigned long long both =
@@ -734,7 +750,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
             wave_lds_fence();
             for (int g = 0; g < ng; ++g) {
                 const int src = __builtin_amdgcn_readfirstlane(g * gs);
-                const float sc = lane_value(amax, src) * (1.0f / kFixL);
+                const float sc = kFromP ? 1.0f / kFixP : lane_value(amax, src) * (1.0f / kFixL);
                 const Slice<T, D> sx = cur.x.lane(src);
                 float bx[D / 4], by[D / 4];
                 if constexpr (kMfmaUpdate) sx.quad_channels(lane, bx);
@@ -765,7 +781,8 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KEY_OWNED ? 2 : 3) : 1)) vo
                         int4 *cell = reinterpret_cast<int4 *>(hist_a + (g * kFlat + m * 64 + lane) * kCopies);
                         const int4 four = *cell;
                         *cell = make_int4(0, 0, 0, 0);
-                        const float gsum = static_cast<float>(four.x + four.y + four.z + four.w) * sc;
+                        const int cells = four.x + four.y + four.z + four.w;
+                        const float gsum = (kFromP ? static_cast<float>(static_cast<unsigned>(cells)) : static_cast<float>(cells)) * sc;
                         if constexpr (kMfmaUpdate) mfma_update(acc_a[m], gsum, bx);
                         else sx.fma_to(acc_a[m], gsum);
                     }
@@ -867,12 +884,12 @@ int bwd_grid(int H, int per_cu = 2)
     return (per_cu * cus / set > 0 ? per_cu * cus / set : 1) * set;
 }
 
-template <typename T, int D, int ND, bool KEY_OWNED, int BLK>
+template <typename T, int D, int ND, int KIND, int BLK>
 int launch_tables_blk(const BwdArgs &a, int grid, hipStream_t stream)
 {
-    constexpr int kinds = KEY_OWNED ? 2 : 1;
-    auto kernel = attn_bwd_tables_kernel<T, D, ND, KEY_OWNED, BLK>;
-    constexpr int copies = KEY_OWNED ? 2 : 4;
+    constexpr int kinds = KIND == 1 ? 2 : 1;
+    auto kernel = attn_bwd_tables_kernel<T, D, ND, KIND, BLK>;
+    constexpr int copies = KIND == 1 ? 2 : 4;
     const size_t lds = sizeof(int) * kBwdWaves * kinds * 2 * static_cast<size_t>(BLK) * 64 * copies;
     S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
@@ -885,22 +902,23 @@ int launch_tables_blk(const BwdArgs &a, int grid, hipStream_t stream)
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
     const int threads = 2 * a.total_rows * a.H * a.D;
+    float *first = KIND == 0 ? a.dtk : KIND == 3 ? a.dtv : a.dtq;
     hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
-                       a, KEY_OWNED ? a.dtq : a.dtk, KEY_OWNED ? a.dtv : nullptr, BLK * 64, grid);
+                       a, first, KIND == 1 ? a.dtv : nullptr, BLK * 64, grid);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
 }
 
-template <typename T, int D, int ND, bool KEY_OWNED>
+template <typename T, int D, int ND, int KIND>
 int launch_tables(const BwdArgs &a, int grid, hipStream_t stream)
 {
     const int blocks = (a.total_rows + 63) / 64;
     constexpr int kSmall = 2 * ND / 3;
     if constexpr (ND == 9) {
-        if (blocks <= 5) return launch_tables_blk<T, D, ND, KEY_OWNED, 5>(a, grid, stream);
+        if (blocks <= 5) return launch_tables_blk<T, D, ND, KIND, 5>(a, grid, stream);
     }
-    if (blocks <= kSmall) return launch_tables_blk<T, D, ND, KEY_OWNED, kSmall>(a, grid, stream);
-    return launch_tables_blk<T, D, ND, KEY_OWNED, ND>(a, grid, stream);
+    if (blocks <= kSmall) return launch_tables_blk<T, D, ND, KIND, kSmall>(a, grid, stream);
+    return launch_tables_blk<T, D, ND, KIND, ND>(a, grid, stream);
 }
 
 // table-gradient registers for as many 64-row blocks as the head's flat table has: 5 for window 5 at four steps
@@ -931,8 +949,15 @@ int launch_bwd(const BwdArgs &a, const BwdPairArgs &pairs, int dtype, hipStream_
     if (a.pairs > 0) {
         // dq, dk, dv by the pair sweeps, which leave dL and P of every (pair, head); the table gradients from those
         if (int rc = launch_attn_bwd_pairs(pairs, dtype, stream)) return rc;
-        if (int rc = launch_tables<T, D, ND, true>(a, grid, stream)) return rc;
-        return launch_tables<T, D, ND, false>(a, grid, stream);
+        // head_dim 16: dTq and dTv as kernels of their own, two wavefronts per SIMD each instead of one for both
+        // (2.37 -> 2.27 ms at the 6-head window-7 layer; at head_dim 8 the split measured +8 %)
+        if constexpr (D > 8) {
+            if (int rc = launch_tables<T, D, ND, 2>(a, grid, stream)) return rc;
+            if (int rc = launch_tables<T, D, ND, 3>(a, grid, stream)) return rc;
+        } else {
+            if (int rc = launch_tables<T, D, ND, 1>(a, grid, stream)) return rc;
+        }
+        return launch_tables<T, D, ND, 0>(a, grid, stream);
     }
     // one key-owned sweep for dk, dv and both of its table gradients; at head_dim 16 with more than six 64-row
     // blocks of table rows (quant 8) the two sets of accumulation registers no longer fit one wavefront

@@ -1079,12 +1079,8 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
 template <typename T, int D, int ND>
 int launch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
 {
-    // two heads per wavefront where the registers allow it: fp16 at head_dim 8
-#ifdef S3D_BWD_PAIR_HEADS2
-    if constexpr (sizeof(T) == 2 && D == 8) {
-        if (b.f.H % 2 == 0) return launch_bwd_pairs_heads<T, D, ND, 2>(b, stream);
-    }
-#endif
+    // one head per wavefront: with two (fp16, head_dim 8) the key-owned sweep needs more than 256 registers and the
+    // pair of sweeps measured 0.3 ms slower at the 6-head layer
     return launch_bwd_pairs_heads<T, D, ND, 1>(b, stream);
 }
 

@@ -419,6 +419,9 @@ class SelfAttnAIOFunction(Function):
         out, omax, osum = res
         ctx.precision = precision
         ctx.table_sizes = _host_table_sizes(table_offsets)
+        # the window set's pair count, for the backward's pair store: on the tensor when the window index of this
+        # package built it, else read from w_sizes once (and kept on it)
+        ctx.pairs = _pairs_of(w_sizes, w_sizes) if BWD_PAIR_STORE else 0
         ctx.save_for_backward(out, omax, osum, *raw, w_sizes, w2n, n2n, n_coords)
         return out
 
@@ -436,7 +439,8 @@ class SelfAttnAIOFunction(Function):
         feats = [t.to(c_dtype).contiguous() for t in raw[:3]]
         tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
         grads = window_attention_backward(*feats, *tables, ctx.table_sizes, w_sizes, w2n, n2n, n_coords,
-                                          out.to(c_dtype), omax, osum, dout.to(c_dtype).contiguous())
+                                          out.to(c_dtype), omax, osum, dout.to(c_dtype).contiguous(),
+                                          pairs=ctx.pairs)
         grads = [g.to(t.dtype).reshape(t.shape) if need else None
                  for g, t, need in zip(grads, raw, ctx.needs_input_grad[:6])]
         return (*grads, None, None, None, None, None, None)

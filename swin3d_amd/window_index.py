@@ -88,6 +88,7 @@ def build_window_indices(coords, stride, window_size, shifts):
                              "-8192..8191)")
         sizes = w_sizes[:num_w]
         sizes.max_window_voxels = int(max_w)   # read by the attention op (the MFMA kernel sizes its partial results with it)
+        sizes._s3d_pairs = (sizes._version, int(num_m))   # ... and by its backward (the size of the pair store)
         result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window)))
     return result
 
