@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (0 = the library picks, 1 = sweep kernel, 2 = MFMA kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
+    ap.add_argument("--no-other-shapes", action="store_true",
+                    help="skip the window-7 layers of the side figures (a profile then holds the headline layer's kernels only)")
     ap.add_argument("--no-encoder", action="store_true",
                     help="skip the Swin3D-L encoder end-to-end latency")
     ap.add_argument("--window-ordered", action="store_true",
@@ -288,7 +290,8 @@ def main():
                        reps=5, warm=2)
         result["extras"]["attn_bwd"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3),
                                         "vs_forward": ms / kernel_ms, "dtype": "f16 I/O, f32 arithmetic"}
-        result["extras"]["other_shapes"] = other_shapes(torch, swin3d_amd, synth, crse, scene, dev)
+        if not args.no_other_shapes:
+            result["extras"]["other_shapes"] = other_shapes(torch, swin3d_amd, synth, crse, scene, dev)
         # the headline layer in fp32, the compute type of the operator when autocast is off (PrecisionMode.HALF_NONE)
         f32_args = tuple(x.float() for x in fwd_args[:6]) + fwd_args[6:]
         ms = _time_gpu(torch, lambda: swin3d_amd.window_attention_forward(*f32_args), reps=10)

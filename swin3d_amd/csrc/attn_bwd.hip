@@ -31,6 +31,7 @@ namespace {
 
 using namespace sweep;
 
+constexpr int kCounterSets = 4;
 constexpr int kBwdThreads = 256;
 constexpr int kBwdWaves = kBwdThreads / 64;
 constexpr int kChunk = 64;            // owned elements per unit = lanes of a wavefront
@@ -98,8 +99,15 @@ __global__ void bwd_prepare_kernel(BwdArgs a)
     const T *go = static_cast<const T *>(a.dout);
     const T *o = static_cast<const T *>(a.out);
     for (int64_t t = t0; t < a.N * a.H; t += stride) {
+        // head_dim is a multiple of 8: rows in pieces of eight channels (16- or 32-byte loads)
         float s = 0.0f;
-        for (int c = 0; c < a.D; ++c) s += to_float(go[t * a.D + c]) * to_float(o[t * a.D + c]);
+        for (int c0 = 0; c0 < a.D; c0 += 8) {
+            float x[8], y[8];
+            load_row<8>(go + t * a.D + c0, x);
+            load_row<8>(o + t * a.D + c0, y);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) s += x[c] * y[c];
+        }
         a.delta[t] = s;
     }
     for (int64_t t = t0; t < a.table_len; t += stride) {
@@ -107,10 +115,12 @@ __global__ void bwd_prepare_kernel(BwdArgs a)
         a.dtk[t] = 0.0f;
         a.dtv[t] = 0.0f;
     }
-    for (int64_t t = t0; t < a.H * kQueues; t += stride) a.units[t * kCounterStride] = 0;
+    for (int64_t t = t0; t < kCounterSets * a.H * kQueues; t += stride) a.units[t * kCounterStride] = 0;
 }
 
-__host__ __device__ inline size_t units_total_index(int H) { return static_cast<size_t>(H) * kQueues * kCounterStride; }
+// kCounterSets sets of H * kQueues work counters: every table-gradient kernel of a call draws from a set of its own
+// (sets 0..3 by kind), so none has to wait for the counters to be put back; the fused sweeps share set 0 and reset it
+__host__ __device__ inline size_t units_total_index(int H) { return static_cast<size_t>(kCounterSets) * H * kQueues * kCounterStride; }
 __host__ __device__ inline size_t units_list_index(int H) { return units_total_index(H) + 64; }
 
 // unit list in window order: one (window, chunk of 64 owned elements) descriptor per unit, and the unit count;
@@ -175,28 +185,37 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
         }
     }
     __syncthreads();
-    {
-        // where the (pair, head) records of a window start in the pair store: written at the window's first position
-        long long before = wave_pairs[wave] + pairs_incl - pairs_mine;
-        for (int w = begin; w < end; ++w) {
-            const int n = a.w_sizes[w];
-            if (n > 0) a.pos_base[a.w2n[w]] = before;
-            before += static_cast<long long>(n) * n;
-        }
-    }
+    // where the (pair, head) records of a window start in the pair store: written at the window's first position
+    long long before = wave_pairs[wave] + pairs_incl - pairs_mine;
     int run[kClasses];
 #pragma unroll
     for (int c = 0; c < kClasses; ++c) run[c] = wave_sum[wave][c] + incl[c] - mine[c];
     int2 *list = reinterpret_cast<int2 *>(a.units + units_list_index(a.H));
-    for (int w = begin; w < end; ++w) {
-        const int n = a.w_sizes[w];
-        const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
-        int at = 0;
+    // four windows at a time: their sizes and first positions are loaded before any of their stores (a load after
+    // a store through another pointer waits for it)
+    for (int w0 = begin; w0 < end; w0 += 4) {
+        int n4[4], s4[4];
 #pragma unroll
-        for (int c = 0; c < kClasses; ++c) {
-            if (c == cls) { at = run[c]; run[c] += chunks; }
+        for (int e = 0; e < 4; ++e) {
+            const int w = min(w0 + e, end - 1);
+            n4[e] = a.w_sizes[w];
+            s4[e] = a.w2n[w];
         }
-        for (int c = 0; c < chunks; ++c) list[at + c] = make_int2(w, c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int w = w0 + e;
+            if (w >= end) break;
+            const int n = n4[e];
+            if (n > 0) a.pos_base[s4[e]] = before;
+            before += static_cast<long long>(n) * n;
+            const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
+            int at = 0;
+#pragma unroll
+            for (int c = 0; c < kClasses; ++c) {
+                if (c == cls) { at = run[c]; run[c] += chunks; }
+            }
+            for (int c = 0; c < chunks; ++c) list[at + c] = make_int2(w, c);
+        }
     }
     if (threadIdx.x == 0) a.units[units_total_index(a.H)] = class_start[kClasses];
 }
@@ -637,7 +656,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND 
 
     const int2 *unit_list = reinterpret_cast<const int2 *>(a.units + units_list_index(H));
     const int total_units = __builtin_amdgcn_readfirstlane(a.units[units_total_index(H)]);
-    int *counters = a.units + h * kQueues * kCounterStride;
+    int *counters = a.units + (KIND * H + h) * kQueues * kCounterStride;
 
     int queue = xcd_id() % kQueues;
     int tried = 0;
@@ -813,28 +832,37 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND 
     }
 }
 
-// Sums the per-wavefront table gradients of a sweep over the wavefronts of each head: one thread per
-// (kind, flat row, head, channel).  dst_a / dst_b: the gradient tables of kind 0 / 1 (null = not produced).
+// Sums the per-wavefront table gradients of a sweep over the wavefronts of each head.  One wavefront per (kind, flat
+// row, head): its lanes are the D channels of the row times 64 / D shares of the head's slots, which they read 4 D
+// bytes at a time and add up by shuffles at the end.  dst_a / dst_b: the gradient tables of kind 0 / 1 (null = not
+// produced).
 __global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float *dst_a, float *dst_b, int flat_rows,
                                                                  int groups)
 {
     const int H = a.H, D = a.D;
-    const int per_kind = a.total_rows * H * D;
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= 2 * per_kind) return;
-    const int kind = t / per_kind;
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);   // (kind, row, head)
+    if (item >= 2 * a.total_rows * H) return;
+    const int kind = item / (a.total_rows * H);
     float *dst = kind == 0 ? dst_a : dst_b;
     if (!dst) return;
-    const int e = t - kind * per_kind;
-    const int c = e % D, h = (e / D) % H, row = e / (D * H);
+    const int e = item - kind * a.total_rows * H;
+    const int h = e % H, row = e / H;
+    const int c = lane % D, share = lane / D, shares = 64 / D;
     const size_t slot_floats = 2 * static_cast<size_t>(flat_rows) * D;
     const size_t in_slot = (static_cast<size_t>(kind) * flat_rows + row) * D + c;
-    // workgroup b serves head (b / kQueues) % H
+    // workgroup b of the sweep serves head (b / kQueues) % H: the head's slots are those of workgroups
+    // (set * H + h) * kQueues + x, x < kQueues, four wavefronts each
+    const int sets = groups / (H * kQueues);
+    const int head_slots = sets * kQueues * kBwdWaves;
     float sum = 0.0f;
-    for (int b = h * kQueues; b < groups; b += H * kQueues)
-        for (int x = 0; x < kQueues * kBwdWaves; ++x)
-            sum += a.tgrad[(static_cast<size_t>(b) * kBwdWaves + x) * slot_floats + in_slot];
-    dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
+    for (int x = share; x < head_slots; x += shares) {
+        const int set = x / (kQueues * kBwdWaves), in_set = x - set * (kQueues * kBwdWaves);
+        const size_t slot = (static_cast<size_t>(set) * H + h) * (kQueues * kBwdWaves) + in_set;
+        sum += a.tgrad[slot * slot_floats + in_slot];
+    }
+    for (int other = D; other < 64; other <<= 1) sum += __shfl_xor(sum, other);
+    if (share == 0) dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
 }
 
 template <typename T, int D>
@@ -861,8 +889,8 @@ int launch_sweep_blk(const BwdArgs &a, int grid, hipStream_t stream)
     S3D_HIP_CHECK(hipGetLastError());
     float *dst_a = need_dl ? (KEY_OWNED ? a.dtq : a.dtk) : nullptr;
     float *dst_b = (KEY_OWNED && MODE != 1) ? a.dtv : nullptr;
-    const int threads = 2 * a.total_rows * a.H * a.D;
-    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
+    const int items = 2 * a.total_rows * a.H;
+    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((items + 3) / 4)), dim3(256), 0, stream,
                        a, dst_a, dst_b, BLK * 64, grid);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;
@@ -898,12 +926,11 @@ int launch_tables_blk(const BwdArgs &a, int grid, hipStream_t stream)
     int fit = 0;
     S3D_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, reinterpret_cast<const void *>(kernel), kBwdThreads, lds));
     grid = bwd_grid(a.H, fit < 1 ? 1 : fit > kTablesPerCu ? kTablesPerCu : fit);
-    hipLaunchKernelGGL(bwd_reset_counters_kernel, dim3(1), dim3(64), 0, stream, a);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBwdThreads), lds, stream, a);
     S3D_HIP_CHECK(hipGetLastError());
-    const int threads = 2 * a.total_rows * a.H * a.D;
+    const int items = 2 * a.total_rows * a.H;
     float *first = KIND == 0 ? a.dtk : KIND == 3 ? a.dtv : a.dtq;
-    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(bwd_reduce_tables_kernel, dim3(static_cast<unsigned>((items + 3) / 4)), dim3(256), 0, stream,
                        a, first, KIND == 1 ? a.dtv : nullptr, BLK * 64, grid);
     S3D_HIP_CHECK(hipGetLastError());
     return S3D_OK;

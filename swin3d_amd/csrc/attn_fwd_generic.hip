@@ -699,7 +699,9 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
 template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_threads() { return 256; }
 
 template <typename T, int D, int ND, int HP, bool kKeyOwned>
-__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>())) void attn_bwd_pairs_kernel(BwdPairArgs b)
+// fp16 at head_dim 8: capped at 128 registers, four wavefronts per SIMD (-1 to -2 % against the three that the
+// key-owned sweep's 133 registers allow)
+__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && D == 8 ? 4 : 1)) void attn_bwd_pairs_kernel(BwdPairArgs b)
 {
     const AttnArgs &a = b.f;
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
