@@ -303,8 +303,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     pairs: M = sum(w_sizes^2) of the window set (the reference's index arrays have this length,
     swin3d_layers.py:96-103); None = read it from w_sizes once and keep it on that tensor.  With it the library
     runs the pair sweeps, which keep dL and P of every (pair, head) in the workspace (12 bytes each); 0, or a
-    store above BWD_PAIR_STORE_MAX_BYTES, selects the fused sweeps, which need no such store and take about
-    twice as long."""
+    store above BWD_PAIR_STORE_MAX_BYTES, selects the fused sweeps, which need no such store and take about a
+    third longer."""
     w_sizes_in = w_sizes
     _require_cuda("query", q)
     dev = q.device

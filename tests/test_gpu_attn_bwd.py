@@ -289,3 +289,12 @@ def test_pair_count_larger_than_needed(oracle_lib, hip_lib):
         assert torch.equal(a, b)
     for a, b in zip(exact[3:], roomy[3:]):
         assert float((a - b).abs().max()) <= 1e-5 * float(a.abs().max())
+
+
+@pytest.mark.parametrize("heads,dim", [(10, 16), (20, 16), (40, 16), (40, 8)])
+def test_head_counts_of_the_large_model(oracle_lib, hip_lib, heads, dim):
+    """Swin3D-L runs 10, 20 and 40 heads of 16 channels (many head groups: the sweeps' workgroups then take the
+    head groups in turn instead of in whole sets per XCD)."""
+    case = make_attn_case(oracle_lib, seed=300 + heads, n=700, ws=7, quant=4, heads=heads, dim=dim, extent=(12, 12, 6),
+                          recipe="layer")
+    _check(oracle_lib, case, torch.float16, seed=heads)
