@@ -698,7 +698,7 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
 // the lanes of a window write consecutive addresses.
 template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_threads() { return 256; }
 
-template <typename T, int D, int ND, int HP, bool kKeyOwned>
+template <typename T, int D, int ND, int HP, bool kKeyOwned, bool kShared>
 // fp16 at head_dim 8: capped at 128 registers, four wavefronts per SIMD (-1 to -2 % against the three that the
 // key-owned sweep's 133 registers allow)
 __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && D == 8 ? 4 : 1)) void attn_bwd_pairs_kernel(BwdPairArgs b)
@@ -757,7 +757,10 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
     }
     // the one table-row sum that enters the owned gradient as a vector (Tq for dq_i, Tk for dk_j) sits behind the
     // q-side slice in the query-owned sweep and behind the k-side slice in the key-owned one
-    constexpr uint32_t kVecSlice = kKeyOwned ? D * sizeof(T) : 0;
+    // kShared: the key-owned sweep reads dL and P from records that the query-owned sweep, which ran before it,
+    // wrote beside its own
+    constexpr bool kRead = kKeyOwned && kShared;
+    constexpr bool kWriteBoth = !kKeyOwned && kShared;
 
     int queue = xcd_id() % kQueues;
     int tried = 0;
@@ -806,7 +809,7 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
             const int64_t at_row = static_cast<int64_t>(own_row) * HD + (h + hh) * D;
             if constexpr (kKeyOwned) {
                 own_x[hh].load(gk + at_row);
-                own_y[hh].load(gv + at_row);
+                if constexpr (!kRead) own_y[hh].load(gv + at_row);
             } else {
                 own_x[hh].load(gq + at_row);
                 own_y[hh].load(ggo + at_row);
@@ -838,7 +841,11 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
 #pragma unroll
             for (int hh = 0; hh < HP; ++hh) {
                 const int64_t at_row = static_cast<int64_t>(st_row) * HD + (h + hh) * D;
-                if constexpr (kKeyOwned) {
+                if constexpr (kRead) {
+                    st_x[hh].load(gq + at_row);
+                    st_y[hh].load(ggo + at_row);
+                    st_m[hh] = st_inv[hh] = st_delta[hh] = 0.0f;
+                } else if constexpr (kKeyOwned) {
                     st_x[hh].load(gq + at_row);
                     st_y[hh].load(ggo + at_row);
                     st_m[hh] = b.stat_max[static_cast<int64_t>(st_row) * H + h + hh];
@@ -867,8 +874,16 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
                 const Slice<T, D> &kv = kKeyOwned ? own_x[hh] : st_x[hh];
                 const Slice<T, D> &vv = kKeyOwned ? own_y[hh] : st_y[hh];
                 const Slice<T, D> &gov = kKeyOwned ? st_y[hh] : own_y[hh];
-                float logit = qv.dot(kv, 0.0f);
-                float dp = gov.dot(vv, 0.0f);
+                const int64_t head_at = static_cast<int64_t>(h + hh) * b.pairs + pair_base;
+                float2 rec = make_float2(0.0f, 0.0f);
+                if constexpr (kRead) {
+                    if (valid) rec = b.pd[head_at + static_cast<int64_t>(st_in) * n_w + own_in];
+                }
+                float logit = 0.0f, dp = 0.0f;
+                if constexpr (!kRead) {
+                    logit = qv.dot(kv, 0.0f);
+                    dp = gov.dot(vv, 0.0f);
+                }
                 // sums of three rows of the table that enters the owned gradient as a vector (packed fp16 adds for
                 // fp16 I/O, as the forward adds its value-table rows)
                 constexpr int kGroup = 3;
@@ -876,13 +891,15 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
 #pragma unroll
                 for (int n = 0; n < ND; ++n) {
                     Slice<T, D> tq_r, tk_r, tv_r;
-                    tq_r.load_lds(off[n] + hh * kHeadBytes);
                     tk_r.load_lds(off[n] + hh * kHeadBytes + D * sizeof(T));
-                    tv_r.load_lds(off[n] + hh * kHeadBytes + 2 * D * sizeof(T));
-                    if (Slice<T, D>::kChainLogit) logit = kv.dot(tk_r, qv.dot(tq_r, logit));
-                    else logit += kv.dot(tk_r, qv.dot(tq_r, 0.0f));
-                    if (Slice<T, D>::kChainLogit) dp = gov.dot(tv_r, dp);
-                    else dp += gov.dot(tv_r, 0.0f);
+                    if constexpr (!kRead) {
+                        tq_r.load_lds(off[n] + hh * kHeadBytes);
+                        tv_r.load_lds(off[n] + hh * kHeadBytes + 2 * D * sizeof(T));
+                        if (Slice<T, D>::kChainLogit) logit = kv.dot(tk_r, qv.dot(tq_r, logit));
+                        else logit += kv.dot(tk_r, qv.dot(tq_r, 0.0f));
+                        if (Slice<T, D>::kChainLogit) dp = gov.dot(tv_r, dp);
+                        else dp += gov.dot(tv_r, 0.0f);
+                    }
                     const Slice<T, D> &vec_r = kKeyOwned ? tk_r : tq_r;
                     if (n % kGroup == 0) vec_sum[n / kGroup] = vec_r;
                     else vec_sum[n / kGroup].add(vec_r);
@@ -890,17 +907,24 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
                 const float m_i = kKeyOwned ? st_m[hh] : own_m[hh];
                 const float inv_i = kKeyOwned ? 1.0f / st_inv[hh] : own_inv[hh];
                 const float delta_i = kKeyOwned ? st_delta[hh] : own_delta[hh];
-                const float p = valid ? __expf(logit - m_i) * inv_i : 0.0f;
-                const float dl = p * (dp - delta_i);
+                const float p = kRead ? rec.y : valid ? __expf(logit - m_i) * inv_i : 0.0f;
+                const float dl = kRead ? rec.x : p * (dp - delta_i);
                 // dq_i += dL (k_j + Tq)   or   dk_j += dL (q_i + Tk)
                 st_x[hh].fma_to(res_x[hh], dl);
 #pragma unroll
                 for (int g = 0; g < (ND + kGroup - 1) / kGroup; ++g) vec_sum[g].fma_to(res_x[hh], dl);
                 if constexpr (kKeyOwned) st_y[hh].fma_to(res_y[hh], p);     // dv_j += P dout_i
                 if (valid) {
-                    const int64_t head_at = static_cast<int64_t>(h + hh) * b.pairs + pair_base;
-                    if constexpr (kKeyOwned) b.pd[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = make_float2(dl, p);
-                    else b.dl_t[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = dl;
+                    if constexpr (kRead) {
+                        // nothing to leave: the records are the query-owned sweep's
+                    } else if constexpr (kKeyOwned) {
+                        b.pd[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = make_float2(dl, p);
+                    } else {
+                        b.dl_t[head_at + static_cast<int64_t>(st_in) * n_w + own_in] = dl;
+                        // (dL, P) at [i][j] as well: a lane's records of successive steps are consecutive, the lanes'
+                        // n records apart
+                        if constexpr (kWriteBoth) b.pd[head_at + static_cast<int64_t>(own_in) * n_w + st_in] = make_float2(dl, p);
+                    }
                 }
             }
         }
@@ -1033,7 +1057,7 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream, int what)
 
 namespace {
 
-template <typename T, int D, int ND, int HP>
+template <typename T, int D, int ND, int HP, bool kShared>
 int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
 {
     const AttnArgs &a = b0.f;
@@ -1041,8 +1065,8 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
-    auto q_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, false>;
-    auto k_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, true>;
+    auto q_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, false, kShared>;
+    auto k_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, true, kShared>;
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
     int per_cu = 1;
     for (auto kernel : {q_sweep, k_sweep}) {
@@ -1083,7 +1107,17 @@ int launch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
 {
     // one head per wavefront: with two (fp16, head_dim 8) the key-owned sweep needs more than 256 registers and the
     // pair of sweeps measured 0.3 ms slower at the 6-head layer
-    return launch_bwd_pairs_heads<T, D, ND, 1>(b, stream);
+    //
+    // Who computes dL and P for the key-owned sweep.  Either it does, as the query-owned sweep does (the logits, dP,
+    // the exponential: 125 of its 280 instructions per pair and head), or the query-owned sweep, which runs first,
+    // leaves its values at [i][j] as well and the key-owned sweep reads them.  That second copy is written with the
+    // lanes n records apart (a lane's own records of successive steps are consecutive); windows of more than 64
+    // voxels, whose queries have several lanes each on adjacent records, write it in longer runs.  Measured, whole
+    // backward, own values / shared: 1.76 / 1.87 ms on 26-voxel windows (6 heads of 8), 2.24 / 2.12 and 2.33 / 2.25
+    // ms on the window-7 layers of 57 voxels a window (6 heads of 16, 12 of 8).  Shared where the mean window has
+    // more than 32 voxels.
+    if (b.f.N > 32 * b.f.W) return launch_bwd_pairs_heads<T, D, ND, 1, true>(b, stream);
+    return launch_bwd_pairs_heads<T, D, ND, 1, false>(b, stream);
 }
 
 template <typename T>
