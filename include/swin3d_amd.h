@@ -191,7 +191,8 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *                  kind of work list (dq; dk and dv), which leave dL and P of every (pair, head) in the workspace
  *                  - 12 * H * pairs bytes -, and two table-gradient sweeps that read them.  With 0 it runs two fused
  *                  sweeps that recompute the logits for the table gradients and need no such store (about a third
- *                  more time).  A value below M leaves the gradients of the windows beyond it unwritten.
+ *                  more time).  A value below M cannot hold the records of every window: the rows of dq, dk, dv
+ *                  that belong to the windows beyond it and all three table gradients then come out as NaN.
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs) bytes
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *

@@ -183,6 +183,8 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
             wave_pairs[v] = before;
             before += add;
         }
+        // a pair store shorter than the window set's pairs: the call's results are marked (NaN), see the reduction
+        a.units[units_total_index(a.H) + 1] = a.pairs > 0 && before > a.pairs;
     }
     __syncthreads();
     // where the (pair, head) records of a window start in the pair store: written at the window's first position
@@ -862,6 +864,8 @@ __global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float
         sum += a.tgrad[slot * slot_floats + in_slot];
     }
     for (int other = D; other < 64; other <<= 1) sum += __shfl_xor(sum, other);
+    // the caller's pair count was too small for the window set: windows were skipped, so no sum is valid
+    if (a.pairs > 0 && a.units[units_total_index(H) + 1]) sum = __int_as_float(0x7fc00000);
     if (share == 0) dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
 }
 

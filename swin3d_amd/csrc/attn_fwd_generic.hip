@@ -939,7 +939,16 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
                     for (int c = 0; c < D; ++c) res_y[hh][c] += __shfl_xor(res_y[hh][c], other);
                 }
             }
-            if (own_valid && sub == 0 && fits) {
+            if (own_valid && sub == 0) {
+                // a window beyond the caller's pair store was skipped: its rows say so
+                if (!fits) {
+#pragma unroll
+                    for (int c = 0; c < D; ++c) res_x[hh][c] = __int_as_float(0x7fc00000);
+                    if constexpr (kKeyOwned) {
+#pragma unroll
+                        for (int c = 0; c < D; ++c) res_y[hh][c] = __int_as_float(0x7fc00000);
+                    }
+                }
                 const int64_t at_row = static_cast<int64_t>(own_row) * HD + (h + hh) * D;
                 if constexpr (kKeyOwned) {
                     store_row<D>(static_cast<T *>(b.dk) + at_row, res_x[hh]);

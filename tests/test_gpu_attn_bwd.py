@@ -298,3 +298,28 @@ def test_head_counts_of_the_large_model(oracle_lib, hip_lib, heads, dim):
     case = make_attn_case(oracle_lib, seed=300 + heads, n=700, ws=7, quant=4, heads=heads, dim=dim, extent=(12, 12, 6),
                           recipe="layer")
     _check(oracle_lib, case, torch.float16, seed=heads)
+
+
+def test_pair_count_too_small_is_loud(oracle_lib, hip_lib):
+    """A pair count below the window set's sum of squares cannot hold every window's records: no fault, and the
+    gradients that are incomplete come out as NaN (all three table gradients, the rows of the skipped windows)."""
+    import swin3d_amd
+    case = make_attn_case(oracle_lib, seed=79, n=3000, ws=5, quant=4, heads=6, dim=8, extent=(16, 16, 8), recipe="layer")
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    feats = [t(x).half() for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
+    idx = [t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)]
+    sizes = [int(x) for x in case.table_sizes]
+    out, mx, sm = swin3d_amd.window_attention_forward(*feats, sizes, *idx, return_stats=True)
+    dout = torch.randn_like(out)
+    m = int((idx[0].long() ** 2).sum())
+    full = swin3d_amd.window_attention_backward(*feats, sizes, *idx, out, mx, sm, dout, pairs=m)
+    short = swin3d_amd.window_attention_backward(*feats, sizes, *idx, out, mx, sm, dout, pairs=m // 2)
+    torch.cuda.synchronize()
+    for g in short[3:]:
+        assert torch.isnan(g).all()
+    for g, ref in zip(short[:3], full[:3]):
+        bad = torch.isnan(g.float()).any(dim=2).any(dim=1)
+        assert bad.any() and not bad.all()
+        assert torch.equal(g[~bad], ref[~bad])      # the windows inside the store are complete
