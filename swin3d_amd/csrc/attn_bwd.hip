@@ -6,7 +6,11 @@
 //   dv_j  += P dout_i                              dTv[n][row_n(i,j)] += P dout_i
 //   dq_i  += dL (k_j + Tq(i,j))                    dTq[n][row_n(i,j)] += dL q_i
 //   dk_j  += dL (q_i + Tk(i,j))                    dTk[n][row_n(i,j)] += dL k_j
-// The reference adds every term with a global atomic.  Here every output element has ONE owner:
+// The reference adds every term with a global atomic.  Here every output element has ONE owner, and the call has two
+// forms.  With the window set's pair count it runs the pair sweeps of attn_fwd_generic.hip (dq; dk and dv; on the
+// forward's packed work list), which leave dL and P of every (pair, head) in the workspace, and the table-gradient
+// kernels below (attn_bwd_tables_kernel), which read them.  Without it, the fused sweeps (attn_bwd_sweep_kernel),
+// which recompute the logits and need no store:
 //
 //  * a key-owned sweep gives a lane one key j and streams the window's queries through the wavefront:
 //    dk_j, dv_j accumulate in the lane's registers and are stored once;

@@ -1,14 +1,16 @@
-// Sparse-voxel windowed self-attention forward with cRSE tables (gfx950): sweep kernel.
+// Sparse-voxel windowed self-attention with cRSE tables (gfx950): the sweep kernel of the forward and, on the same
+// work list, the pair sweeps of the backward (dq; dk and dv - further down).
 //
 // Covers every dtype / shape the library accepts on the vector ALU (fp32 arithmetic; fp16 inputs enter through
-// packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one head (or two)
+// packed dot products and mixed-precision FMAs with fp32 accumulation).  A workgroup serves one to three heads
 // for its whole life and keeps the slices of the three relative-signal tables in LDS (loaded once, not once
 // per window).  Lane = one query against (a share of) the keys of its window: q_i, the running
 // maximum, sum and output stay in the lane's registers while the lane streams its own window's keys, one per
 // step, no atomic on data and no O(pairs) index array; the result is
 // deterministic.  The slots of all windows, sorted by step count, are packed into units of 64 (the lanes of a
 // wavefront carry queries of several small windows); wavefronts draw units from the head's work queues.
-// Windows of more than 64 voxels leave one partial result per key block, combined by generic_merge_kernel.
+// A query of a window of more than the step target gets 2, 4 or 8 adjacent lanes that take alternate keys and merge
+// their softmax states by shuffles at the end of the unit.
 //
 // Math (per window, sorted positions i, j, head h), following the reference kernels
 // Swin3D/src/attn/self_attn_aio_fwd.cu:16-52 and :111-188:
