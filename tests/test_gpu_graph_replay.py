@@ -1,4 +1,4 @@
-"""The forward that allocates nothing (s3d_attn_fwd_noalloc) and the planned forward under HIP graph capture: the
+"""The forward that allocates nothing (s3d_attn_fwd_noalloc), the planned forward and the backward under HIP graph capture: the
 launches are recorded once and replayed on changed inputs, with the program's own eager work and synchronisations
 between the replays; every replay must give the bits of the eager call on the same inputs.  (The work list's
 queue counters are put back to zero by the sweep kernel itself, so a replay needs no clearing node.)"""
@@ -74,3 +74,62 @@ def test_replays_equal_eager_calls(oracle_lib, hip_lib, entry):
         torch.cuda.synchronize()
         assert torch.isfinite(replayed).all()
         assert torch.equal(replayed, out)
+
+
+def test_backward_replays_equal_eager_calls(oracle_lib, hip_lib):
+    """s3d_attn_bwd with its pair store under graph capture: the whole call - list builds, pair sweeps,
+    table-gradient kernels, reductions - is kernels on the caller's stream and clears what it needs itself."""
+    from swin3d_amd import _lib
+    import swin3d_amd
+    case, x = _inputs(oracle_lib, 102)
+    n, h, d = x["q"].shape
+    w = x["w_sizes"].numel()
+    sizes = [int(s) for s in case.table_sizes]
+    c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
+    table_len = x["tq"].numel()
+    pairs = int((x["w_sizes"].long() ** 2).sum())
+    out, omax, osum = swin3d_amd.window_attention_forward(x["q"], x["k"], x["v"], x["tq"], x["tk"], x["tv"], sizes,
+                                                          x["w_sizes"], x["w2n"], x["n2n"], x["n_coords"],
+                                                          return_stats=True)
+    dout = torch.randn_like(out)
+    grads = [torch.empty_like(x["q"]) for _ in range(3)] + [torch.empty(table_len, dtype=torch.float32, device="cuda")
+                                                           for _ in range(3)]
+    nbytes = hip_lib.s3d_attn_bwd_workspace_bytes(h, d, len(sizes), n, w, pairs)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()      # default priority
+
+    def launch(stream):
+        status = hip_lib.s3d_attn_bwd(
+            x["q"].data_ptr(), x["k"].data_ptr(), x["v"].data_ptr(), x["tq"].data_ptr(), x["tk"].data_ptr(),
+            x["tv"].data_ptr(), c_sizes, len(sizes), table_len, x["w_sizes"].data_ptr(), x["w2n"].data_ptr(),
+            x["n2n"].data_ptr(), x["n_coords"].data_ptr(), out.data_ptr(), omax.data_ptr(), osum.data_ptr(),
+            dout.data_ptr(), *(g.data_ptr() for g in grads), n, h, d, w, pairs, _lib.S3D_DTYPE_F16,
+            workspace.data_ptr(), nbytes, stream)
+        _lib.check(status, "s3d_attn_bwd")
+
+    launch(torch.cuda.current_stream().cuda_stream)          # eager warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        launch(side.cuda_stream)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    rng = torch.Generator(device="cuda").manual_seed(8)
+    for _ in range(3):
+        dout.copy_(torch.randn(dout.shape, generator=rng, device="cuda").half())
+        for g in grads:
+            g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = [g.clone() for g in grads]
+        for g in grads:
+            g.fill_(float("nan"))
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for a, b in zip(replayed[:3], grads[:3]):
+            assert torch.isfinite(a).all() and torch.equal(a, b)
+        for a, b in zip(replayed[3:], grads[3:]):
+            assert torch.isfinite(a).all()
+            assert float((a - b).abs().max()) <= 1e-5 * float(b.abs().max())
