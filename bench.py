@@ -80,6 +80,8 @@ def main():
                     help="with --encoder-only: keep every level's voxels in the order of its regular windows")
     ap.add_argument("--sources-hash", action="store_true",
                     help="print the hash of the headline kernel's sources (recorded in the profile summary) and exit")
+    ap.add_argument("--train-only", action="store_true",
+                    help="run only the Swin3D-S training-step side figure")
     ap.add_argument("--encoder-only", action="store_true",
                     help="run only the Swin3D-L encoder forward (1 warm-up + 3 timed passes, no UNet) and print its "
                          "figures: the command the encoder's kernel trace is taken with")
@@ -105,6 +107,9 @@ def main():
         return 3
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.train_only:
+        print(json.dumps({"train_step_swin3d_s": train_step_latency(torch, synth, dev)}))
+        return 0
     if args.encoder_only:
         print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False,
                                                               window_ordered=args.window_ordered)}))
@@ -300,6 +305,7 @@ def main():
 
     if not args.no_extras and not args.no_encoder:
         result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)
+        result["extras"]["train_step_swin3d_s"] = train_step_latency(torch, synth, dev)
 
     if not args.no_cpu_baseline and not args.no_extras:
         import oracle
@@ -461,6 +467,45 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     result["unet_ms"] = float(np.median(times))
     result["unet_finite"] = bool(torch.isfinite(logits).all().item())
     return result
+
+
+def train_step_latency(torch, synth, dev, voxels=200_000, reps=3):
+    """One optimisation step of the Swin3D-S segmentation network (forward, cross-entropy, backward through
+    s3d_attn_bwd and the interpolation backward, SGD) on one synthetic room: fp16 attention I/O under autocast
+    (fp16_mode 1: the backward in fp32 arithmetic on fp16 tensors), random-init weights, synthetic labels."""
+    from swin3d_amd import encoder
+    scene = synth.make_room((10.0, 8.0, 3.0), 30, voxels, seed=0)
+    feats, signals = synth.encoder_inputs(scene)
+    vox = encoder.SparseVoxels(torch.from_numpy(scene.coords).to(dev), torch.from_numpy(feats).to(dev), 1)
+    sig = torch.from_numpy(signals).to(dev)
+    labels = (vox.coords[:, 3] // 8 % 13).long()
+    torch.manual_seed(0)
+    model = encoder.Swin3DUNet(**encoder.SWIN3D_S, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=1,
+                               upsample="linear_attn", num_classes=13).to(dev).train()
+    opt = torch.optim.SGD(model.parameters(), lr=1e-3)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.float16):
+            logits = model(vox, sig)
+        loss = torch.nn.functional.cross_entropy(logits.float(), labels)
+        loss.backward()
+        opt.step()
+        return loss
+
+    loss = step()                                     # warm-up (allocator, hipBLASLt heuristics)
+    _settle(torch, step, 2 * SETTLE["ms"], batch=1)
+    times = []
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        loss = step()
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    return {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
+            "loss_finite": bool(torch.isfinite(loss).item()),
+            "config": "Swin3D-S UNet (channels [48,96,192,384,384], heads [6,6,12,24,24], depths [2,4,9,4,4]), "
+                      "one room, fp16_mode 1, forward + backward + SGD"}
 
 
 def cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m):

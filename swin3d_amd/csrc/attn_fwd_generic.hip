@@ -702,8 +702,9 @@ template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_
 
 template <typename T, int D, int ND, int HP, bool kKeyOwned, bool kShared>
 // fp16 at head_dim 8: capped at 128 registers, four wavefronts per SIMD (-1 to -2 % against the three that the
-// key-owned sweep's 133 registers allow)
-__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && D == 8 ? 4 : 1)) void attn_bwd_pairs_kernel(BwdPairArgs b)
+// key-owned sweep's 133 registers allow).  The others at two: fp32 at head_dim 16 would take 286 registers and run
+// one wavefront per SIMD (the backward of a 6-head window-7 layer: 3.16 ms; capped at 256 with 24 spilled: 2.89)
+__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && D == 8 ? 4 : 2)) void attn_bwd_pairs_kernel(BwdPairArgs b)
 {
     const AttnArgs &a = b.f;
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
@@ -888,7 +889,8 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && 
                 }
                 // sums of three rows of the table that enters the owned gradient as a vector (packed fp16 adds for
                 // fp16 I/O, as the forward adds its value-table rows)
-                constexpr int kGroup = 3;
+                // (fp32: one sum of all rows - plain adds, no packing to gain, and two sums fewer to hold)
+                constexpr int kGroup = sizeof(T) == 4 ? ND : 3;
                 Slice<T, D> vec_sum[(ND + kGroup - 1) / kGroup];
 #pragma unroll
                 for (int n = 0; n < ND; ++n) {
