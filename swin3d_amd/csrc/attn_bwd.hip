@@ -600,9 +600,10 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
 // come from HBM and a step is a short dependent chain (rows, histogram atomics, read-back), so their latency would
 // be most of it.
 // Wavefronts per SIMD: two for KIND 1 at head_dim 8 (80 accumulators; capped at 168 registers for three it spills
-// and measured 1.7x the time), three for the one-table kinds; at head_dim 16 one, and two for the halves.
+// and measured 1.7x the time), three for the one-table kinds; at head_dim 16 one for KIND 1 and two for the
+// one-table kinds (KIND 0 capped at 256 registers spills 40 of them and is still 2-3 % of the call faster than at one).
 template <typename T, int D, int ND, int KIND, int BLK>
-__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND >= 2 ? 2 : 1))) void attn_bwd_tables_kernel(BwdArgs a)
+__global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND != 1 ? 2 : 1))) void attn_bwd_tables_kernel(BwdArgs a)
 {
     constexpr bool KEY_OWNED = KIND != 0;
     constexpr bool kAccB = KIND == 1;                          // two histograms and two sets of accumulators
