@@ -127,8 +127,11 @@ __global__ void bwd_prepare_kernel(BwdArgs a)
 __host__ __device__ inline size_t units_total_index(int H) { return static_cast<size_t>(kCounterSets) * H * kQueues * kCounterStride; }
 __host__ __device__ inline size_t units_list_index(int H) { return units_total_index(H) + 64; }
 
-// unit list in window order: one (window, chunk of 64 owned elements) descriptor per unit, and the unit count;
-// one workgroup
+// unit list: one (window, chunk of 64 owned elements, segment of 64 streamed elements) descriptor per unit, and the
+// unit count; one workgroup.  The table-gradient kernels (a.pairs > 0) take a window of more than 64 voxels in
+// segments of 64 streamed voxels - what a unit adds to the table gradients is a sum over the streamed side, and one
+// unit for all 343 voxels of a full window was three times the average wavefront's share of a launch; the fused
+// sweeps, whose owned gradients need the whole stream, get one unit per chunk (segment 0).
 __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
 {
     // units are listed longest first, in classes of window size (a unit streams the whole window: n steps, or
@@ -148,8 +151,9 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
     for (int w = begin; w < end; ++w) {
         const int n = a.w_sizes[w];
         const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
+        const int units_w = a.pairs > 0 ? chunks * chunks : chunks;
 #pragma unroll
-        for (int c = 0; c < kClasses; ++c) mine[c] += c == cls ? chunks : 0;
+        for (int c = 0; c < kClasses; ++c) mine[c] += c == cls ? units_w : 0;
         pairs_mine += static_cast<long long>(n) * n;
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -215,12 +219,14 @@ __global__ __launch_bounds__(1024) void bwd_units_kernel(BwdArgs a)
             if (n > 0) a.pos_base[s4[e]] = before;
             before += static_cast<long long>(n) * n;
             const int chunks = n > 0 ? (n + kChunk - 1) / kChunk : 0, cls = class_of(n);
+            const int segs = a.pairs > 0 ? chunks : 1;
             int at = 0;
 #pragma unroll
             for (int c = 0; c < kClasses; ++c) {
-                if (c == cls) { at = run[c]; run[c] += chunks; }
+                if (c == cls) { at = run[c]; run[c] += chunks * segs; }
             }
-            for (int c = 0; c < chunks; ++c) list[at + c] = make_int2(w, c);
+            for (int c = 0; c < chunks; ++c)
+                for (int sg = 0; sg < segs; ++sg) list[at + c * segs + sg] = make_int2(w, c | (sg << 16));
         }
     }
     if (threadIdx.x == 0) a.units[units_total_index(a.H)] = class_start[kClasses];
@@ -341,7 +347,7 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? 2 : 1)) void attn_bwd_sweep_
         if (unit >= total_units) break;
         const int2 desc = unit_list[unit];
         const int w = __builtin_amdgcn_readfirstlane(desc.x);
-        const int chunk = __builtin_amdgcn_readfirstlane(desc.y);
+        const int chunk = __builtin_amdgcn_readfirstlane(desc.y) & 0xffff;
         const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         // group size: a window of at most 32 voxels streams two elements per step
@@ -679,7 +685,8 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND 
         if (unit >= total_units) break;
         const int2 desc = unit_list[unit];
         const int w = __builtin_amdgcn_readfirstlane(desc.x);
-        const int chunk = __builtin_amdgcn_readfirstlane(desc.y);
+        const int chunk = __builtin_amdgcn_readfirstlane(desc.y) & 0xffff;
+        const int seg = __builtin_amdgcn_readfirstlane(desc.y) >> 16;   // segment of 64 streamed voxels (windows > 64)
         const int n_w = __builtin_amdgcn_readfirstlane(a.w_sizes[w]);
         const int s0 = __builtin_amdgcn_readfirstlane(a.w2n[w]);
         const int gs = n_w <= 32 ? 32 : 64;
@@ -698,7 +705,9 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND 
 #pragma unroll
         for (int n = 0; n < ND; ++n) own_c[n] = a.n_coords[static_cast<int64_t>(s0 + own_in) * ND + n];
 
-        const int steps = (n_w + ng - 1) / ng;
+        // the unit's steps: the whole window, or the segment's 64 streamed voxels (one per step: ng = 1 there)
+        const int it_begin = seg * kChunk;
+        const int steps = n_w > kChunk ? min(n_w, it_begin + kChunk) : (n_w + ng - 1) / ng;
         // The inputs of step `it` for this lane's group (streamed element st = it ng + grp): the streamed rows and
         // coordinates are fetched one step ahead, the lane's records kPrefetch steps ahead.  Every load of the loop is
         // unconditional (clamped positions; what lies past the end is masked where it is used), so the waits count
@@ -733,10 +742,10 @@ __global__ __launch_bounds__(kBwdThreads, (D <= 8 ? (KIND == 1 ? 2 : 3) : (KIND 
         StepIn next;
         float2 rec_ahead[kPrefetch];
 #pragma unroll
-        for (int e = 0; e < kPrefetch; ++e) rec_ahead[e] = fetch_record(e);
-        int row_after = a.n2n[s0 + min(ng + grp, n_w - 1)];   // row of step 1's element
-        fetch(0, a.n2n[s0 + min(grp, n_w - 1)], next);
-        for (int it = 0; it < steps; ++it) {
+        for (int e = 0; e < kPrefetch; ++e) rec_ahead[e] = fetch_record(it_begin + e);
+        int row_after = a.n2n[s0 + min((it_begin + 1) * ng + grp, n_w - 1)];   // row of the second step's element
+        fetch(it_begin, a.n2n[s0 + min(it_begin * ng + grp, n_w - 1)], next);
+        for (int it = it_begin; it < steps; ++it) {
             const StepIn cur = next;
             const bool have = own_valid && fits && it * ng + grp < n_w;
             const float2 rec = rec_ahead[0];
@@ -1032,9 +1041,12 @@ int fill_bwd_axes(BwdArgs &a, const int32_t *table_sizes, int nd, int64_t table_
     return S3D_OK;
 }
 
-size_t bwd_units_bytes(int64_t W, int64_t N, int H)
+// units: one per (window, chunk), and with a pair count one per (window, chunk, segment): the sum over the windows of
+// ceil(n / 64)^2 <= n^2 / 4096 + n / 32 + 1
+size_t bwd_units_bytes(int64_t W, int64_t N, int H, int64_t pairs)
 {
-    const size_t max_units = static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / kChunk;
+    const size_t max_units = static_cast<size_t>(W > 0 ? W : 1) + static_cast<size_t>(N > 0 ? N : 0) / 32 +
+                             static_cast<size_t>(pairs > 0 ? pairs : 0) / 4096;
     return align_up(sizeof(int32_t) * (units_list_index(H) + 2 * max_units), 256);
 }
 
@@ -1061,7 +1073,7 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_
 {
     using namespace s3d;
     if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || N < 0 || W < 0 || pairs < 0) return 0;
-    size_t need = bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
+    size_t need = bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
     if (pairs > 0)
         need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_generic_workspace_bytes(H, W, N), 256);
     return need;
@@ -1112,8 +1124,8 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
     a.units = static_cast<int32_t *>(workspace);
-    a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H));
-    char *at = static_cast<char *>(workspace) + bwd_units_bytes(W, N, H) + bwd_delta_bytes(N, H);
+    a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H, pairs));
+    char *at = static_cast<char *>(workspace) + bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H);
     a.tgrad = reinterpret_cast<float *>(at);
     at += bwd_tgrad_bytes(H, D, nd);
     a.pos_base = reinterpret_cast<int64_t *>(at);
