@@ -701,10 +701,12 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
 template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_threads() { return 256; }
 
 template <typename T, int D, int ND, int HP, bool kKeyOwned, bool kShared>
-// fp16 at head_dim 8: capped at 128 registers, four wavefronts per SIMD (-1 to -2 % against the three that the
-// key-owned sweep's 133 registers allow).  The others at two: fp32 at head_dim 16 would take 286 registers and run
-// one wavefront per SIMD (the backward of a 6-head window-7 layer: 3.16 ms; capped at 256 with 24 spilled: 2.89)
-__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 && D == 8 ? 4 : 2)) void attn_bwd_pairs_kernel(BwdPairArgs b)
+// Wavefronts per SIMD, by register cap.  fp16 at head_dim 8: four (128 registers; -1 to -2 % against the three that
+// the key-owned sweep's 133 registers allow).  fp16 at head_dim 16 and fp32 at head_dim 8: three (168 registers, 3 to
+// 20 of them spilled: the backward of the window-7 layer with 6 heads of 16 2.05 -> 1.99 ms, of the headline layer
+// in fp32 2.28 -> 2.05 ms).  fp32 at head_dim 16: two - uncapped it takes 286 registers and runs one wavefront per
+// SIMD (6-head window-7 layer 3.16 ms; capped at 256 with 24 spilled 2.89).
+__global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 ? (D == 8 ? 4 : 3) : (D == 8 ? 3 : 2))) void attn_bwd_pairs_kernel(BwdPairArgs b)
 {
     const AttnArgs &a = b.f;
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
