@@ -1,5 +1,5 @@
-"""The ctypes stub printed in INTEGRATION.md (the stand-in for the reference's pybind pair cal_max_coffs +
-self_attn_forward) is executed as written and checked against the oracle."""
+"""The ctypes stub that the repository's integration notes print (the stand-in for the reference's pybind pair
+cal_max_coffs + self_attn_forward) is executed as written and checked against the oracle."""
 import os
 import re
 
