@@ -108,7 +108,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.train_only:
-        print(json.dumps({"train_step_swin3d_s": train_step_latency(torch, synth, dev)}))
+        print(json.dumps({"train_step_swin3d_s": train_step_latency(torch, synth, dev),
+                          "train_step_swin3d_s_fp16_mode2": train_step_latency(torch, synth, dev, fp16_mode=2)}))
         return 0
     if args.encoder_only:
         print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False,
@@ -306,6 +307,7 @@ def main():
     if not args.no_extras and not args.no_encoder:
         result["extras"]["encoder_swin3d_l"] = encoder_latency(torch, synth, dev)
         result["extras"]["train_step_swin3d_s"] = train_step_latency(torch, synth, dev)
+        result["extras"]["train_step_swin3d_s_fp16_mode2"] = train_step_latency(torch, synth, dev, fp16_mode=2)
 
     if not args.no_cpu_baseline and not args.no_extras:
         import oracle
@@ -469,10 +471,12 @@ def encoder_latency(torch, synth, dev, voxels_per_scene=300_000, reps=3, unet=Tr
     return result
 
 
-def train_step_latency(torch, synth, dev, voxels=200_000, reps=3):
+def train_step_latency(torch, synth, dev, voxels=200_000, reps=3, fp16_mode=1):
     """One optimisation step of the Swin3D-S segmentation network (forward, cross-entropy, backward through
-    s3d_attn_bwd and the interpolation backward, SGD) on one synthetic room: fp16 attention I/O under autocast
-    (fp16_mode 1: the backward in fp32 arithmetic on fp16 tensors), random-init weights, synthetic labels."""
+    s3d_attn_bwd and the interpolation backward, SGD) on one synthetic room: fp16 attention I/O under autocast,
+    random-init weights, synthetic labels.  fp16_mode 1 (the reference README's setting): the attention backward
+    in fp32 on tensors cast up from fp16; fp16_mode 2 (the reference's example scripts): the backward on fp16
+    tensors."""
     from swin3d_amd import encoder
     scene = synth.make_room((10.0, 8.0, 3.0), 30, voxels, seed=0)
     feats, signals = synth.encoder_inputs(scene)
@@ -480,7 +484,7 @@ def train_step_latency(torch, synth, dev, voxels=200_000, reps=3):
     sig = torch.from_numpy(signals).to(dev)
     labels = (vox.coords[:, 3] // 8 % 13).long()
     torch.manual_seed(0)
-    model = encoder.Swin3DUNet(**encoder.SWIN3D_S, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=1,
+    model = encoder.Swin3DUNet(**encoder.SWIN3D_S, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=fp16_mode,
                                upsample="linear_attn", num_classes=13).to(dev).train()
     opt = torch.optim.SGD(model.parameters(), lr=1e-3)
 
@@ -505,7 +509,7 @@ def train_step_latency(torch, synth, dev, voxels=200_000, reps=3):
     return {"ms": float(np.median(times)), "ms_all": times, "voxels": int(scene.coords.shape[0]),
             "loss_finite": bool(torch.isfinite(loss).item()),
             "config": "Swin3D-S UNet (channels [48,96,192,384,384], heads [6,6,12,24,24], depths [2,4,9,4,4]), "
-                      "one room, fp16_mode 1, forward + backward + SGD"}
+                      f"one room, fp16_mode {fp16_mode}, forward + backward + SGD"}
 
 
 def cpu_baseline(q, k, v, tables, sizes, index, n_crse, num_m):
