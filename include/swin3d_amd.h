@@ -36,6 +36,10 @@ extern "C" {
 /* element type of q/k/v, the tables and the attention output */
 #define S3D_DTYPE_F32 0
 #define S3D_DTYPE_F16 1
+/* s3d_attn_bwd only: fp32 tables beside fp16 rows (q, k, v, out, dout, dq, dk, dv): the backward of an fp16 forward
+ * computed in fp32, as PrecisionMode.HALF_FORWARD asks (Swin3D/sparse_dl/attn/attn_coff.py:206-215 casts the rows
+ * up and the gradients down; here they are widened as they are loaded and rounded as they are stored) */
+#define S3D_DTYPE_F32_F16_ROWS 2
 
 /* largest K of s3d_knn (K_MAX of Swin3D/src/knn/knn_cuda_kernel.cu:4) */
 #define S3D_KNN_KMAX 64
@@ -194,6 +198,9 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *                  more time).  A value below M cannot hold the records of every window: the rows of dq, dk, dv
  *                  that belong to the windows beyond it and all three table gradients then come out as NaN.
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs) bytes
+ *   dtype          S3D_DTYPE_F32, S3D_DTYPE_F16, or S3D_DTYPE_F32_F16_ROWS: the tables fp32, every [N,H,D] tensor
+ *                  fp16, the results those of dtype S3D_DTYPE_F32 on fp32 copies of the rows with dq, dk, dv
+ *                  rounded to fp16 (dq, dk, dv bit for bit); needs pairs > 0
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
  * No global atomics.  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on

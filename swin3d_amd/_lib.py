@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libswin3d_amd.so")
 
 S3D_DTYPE_F32 = 0
 S3D_DTYPE_F16 = 1
+S3D_DTYPE_F32_F16_ROWS = 2     # s3d_attn_bwd only: fp32 tables beside fp16 rows
 KNN_KMAX = 64
 S3D_ATTN_FORCE_GENERIC = 1
 S3D_ATTN_FORCE_MFMA = 2

@@ -981,6 +981,9 @@ int launch_sweep(const BwdArgs &a, int grid, hipStream_t stream)
     return launch_sweep_blk<T, D, ND, KEY_OWNED, MODE, ND>(a, grid, stream);
 }
 
+// T is the type of the feature rows (q, k, v, out, dout, dq, dk, dv); the tables have it too unless dtype says
+// that they are fp32 beside fp16 rows: the pair sweeps, the only kernels of the pair form that read tables, are
+// chosen by dtype, the other kernels of that form read rows and records only.
 template <typename T, int D, int ND>
 int launch_bwd(const BwdArgs &a, const BwdPairArgs &pairs, int dtype, hipStream_t stream)
 {
@@ -1096,8 +1099,11 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     if (D != 8 && D != 16) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8 or 16)", D);
     if (W > 0x7fffffffLL || N > 0x7fffffffLL || H > 65535)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: N, W must fit 31 bits and H 16 bits");
-    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16)
-        return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16 && dtype != S3D_DTYPE_F32_F16_ROWS)
+        return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16, 2 = fp32 on fp16 rows)", dtype);
+    if (dtype == S3D_DTYPE_F32_F16_ROWS && pairs == 0)
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: fp32 arithmetic on fp16 rows (dtype 2) needs the pair count; "
+                    "without it pass fp32 copies of the rows with dtype 0");
     if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: table_sizes (host) is null");
     BwdArgs a{};
     a.H = H;
@@ -1164,7 +1170,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     }
 #define S3D_BWD_CASE(DD, NN)                                                              \
     if (D == DD && nd == NN)                                                              \
-        return dtype == S3D_DTYPE_F16 ? launch_bwd<__half, DD, NN>(a, pr, dtype, s) : launch_bwd<float, DD, NN>(a, pr, dtype, s);
+        return dtype == S3D_DTYPE_F32 ? launch_bwd<float, DD, NN>(a, pr, dtype, s) : launch_bwd<__half, DD, NN>(a, pr, dtype, s);
     S3D_BWD_CASE(8, 3) S3D_BWD_CASE(8, 6) S3D_BWD_CASE(8, 9)
     S3D_BWD_CASE(16, 3) S3D_BWD_CASE(16, 6) S3D_BWD_CASE(16, 9)
 #undef S3D_BWD_CASE

@@ -700,7 +700,11 @@ __global__ __launch_bounds__((group_threads<T, D, HP>()), (groups_per_cu<T, D, H
 // the lanes of a window write consecutive addresses.
 template <typename T, int D, int HP> __host__ __device__ constexpr int bwd_pair_threads() { return 256; }
 
-template <typename T, int D, int ND, int HP, bool kKeyOwned, bool kShared>
+// TF is the type the feature rows are stored in (q, k, v, dout and the gradients dq, dk, dv); T the type of the
+// tables and of the arithmetic.  TF = __half with T = float serves an fp16 forward whose backward runs in fp32: the
+// rows are widened as they are loaded and the gradients rounded as they are stored, the arithmetic is that of T = TF
+// = float on widened copies.
+template <typename T, typename TF, int D, int ND, int HP, bool kKeyOwned, bool kShared>
 // Wavefronts per SIMD, by register cap.  fp16 at head_dim 8: four (128 registers; -1 to -2 % against the three that
 // the key-owned sweep's 133 registers allow).  fp16 at head_dim 16 and fp32 at head_dim 8: three (168 registers, 3 to
 // 20 of them spilled: the backward of the window-7 layer with 6 heads of 16 2.05 -> 1.99 ms, of the headline layer
@@ -739,10 +743,10 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 ? (
     __syncthreads();   // the only workgroup barrier
 
     const int lane = threadIdx.x & 63;
-    const T *gq = static_cast<const T *>(a.q);
-    const T *gk = static_cast<const T *>(a.k);
-    const T *gv = static_cast<const T *>(a.v);
-    const T *ggo = static_cast<const T *>(b.dout);
+    const TF *gq = static_cast<const TF *>(a.q);
+    const TF *gk = static_cast<const TF *>(a.k);
+    const TF *gv = static_cast<const TF *>(a.v);
+    const TF *ggo = static_cast<const TF *>(b.dout);
     const char *ws = static_cast<const char *>(a.workspace);
     const int4 *unit_info = reinterpret_cast<const int4 *>(ws + ws_units_offset(H));
     const int4 *entries = reinterpret_cast<const int4 *>(ws + ws_entries_offset(H, a.N));
@@ -957,10 +961,10 @@ __global__ __launch_bounds__((bwd_pair_threads<T, D, HP>()), (sizeof(T) == 2 ? (
                 }
                 const int64_t at_row = static_cast<int64_t>(own_row) * HD + (h + hh) * D;
                 if constexpr (kKeyOwned) {
-                    store_row<D>(static_cast<T *>(b.dk) + at_row, res_x[hh]);
-                    store_row<D>(static_cast<T *>(b.dv) + at_row, res_y[hh]);
+                    store_row<D>(static_cast<TF *>(b.dk) + at_row, res_x[hh]);
+                    store_row<D>(static_cast<TF *>(b.dv) + at_row, res_y[hh]);
                 } else {
-                    store_row<D>(static_cast<T *>(b.dq) + at_row, res_x[hh]);
+                    store_row<D>(static_cast<TF *>(b.dq) + at_row, res_x[hh]);
                 }
             }
         }
@@ -1072,7 +1076,7 @@ int dispatch_shape(const AttnArgs &a, hipStream_t stream, int what)
 
 namespace {
 
-template <typename T, int D, int ND, int HP, bool kShared>
+template <typename T, typename TF, int D, int ND, int HP, bool kShared>
 int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
 {
     const AttnArgs &a = b0.f;
@@ -1080,8 +1084,8 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
     if (lds > 160 * 1024)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
-    auto q_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, false, kShared>;
-    auto k_sweep = attn_bwd_pairs_kernel<T, D, ND, HP, true, kShared>;
+    auto q_sweep = attn_bwd_pairs_kernel<T, TF, D, ND, HP, false, kShared>;
+    auto k_sweep = attn_bwd_pairs_kernel<T, TF, D, ND, HP, true, kShared>;
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
     int per_cu = 1;
     for (auto kernel : {q_sweep, k_sweep}) {
@@ -1117,7 +1121,7 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
     return S3D_OK;
 }
 
-template <typename T, int D, int ND>
+template <typename T, typename TF, int D, int ND>
 int launch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
 {
     // one head per wavefront: with two (fp16, head_dim 8) the key-owned sweep needs more than 256 registers and the
@@ -1131,15 +1135,15 @@ int launch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
     // backward, own values / shared: 1.76 / 1.87 ms on 26-voxel windows (6 heads of 8), 2.24 / 2.12 and 2.33 / 2.25
     // ms on the window-7 layers of 57 voxels a window (6 heads of 16, 12 of 8).  Shared where the mean window has
     // more than 32 voxels.
-    if (b.f.N > 32 * b.f.W) return launch_bwd_pairs_heads<T, D, ND, 1, true>(b, stream);
-    return launch_bwd_pairs_heads<T, D, ND, 1, false>(b, stream);
+    if (b.f.N > 32 * b.f.W) return launch_bwd_pairs_heads<T, TF, D, ND, 1, true>(b, stream);
+    return launch_bwd_pairs_heads<T, TF, D, ND, 1, false>(b, stream);
 }
 
-template <typename T>
+template <typename T, typename TF>
 int dispatch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
 {
 #define S3D_CASE(DD, NN) \
-    if (b.f.D == DD && b.f.nd == NN) return launch_bwd_pairs<T, DD, NN>(b, stream);
+    if (b.f.D == DD && b.f.nd == NN) return launch_bwd_pairs<T, TF, DD, NN>(b, stream);
     S3D_CASE(8, 3) S3D_CASE(8, 6) S3D_CASE(8, 9)
     S3D_CASE(16, 3) S3D_CASE(16, 6) S3D_CASE(16, 9)
 #undef S3D_CASE
@@ -1151,9 +1155,10 @@ int dispatch_bwd_pairs(const BwdPairArgs &b, hipStream_t stream)
 int launch_attn_bwd_pairs(const BwdPairArgs &b, int dtype, hipStream_t stream)
 {
     switch (dtype) {
-    case S3D_DTYPE_F32: return dispatch_bwd_pairs<float>(b, stream);
-    case S3D_DTYPE_F16: return dispatch_bwd_pairs<__half>(b, stream);
-    default: return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16)", dtype);
+    case S3D_DTYPE_F32: return dispatch_bwd_pairs<float, float>(b, stream);
+    case S3D_DTYPE_F16: return dispatch_bwd_pairs<__half, __half>(b, stream);
+    case S3D_DTYPE_F32_F16_ROWS: return dispatch_bwd_pairs<float, __half>(b, stream);
+    default: return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16, 2 = fp32 on fp16 rows)", dtype);
     }
 }
 

@@ -96,6 +96,8 @@ template <typename T, int D> struct Slice;
 template <int D> struct Slice<float, D> {
     float x[D];
     __device__ __forceinline__ void load(const float *p) { load_row<D>(p, x); }
+    // a row stored in fp16, widened as it is loaded (fp32 arithmetic on fp16 features)
+    __device__ __forceinline__ void load(const __half *p) { load_row<D>(p, x); }
     __device__ __forceinline__ void load_lds(uint32_t addr)
     {
 #pragma unroll

@@ -298,7 +298,9 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
                               out, out_max, out_sum, dout, pairs=None):
     """Gradients of window_attention_forward -> (dq, dk, dv [N,H,D] in the dtype of q,
     dtable_q, dtable_k, dtable_v flat fp32).  out / out_max / out_sum are the forward's results
-    (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes.
+    (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes.  The tables have the dtype of q, or
+    are fp32 beside fp16 features: the backward of an fp16 forward computed in fp32 (PrecisionMode.HALF_FORWARD,
+    attn_coff.py:206-215), whose results are those of fp32 copies of the features with dq, dk, dv rounded to fp16.
 
     pairs: M = sum(w_sizes^2) of the window set (the reference's index arrays have this length,
     swin3d_layers.py:96-103); None = read it from w_sizes once and keep it on that tensor.  With it the library
@@ -329,10 +331,12 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
                          f"to the table length {table_len}")
     if sum(sizes) // (h * d) > BWD_MAX_ROWS_PER_AXIS * nd:
         raise NotImplementedError(f"attention backward supports at most {BWD_MAX_ROWS_PER_AXIS * nd} table rows per head")
+    mixed = q.dtype == torch.float16 and table_q.dtype == torch.float32
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
-        if t.dtype != q.dtype or t.numel() != table_len:
-            raise ValueError(f"{name} must have the dtype of the features and {table_len} elements")
+        if t.dtype != table_q.dtype or (t.dtype != q.dtype and not mixed) or t.numel() != table_len:
+            raise ValueError(f"{name} must have the dtype of the features (or float32 beside float16 features) "
+                             f"and {table_len} elements")
     for name, t in (("out_max", out_max), ("out_sum", out_sum)):
         _require_cuda(name, t, dev)
         if t.dtype != torch.float32 or t.shape != (n, h):
@@ -344,11 +348,6 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
         raise ValueError(f"n_coords must be float32 [{n},{nd}]")
     c_sizes = (ctypes.c_int32 * nd)(*sizes)
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
-    dtq, dtk, dtv = (torch.empty(table_len, dtype=torch.float32, device=dev) for _ in range(3))
-    lib = _lib.lib()
-    tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
-    out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
     if pairs is None:
         pairs = _pairs_of(w_sizes_in, w_sizes) if BWD_PAIR_STORE else 0
     pairs = int(pairs)
@@ -356,6 +355,16 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
         raise ValueError(f"pairs = {pairs}")
     if 12 * pairs * h > BWD_PAIR_STORE_MAX_BYTES:
         pairs = 0
+    code = _lib.S3D_DTYPE_F32_F16_ROWS if mixed else _DTYPE_CODE[q.dtype]
+    if mixed and pairs == 0:
+        # the fused sweeps take one dtype: fp32 copies of the features, the gradients rounded afterwards
+        q, k, v, out, dout = (t.float() for t in (q, k, v, out, dout))
+        code = _lib.S3D_DTYPE_F32
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    dtq, dtk, dtv = (torch.empty(table_len, dtype=torch.float32, device=dev) for _ in range(3))
+    lib = _lib.lib()
+    tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
+    out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
     with torch.cuda.device(dev):
         ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, n, w_sizes.numel(), pairs)
         workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -364,9 +373,11 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
             *(t.data_ptr() for t in tensors), c_sizes, nd, table_len, w_sizes.data_ptr(), w2n.data_ptr(),
             n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(), out_max.data_ptr(), out_sum.data_ptr(),
             dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dtq.data_ptr(), dtk.data_ptr(),
-            dtv.data_ptr(), n, h, d, w_sizes.numel(), pairs, _DTYPE_CODE[q.dtype], workspace.data_ptr(), ws_bytes,
+            dtv.data_ptr(), n, h, d, w_sizes.numel(), pairs, code, workspace.data_ptr(), ws_bytes,
             stream)
     _lib.check(status, "s3d_attn_bwd")
+    if mixed and code == _lib.S3D_DTYPE_F32:
+        dq, dk, dv = dq.half(), dk.half(), dv.half()
     return dq, dk, dv, dtq, dtk, dtv
 
 
@@ -436,10 +447,16 @@ class SelfAttnAIOFunction(Function):
         c_dtype = dout.dtype if ctx.precision == PrecisionMode.HALF_ALL else torch.float32
         if c_dtype not in _DTYPE_CODE:
             raise NotImplementedError(f"compute dtype {c_dtype} is not supported (float16 / float32)")
-        feats = [t.to(c_dtype).contiguous() for t in raw[:3]]
+        # fp32 arithmetic on fp16 tensors (HALF_FORWARD under autocast): the library widens the rows as it loads
+        # them, where the reference makes fp32 copies
+        f_dtype = c_dtype
+        if c_dtype == torch.float32 and dout.dtype == torch.float16 and out.dtype == torch.float16 \
+                and all(t.dtype == torch.float16 for t in raw[:3]):
+            f_dtype = torch.float16
+        feats = [t.to(f_dtype).contiguous() for t in raw[:3]]
         tables = [t.to(c_dtype).contiguous() for t in raw[3:]]
         grads = window_attention_backward(*feats, *tables, ctx.table_sizes, w_sizes, w2n, n2n, n_coords,
-                                          out.to(c_dtype), omax, osum, dout.to(c_dtype).contiguous(),
+                                          out.to(f_dtype), omax, osum, dout.to(f_dtype).contiguous(),
                                           pairs=ctx.pairs)
         grads = [g.to(t.dtype).reshape(t.shape) if need else None
                  for g, t, need in zip(grads, raw, ctx.needs_input_grad[:6])]

@@ -147,6 +147,74 @@ def test_random_shapes(oracle_lib, hip_lib, seed):
     _check(oracle_lib, case, torch.float32 if seed % 2 == 0 else torch.float16, seed=seed)
 
 
+@pytest.mark.parametrize("heads,dim,ws,cRSE", [(6, 8, 5, "XYZ_RGB_NORM"), (3, 16, 7, "XYZ_RGB_NORM"), (2, 16, 7, "XYZ"),
+                                               (4, 8, 3, "XYZ_RGB")])
+def test_fp32_arithmetic_on_fp16_rows(oracle_lib, hip_lib, heads, dim, ws, cRSE):
+    """fp16 features beside fp32 tables (the backward of an fp16 forward computed in fp32, PrecisionMode.HALF_FORWARD,
+    Swin3D/sparse_dl/attn/attn_coff.py:206-215): dq, dk, dv are, bit for bit, the fp32 call's on fp32 copies of the
+    features rounded to fp16; the table gradients agree with that call's as two calls of one form do, and with the
+    oracle at the fp32 tolerance.  Without a pair count the operator makes the copies itself."""
+    import swin3d_amd
+    case = make_attn_case(oracle_lib, seed=91, n=1500 if ws < 7 else 2500, ws=ws, quant=4, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(10, 10, 3) if ws < 7 else (14, 14, 5))
+    case.v *= np.float32(0.4)
+    case.tv *= np.float32(0.2)
+    for name in ("q", "k", "v"):                       # fp16 features, fp32 tables
+        setattr(case, name, getattr(case, name).astype(np.float16).astype(np.float32))
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    feats16 = [t(x).half() for x in (case.q, case.k, case.v)]
+    tables = [t(x) for x in (case.tq, case.tk, case.tv)]
+    idx = (t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
+    # the forward as HALF_FORWARD runs it: fp16 everywhere
+    out, omax, osum = swin3d_amd.window_attention_forward(*feats16, *[x.half() for x in tables], *idx, return_stats=True)
+    dout = torch.from_numpy(np.random.default_rng(92).standard_normal(case.q.shape).astype(np.float32)).to(dev).half()
+    wide = swin3d_amd.window_attention_backward(*[x.float() for x in feats16], *tables, *idx, out.float(), omax, osum,
+                                                dout.float())
+    mixed = swin3d_amd.window_attention_backward(*feats16, *tables, *idx, out, omax, osum, dout)
+    fused = swin3d_amd.window_attention_backward(*feats16, *tables, *idx, out, omax, osum, dout, pairs=0)
+    torch.cuda.synchronize()
+    for name, g, w, f in zip(NAMES[:3], mixed, wide, fused):
+        assert g.dtype == torch.float16 and f.dtype == torch.float16, name
+        assert torch.equal(g, w.half()), name
+    scale = max(float(w.abs().max()) for w in wide[3:])
+    for name, g, w, f in zip(NAMES[3:], mixed[3:], wide[3:], fused[3:]):
+        assert g.dtype == torch.float32, name
+        assert float((g - w).abs().max()) <= 1e-5 * scale, name
+        assert float((f - w).abs().max()) <= 2e-5 * scale, name
+    # against the oracle, which gets what the kernels got: the fp16 output of the fp16 forward enters dout . o
+    ref = oracle_lib.attn_bwd(*case.oracle_args(), dout.float().cpu().numpy())
+    got = [g.double().cpu().numpy() for g in mixed]
+    _assert_close(got, ref, torch.float16)
+
+
+def test_fp16_rows_without_a_pair_count_are_refused_by_the_library(hip_lib):
+    """dtype S3D_DTYPE_F32_F16_ROWS exists in the pair form only: the C entry point says so instead of reading fp16
+    rows as fp32."""
+    import ctypes
+    from swin3d_amd import _lib, crse
+    dev = torch.device("cuda")
+    n, heads, dim = 64, 2, 8
+    sizes = crse.crse_table_sizes(5, 4, heads, dim, "XYZ")
+    table_len = int(sum(sizes))
+    rows = torch.zeros((n, heads, dim), dtype=torch.float16, device=dev)
+    table = torch.zeros(table_len, device=dev)
+    stats = torch.ones((n, heads), device=dev)
+    ints = torch.zeros(n, dtype=torch.int32, device=dev)
+    coords = torch.zeros((n, 3), device=dev)
+    lib = _lib.lib()
+    ws_bytes = lib.s3d_attn_bwd_workspace_bytes(heads, dim, 3, n, 1, 0)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    c_sizes = (ctypes.c_int32 * 3)(*sizes)
+    p = lambda x: x.data_ptr()
+    status = lib.s3d_attn_bwd(p(rows), p(rows), p(rows), p(table), p(table), p(table), c_sizes, 3, table_len, p(ints),
+                              p(ints), p(ints), p(coords), p(rows), p(stats), p(stats), p(rows), p(rows), p(rows), p(rows),
+                              p(table), p(table), p(table), n, heads, dim, 1, 0, _lib.S3D_DTYPE_F32_F16_ROWS, p(ws),
+                              ws_bytes, None)
+    assert status == -4 and b"pair count" in lib.s3d_last_error_string()
+
+
 def test_single_voxel_windows(oracle_lib, hip_lib):
     coords = np.array([[0, 0, 0, 0], [0, 50, 0, 0], [0, 51, 0, 0], [1, 3, 3, 3]], np.int32)
     case = make_attn_case(oracle_lib, seed=64, n=4, ws=5, quant=4, heads=1, dim=8, cRSE="XYZ")
@@ -172,7 +240,8 @@ def test_empty_input(hip_lib):
 
 @pytest.mark.parametrize("precision_name", ["HALF_NONE", "HALF_ALL"])
 def test_autograd_function(oracle_lib, hip_lib, precision_name):
-    """loss.backward() through SelfAttnAIOFunction with the reference's argument list."""
+    """loss.backward() through SelfAttnAIOFunction with the reference's argument list (fp32 leaves; fp16 features
+    from a layer under autocast with HALF_FORWARD: test_autograd_half_forward_on_fp16_features)."""
     from swin3d_amd.sparse_dl.attn.attn_coff import (SelfAttnAIOFunction, PosEmb, TableDims, IndexMode,
                                                      PrecisionMode)
     case = make_attn_case(oracle_lib, seed=65, n=500, ws=5, quant=4, heads=6, dim=8, extent=(8, 8, 3))
@@ -200,6 +269,42 @@ def test_autograd_function(oracle_lib, hip_lib, precision_name):
     got = [leaf.grad.double().cpu().numpy() for leaf in leaves]
     assert all(leaf.grad.dtype == torch.float32 for leaf in leaves)
     _assert_close(got, ref, torch.float16 if half else torch.float32)
+
+
+def test_autograd_half_forward_on_fp16_features(oracle_lib, hip_lib):
+    """HALF_FORWARD as a layer under autocast uses it: q, k, v arrive in fp16 (the output of an autocast linear
+    layer), the tables are fp32 parameters; the forward runs in fp16 and the backward in fp32 on the fp16 tensors.
+    The feature gradients come back in fp16 and equal, bit for bit, those of fp32 leaves holding the same values
+    rounded to fp16 (the reference's own way through this mode: copies cast up, gradients cast down)."""
+    from swin3d_amd.sparse_dl.attn.attn_coff import (SelfAttnAIOFunction, PosEmb, TableDims, IndexMode,
+                                                     PrecisionMode)
+    case = make_attn_case(oracle_lib, seed=67, n=1500, ws=5, quant=4, heads=6, dim=8, extent=(9, 9, 3))
+    case.v *= np.float32(0.4)
+    case.tv *= np.float32(0.2)
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    indices = [None, t(i["w_sizes"]).long(), None, t(i["w2n"]).long(), t(i["n2n"]).long(), t(case.n_coords)]
+    dout = t(np.random.default_rng(68).standard_normal(case.q.shape).astype(np.float32)).half()
+
+    def grads_of(feat_dtype):
+        feats = [t(a).half().to(feat_dtype).requires_grad_(True) for a in (case.q, case.k, case.v)]
+        tables = [t(a).requires_grad_(True) for a in (case.tq, case.tk, case.tv)]
+        with torch.autocast("cuda", dtype=torch.float16):
+            out = SelfAttnAIOFunction.apply(*feats, *tables, case.table_sizes.tolist(), indices, PosEmb.SEPARATE,
+                                            TableDims.D0, IndexMode.INDIRECT, PrecisionMode.HALF_FORWARD)
+        assert out.dtype == torch.float16
+        out.backward(dout)
+        torch.cuda.synchronize()
+        return [x.grad for x in feats + tables]
+
+    half, wide = grads_of(torch.float16), grads_of(torch.float32)
+    for name, h, w in zip(NAMES[:3], half, wide):
+        assert h.dtype == torch.float16 and w.dtype == torch.float32, name
+        assert torch.equal(h, w.half()), name
+    scale = max(float(w.abs().max()) for w in wide[3:])
+    for name, h, w in zip(NAMES[3:], half[3:], wide[3:]):
+        assert h.dtype == torch.float32 and float((h - w).abs().max()) <= 1e-5 * scale, name
 
 
 def test_headline_size_properties(hip_lib):
