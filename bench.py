@@ -82,6 +82,8 @@ def main():
                     help="print the hash of the headline kernel's sources (recorded in the profile summary) and exit")
     ap.add_argument("--train-only", action="store_true",
                     help="run only the Swin3D-S training-step side figure")
+    ap.add_argument("--train-fp16-mode", type=int, choices=(1, 2), default=None,
+                    help="with --train-only: only this fp16_mode (the command the step's kernel trace is taken with)")
     ap.add_argument("--encoder-only", action="store_true",
                     help="run only the Swin3D-L encoder forward (1 warm-up + 3 timed passes, no UNet) and print its "
                          "figures: the command the encoder's kernel trace is taken with")
@@ -108,8 +110,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.train_only:
-        print(json.dumps({"train_step_swin3d_s": train_step_latency(torch, synth, dev),
-                          "train_step_swin3d_s_fp16_mode2": train_step_latency(torch, synth, dev, fp16_mode=2)}))
+        modes = {1: "train_step_swin3d_s", 2: "train_step_swin3d_s_fp16_mode2"}
+        print(json.dumps({name: train_step_latency(torch, synth, dev, fp16_mode=mode) for mode, name in modes.items()
+                          if args.train_fp16_mode in (None, mode)}))
         return 0
     if args.encoder_only:
         print(json.dumps({"encoder_swin3d_l": encoder_latency(torch, synth, dev, unet=False,
