@@ -299,6 +299,12 @@ def main():
                        reps=5, warm=2)
         result["extras"]["attn_bwd"] = {"ms": ms, "pairs_per_s": num_m / (ms * 1e-3),
                                         "vs_forward": ms / kernel_ms, "dtype": "f16 I/O, f32 arithmetic"}
+        # the same with fp32 tables beside the fp16 tensors: the backward of PrecisionMode.HALF_FORWARD
+        mixed_args = fwd_args[:3] + tuple(x.float() for x in fwd_args[3:6]) + fwd_args[6:]
+        ms = _time_gpu(torch, lambda: swin3d_amd.window_attention_backward(*mixed_args, o_d, mx_d, sm_d, dout_d),
+                       reps=5, warm=2)
+        result["extras"]["attn_bwd"]["f32_tables_f16_rows_ms"] = ms
+        del mixed_args
         if not args.no_other_shapes:
             result["extras"]["other_shapes"] = other_shapes(torch, swin3d_amd, synth, crse, scene, dev)
         # the headline layer in fp32, the compute type of the operator when autocast is off (PrecisionMode.HALF_NONE)
