@@ -200,7 +200,8 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs) bytes
  *   dtype          S3D_DTYPE_F32, S3D_DTYPE_F16, or S3D_DTYPE_F32_F16_ROWS: the tables fp32, every [N,H,D] tensor
  *                  fp16, the results those of dtype S3D_DTYPE_F32 on fp32 copies of the rows with dq, dk, dv
- *                  rounded to fp16 (dq, dk, dv bit for bit); needs pairs > 0
+ *                  rounded to fp16 (the same arithmetic; the two launches may pack the windows differently, which
+ *                  reorders the fp32 sums); needs pairs > 0
  *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
  *
  * No global atomics.  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on

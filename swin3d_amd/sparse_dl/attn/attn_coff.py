@@ -300,7 +300,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     dtable_q, dtable_k, dtable_v flat fp32).  out / out_max / out_sum are the forward's results
     (return_stats=True) for the same inputs; arithmetic is fp32 for both dtypes.  The tables have the dtype of q, or
     are fp32 beside fp16 features: the backward of an fp16 forward computed in fp32 (PrecisionMode.HALF_FORWARD,
-    attn_coff.py:206-215), whose results are those of fp32 copies of the features with dq, dk, dv rounded to fp16.
+    attn_coff.py:206-215), whose results are those of fp32 copies of the features with dq, dk, dv rounded to fp16
+    (to the rounding of the fp32 sums).
 
     pairs: M = sum(w_sizes^2) of the window set (the reference's index arrays have this length,
     swin3d_layers.py:96-103); None = read it from w_sizes once and keep it on that tensor.  With it the library
