@@ -154,7 +154,7 @@ def test_random_shapes(oracle_lib, hip_lib, seed):
 
 
 @pytest.mark.parametrize("heads,dim,ws,cRSE", [(6, 8, 5, "XYZ_RGB_NORM"), (3, 16, 7, "XYZ_RGB_NORM"), (2, 16, 7, "XYZ"),
-                                               (4, 8, 3, "XYZ_RGB")])
+                                               (4, 8, 3, "XYZ_RGB"), (20, 16, 7, "XYZ_RGB_NORM")])
 def test_fp32_arithmetic_on_fp16_rows(oracle_lib, hip_lib, heads, dim, ws, cRSE):
     """fp16 features beside fp32 tables (the backward of an fp16 forward computed in fp32, PrecisionMode.HALF_FORWARD,
     Swin3D/sparse_dl/attn/attn_coff.py:206-215): dq, dk, dv are the fp32 call's on fp32 copies of the features,
