@@ -30,6 +30,18 @@ def test_python_signatures_cover_the_header(hip_lib):
     assert sorted(_lib.SIGNATURES) == _declared_symbols()
 
 
+def test_python_constants_equal_the_header():
+    """The codes that the ctypes layer passes are the header's #defines."""
+    from swin3d_amd import _lib
+    text = open(os.path.join(ROOT, "include", "swin3d_amd.h")).read()
+    defines = {name: int(value, 0) for name, value in re.findall(r"^#define (S3D_[A-Z0-9_]+) \(?(-?(?:0x)?[0-9a-fA-F]+)\)?\s*(?:/\*.*)?$",
+                                                              text, flags=re.M)}
+    for name in ("S3D_DTYPE_F32", "S3D_DTYPE_F16", "S3D_DTYPE_F32_F16_ROWS", "S3D_ATTN_FORCE_GENERIC",
+                 "S3D_ATTN_FORCE_MFMA", "S3D_ATTN_PLANNED", "S3D_ATTN_SIZES_ON_DEVICE"):
+        assert defines[name] == getattr(_lib, name), name
+    assert defines["S3D_KNN_KMAX"] == _lib.KNN_KMAX
+
+
 def test_version_and_error_string(hip_lib):
     assert hip_lib.s3d_version() >= 100
     assert isinstance(hip_lib.s3d_last_error_string(), bytes)
