@@ -197,20 +197,27 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  *                  sweeps that recompute the logits for the table gradients and need no such store (about a third
  *                  more time).  A value below M cannot hold the records of every window: the rows of dq, dk, dv
  *                  that belong to the windows beyond it and all three table gradients then come out as NaN.
- *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs) bytes
+ *   workspace      device scratch of at least s3d_attn_bwd_workspace_bytes(H, D, nd, table_len, N, W, pairs) bytes
  *   dtype          S3D_DTYPE_F32, S3D_DTYPE_F16, or S3D_DTYPE_F32_F16_ROWS: the tables fp32, every [N,H,D] tensor
  *                  fp16, the results those of dtype S3D_DTYPE_F32 on fp32 copies of the rows with dq, dk, dv
  *                  rounded to fp16 (the same arithmetic; the two launches may pack the windows differently, which
  *                  reorders the fp32 sums); needs pairs > 0
- *   D in {8,16}, nd in {3,6,9}, at most 64 * nd table rows per head in total.
+ *   D in {8,16,32}, nd in {3,6,9}.  head_dim 32 and tables of more than 64 * nd rows per head in total (quant 8
+ *                  with wide windows) run in a general form in the manner of the reference - one thread per
+ *                  (query, head), atomic adds for dk, dv (fp32 accumulators in the workspace) and for the table
+ *                  gradients (per workgroup in LDS, then global), so only dq is then the same bits on every
+ *                  call; `pairs` is ignored.  It is some fifty times slower per pair than the forms described
+ *                  here (0.2 s for 200 000 voxels at head_dim 32) and exists so that every shape of the forward
+ *                  has a backward; its workspace is 8 * N * H * D bytes plus the statistics.
  *
- * No global atomics.  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on
+ * No global atomics (the general form apart).  dq, dk, dv have one owning lane per row and are sums in a fixed order: the same bits on
  * every call.  The table gradients are accumulated per wavefront over the units it draws from the work queues,
  * left in a slot of the workspace and summed per head, slots in order, by a reduction kernel: which units a
  * wavefront draws varies from call to call, so these sums are regrouped and agree between calls to fp32 rounding
  * (about 1e-6 of the largest element), not bit for bit.
  */
-size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t N, int64_t W, int64_t pairs);
+size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D, int32_t nd, int64_t table_len, int64_t N, int64_t W,
+                                    int64_t pairs);
 int s3d_attn_bwd(const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
                  const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
                  const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords,

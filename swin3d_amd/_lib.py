@@ -36,7 +36,7 @@ SIGNATURES = {
     "s3d_attn_plan": (ctypes.c_int, [_vp, _i32, _i64, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_attn_fwd_noalloc": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
                              [_i64, _i32, _i32, _i64, _i64, _i32, _vp]),
-    "s3d_attn_bwd_workspace_bytes": (ctypes.c_size_t, [_i32, _i32, _i32, _i64, _i64, _i64]),
+    "s3d_attn_bwd_workspace_bytes": (ctypes.c_size_t, [_i32, _i32, _i32, _i64, _i64, _i64, _i64]),
     # q k v tq tk tv sizes | nd len | w_sizes w2n n2n coords out max sum dout dq dk dv dtq dtk dtv | N H D W pairs dtype | ws bytes stream
     "s3d_attn_bwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 14 +
                      [_i64, _i32, _i32, _i64, _i64, _i32, _vp, ctypes.c_size_t, _vp]),

@@ -883,6 +883,220 @@ __global__ __launch_bounds__(256) void bwd_reduce_tables_kernel(BwdArgs a, float
     if (share == 0) dst[(static_cast<size_t>(row) * H + h) * D + c] = sum;
 }
 
+
+// ---- the general form ---------------------------------------------------------------------------------------
+// Shapes that the register-blocked kernels above do not cover - head_dim 32, or more than 64 table rows per axis
+// on average (quant 8 with wide windows) - in the manner of the reference (Swin3D/src/attn/self_attn_aio_bwd.cu:
+// 197-509, one thread per term and a global atomic for each): a thread owns one (window-sorted position, head),
+// walks the keys of its window, keeps dq_i in registers and adds the other terms atomically - dk_j and dv_j into
+// fp32 accumulators in global memory that a second kernel rounds to the output type (the lanes of a wavefront start
+// at different keys, so that they do not meet on one row), the table gradients into a copy of the head's three
+// tables in LDS (a workgroup serves one head and leaves its sums with global atomics at the end; kLdsTables = false,
+// for tables beyond 160 KB per head: global atomics for every term).  No work list; the order of the atomic adds
+// varies, so only dq is the same bits on every call.  Bound by the LDS atomics (27 D per pair and head): 205 ms for
+// 200 000 voxels in windows of 5 at 6 heads of 32 channels, 11.5 ms for 50 000 voxels at window 7, quant 8, 6 heads
+// of 8 with position tables only - some fifty times the forms above per pair; it exists so that every shape the
+// forward takes has a backward.  T: type of the feature rows, TT: of the tables.
+constexpr int kGeneralThreads = 256;
+
+template <typename T, typename TT, int D, bool kLdsTables>
+__global__ __launch_bounds__(kGeneralThreads) void attn_bwd_general_kernel(BwdArgs a, float *dk_acc, float *dv_acc)
+{
+    extern __shared__ float general_tables[];      // [flat row][q-side, k-side, v-side][D] sums of this workgroup
+    const int H = a.H, nd = a.nd;
+    const int64_t HD = static_cast<int64_t>(H) * D;
+    const int h = blockIdx.x % H;
+    const int slot = blockIdx.x / H, slots = gridDim.x / H;
+    const T *gq = static_cast<const T *>(a.q), *gk = static_cast<const T *>(a.k), *gv = static_cast<const T *>(a.v);
+    const T *ggo = static_cast<const T *>(a.dout);
+    const TT *tq = static_cast<const TT *>(a.table_q), *tk = static_cast<const TT *>(a.table_k);
+    const TT *tv = static_cast<const TT *>(a.table_v);
+    if constexpr (kLdsTables) {
+        for (int t = threadIdx.x; t < a.total_rows * 3 * D; t += kGeneralThreads) general_tables[t] = 0.0f;
+        __syncthreads();
+    }
+    // chunks of kGeneralThreads consecutive window-sorted positions, dealt to the workgroups of the head in turn
+    const int64_t chunks = (a.N + kGeneralThreads - 1) / kGeneralThreads;
+    for (int64_t chunk = slot; chunk < chunks; chunk += slots) {
+        const int64_t pos = chunk * kGeneralThreads + threadIdx.x;
+        if (pos >= a.N) continue;
+        // the window of the position: the last one that starts at or before it
+        int64_t lo = 0, hi = a.W - 1;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi + 1) >> 1;
+            if (a.w2n[mid] <= pos) lo = mid;
+            else hi = mid - 1;
+        }
+        const int n_w = a.w_sizes[lo], s0 = a.w2n[lo];
+        const int i = static_cast<int>(pos - s0);
+        if (i >= n_w) continue;      // positions that no window covers (none for a valid index)
+        const int qi = a.n2n[pos];
+        const int64_t q_at = static_cast<int64_t>(qi) * HD + h * D;
+        float q[D], go[D], dq[D], ci[kMaxAxes];
+#pragma unroll
+        for (int c = 0; c < D; c += 8) {
+            load_row<8>(gq + q_at + c, q + c);
+            load_row<8>(ggo + q_at + c, go + c);
+        }
+#pragma unroll
+        for (int c = 0; c < D; ++c) dq[c] = 0.0f;
+        for (int n = 0; n < nd; ++n) ci[n] = a.n_coords[pos * nd + n];
+        const float m_i = a.out_max[static_cast<int64_t>(qi) * H + h];
+        const float inv_i = 1.0f / a.out_sum[static_cast<int64_t>(qi) * H + h];
+        const float delta_i = a.delta[static_cast<int64_t>(qi) * H + h];
+        for (int step = 0; step < n_w; ++step) {
+            int j = i + step;                      // every query starts at its own key
+            if (j >= n_w) j -= n_w;
+            const int kj = a.n2n[s0 + j];
+            const int64_t k_at = static_cast<int64_t>(kj) * HD + h * D;
+            float kr[D], vs[D], tqs[D], tks[D];
+#pragma unroll
+            for (int c = 0; c < D; c += 8) {
+                load_row<8>(gk + k_at + c, kr + c);
+                load_row<8>(gv + k_at + c, vs + c);
+            }
+#pragma unroll
+            for (int c = 0; c < D; ++c) tqs[c] = tks[c] = 0.0f;
+            int row[kMaxAxes];
+            for (int n = 0; n < nd; ++n) {
+                const float cj = a.n_coords[static_cast<int64_t>(s0 + j) * nd + n];
+                row[n] = a.base[n] + crse_row(ci[n], cj, static_cast<float>(a.rows[n] / 2), crse_upper(a.rows[n]));
+                const int64_t row_at = static_cast<int64_t>(row[n]) * HD + h * D;
+#pragma unroll
+                for (int c = 0; c < D; c += 8) {
+                    float x[8], y[8], z[8];
+                    load_row<8>(tq + row_at + c, x);
+                    load_row<8>(tk + row_at + c, y);
+                    load_row<8>(tv + row_at + c, z);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        tqs[c + e] += x[e];
+                        tks[c + e] += y[e];
+                        vs[c + e] += z[e];
+                    }
+                }
+            }
+            float logit = 0.0f, dp = 0.0f;
+#pragma unroll
+            for (int c = 0; c < D; ++c) {
+                logit += q[c] * (kr[c] + tqs[c]) + kr[c] * tks[c];
+                dp += go[c] * vs[c];
+            }
+            const float p = __expf(logit - m_i) * inv_i;
+            const float dl = p * (dp - delta_i);
+#pragma unroll
+            for (int c = 0; c < D; ++c) {
+                dq[c] += dl * (kr[c] + tqs[c]);
+                atomicAdd(dk_acc + k_at + c, dl * (q[c] + tks[c]));
+                atomicAdd(dv_acc + k_at + c, p * go[c]);
+            }
+            for (int n = 0; n < nd; ++n) {
+                if constexpr (kLdsTables) {
+                    float *cell = general_tables + row[n] * 3 * D;
+#pragma unroll
+                    for (int c = 0; c < D; ++c) {
+                        atomicAdd(cell + c, dl * q[c]);
+                        atomicAdd(cell + D + c, dl * kr[c]);
+                        atomicAdd(cell + 2 * D + c, p * go[c]);
+                    }
+                } else {
+                    const int64_t row_at = static_cast<int64_t>(row[n]) * HD + h * D;
+#pragma unroll
+                    for (int c = 0; c < D; ++c) {
+                        atomicAdd(a.dtq + row_at + c, dl * q[c]);
+                        atomicAdd(a.dtk + row_at + c, dl * kr[c]);
+                        atomicAdd(a.dtv + row_at + c, p * go[c]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < D; c += 8) store_row<8>(static_cast<T *>(a.dq) + q_at + c, dq + c);
+    }
+    if constexpr (kLdsTables) {
+        __syncthreads();
+        for (int t = threadIdx.x; t < a.total_rows * 3 * D; t += kGeneralThreads) {
+            const int r = t / (3 * D), rest = t - r * (3 * D), which = rest / D, c = rest - which * D;
+            float *dst = which == 0 ? a.dtq : which == 1 ? a.dtk : a.dtv;
+            const float sum = general_tables[t];
+            if (sum != 0.0f) atomicAdd(dst + static_cast<int64_t>(r) * HD + h * D + c, sum);
+        }
+    }
+}
+
+__global__ void bwd_general_zero_kernel(float *x, int64_t count)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < count; t += stride) x[t] = 0.0f;
+}
+
+// dk, dv from their fp32 accumulators, eight channels per thread
+template <typename T>
+__global__ void bwd_general_store_kernel(BwdArgs a, const float *dk_acc, const float *dv_acc)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    const int64_t pieces = a.N * a.H * a.D / 8;
+    for (int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; t < pieces; t += stride) {
+        float x[8], y[8];
+        load_row<8>(dk_acc + 8 * t, x);
+        load_row<8>(dv_acc + 8 * t, y);
+        store_row<8>(static_cast<T *>(a.dk) + 8 * t, x);
+        store_row<8>(static_cast<T *>(a.dv) + 8 * t, y);
+    }
+}
+
+// head_dim 32, or more table rows than the register blocks of the table-gradient kernels cover
+inline bool bwd_general_form(int H, int D, int nd, int64_t table_len)
+{
+    return D == 32 || table_len / (static_cast<int64_t>(H) * D) > 64 * nd;
+}
+size_t bwd_general_acc_bytes(int64_t N, int H, int D) { return align_up(sizeof(float) * static_cast<size_t>(N) * H * D, 256); }
+
+template <typename T, typename TT, int D>
+int launch_bwd_general_dim(const BwdArgs &a, float *dk_acc, float *dv_acc, hipStream_t stream)
+{
+    const int64_t work = a.N * a.H + a.table_len;
+    const int prep_grid = static_cast<int>(ceil_div(work, 256) < 4096 ? ceil_div(work, 256) : 4096);
+    hipLaunchKernelGGL(bwd_prepare_kernel<T>, dim3(static_cast<unsigned>(prep_grid)), dim3(256), 0, stream, a);
+    const int64_t count = 2 * static_cast<int64_t>(bwd_general_acc_bytes(a.N, a.H, a.D) / sizeof(float));
+    hipLaunchKernelGGL(bwd_general_zero_kernel, dim3(2048), dim3(256), 0, stream, dk_acc, count);
+    S3D_HIP_CHECK(hipGetLastError());
+    // workgroups: about four per CU, a whole number per head, no more than the chunks of positions give work to
+    const size_t lds = sizeof(float) * static_cast<size_t>(a.total_rows) * 3 * D;
+    const int64_t chunks = (a.N + kGeneralThreads - 1) / kGeneralThreads;
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus < 1)
+        cus = 256;
+    int64_t per_head = (4 * cus + a.H - 1) / a.H;
+    if (per_head > chunks) per_head = chunks;
+    if (per_head < 1) per_head = 1;
+    const unsigned grid = static_cast<unsigned>(per_head * a.H);
+    if (lds <= 160 * 1024) {
+        auto kernel = attn_bwd_general_kernel<T, TT, D, true>;
+        S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kGeneralThreads), lds, stream, a, dk_acc, dv_acc);
+    } else {
+        hipLaunchKernelGGL((attn_bwd_general_kernel<T, TT, D, false>), dim3(grid), dim3(kGeneralThreads), 0, stream, a,
+                           dk_acc, dv_acc);
+    }
+    hipLaunchKernelGGL(bwd_general_store_kernel<T>, dim3(2048), dim3(256), 0, stream, a, dk_acc, dv_acc);
+    S3D_HIP_CHECK(hipGetLastError());
+    return S3D_OK;
+}
+
+template <typename T, typename TT>
+int launch_bwd_general(const BwdArgs &a, float *dk_acc, float *dv_acc, hipStream_t stream)
+{
+    switch (a.D) {
+    case 8: return launch_bwd_general_dim<T, TT, 8>(a, dk_acc, dv_acc, stream);
+    case 16: return launch_bwd_general_dim<T, TT, 16>(a, dk_acc, dv_acc, stream);
+    case 32: return launch_bwd_general_dim<T, TT, 32>(a, dk_acc, dv_acc, stream);
+    default: return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8, 16 or 32)", a.D);
+    }
+}
+
 template <typename T, int D>
 size_t bwd_lds_bytes(const BwdArgs &a, int kinds, int blk)
 {
@@ -1039,8 +1253,6 @@ int fill_bwd_axes(BwdArgs &a, const int32_t *table_sizes, int nd, int64_t table_
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: sum(table_sizes) = %lld differs from table_len = %lld",
                     (long long)total, (long long)table_len);
     a.total_rows = base;
-    if (base > 64 * nd)
-        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d table rows per head (at most %d)", base, 64 * nd);
     return S3D_OK;
 }
 
@@ -1071,11 +1283,14 @@ size_t bwd_dlt_bytes(int H, int64_t pairs) { return align_up(sizeof(float) * sta
 }  // namespace s3d
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_bytes(int32_t H, int32_t D,
-                                                                                      int32_t nd, int64_t N,
-                                                                                      int64_t W, int64_t pairs)
+                                                                                      int32_t nd, int64_t table_len,
+                                                                                      int64_t N, int64_t W,
+                                                                                      int64_t pairs)
 {
     using namespace s3d;
-    if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || N < 0 || W < 0 || pairs < 0) return 0;
+    if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || table_len < 1 || N < 0 || W < 0 || pairs < 0) return 0;
+    if (bwd_general_form(H, D, nd, table_len))
+        return bwd_units_bytes(W, N, H, 0) + bwd_delta_bytes(N, H) + 2 * bwd_general_acc_bytes(N, H, D);
     size_t need = bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
     if (pairs > 0)
         need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_generic_workspace_bytes(H, W, N), 256);
@@ -1096,12 +1311,13 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
                     (long long)N, (long long)W, H, D, nd, (long long)table_len, (long long)pairs);
     if (nd != 3 && nd != 6 && nd != 9)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: %d cRSE axes (3, 6 or 9)", nd);
-    if (D != 8 && D != 16) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8 or 16)", D);
+    if (D != 8 && D != 16 && D != 32) return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: head_dim %d (8, 16 or 32)", D);
     if (W > 0x7fffffffLL || N > 0x7fffffffLL || H > 65535)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_bwd: N, W must fit 31 bits and H 16 bits");
     if (dtype != S3D_DTYPE_F32 && dtype != S3D_DTYPE_F16 && dtype != S3D_DTYPE_F32_F16_ROWS)
         return fail(S3D_ERR_BAD_DTYPE, "s3d_attn_bwd: dtype %d (0 = fp32, 1 = fp16, 2 = fp32 on fp16 rows)", dtype);
-    if (dtype == S3D_DTYPE_F32_F16_ROWS && pairs == 0)
+    const bool general = bwd_general_form(H, D, nd, table_len);
+    if (dtype == S3D_DTYPE_F32_F16_ROWS && pairs == 0 && !general)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_bwd: fp32 arithmetic on fp16 rows (dtype 2) needs the pair count; "
                     "without it pass fp32 copies of the rows with dtype 0");
     if (!table_sizes) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: table_sizes (host) is null");
@@ -1115,7 +1331,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     if (int rc = fill_bwd_axes(a, table_sizes, nd, table_len)) return rc;
     if (!dtable_q || !dtable_k || !dtable_v)
         return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null table-gradient pointer");
-    const size_t need = s3d_attn_bwd_workspace_bytes(H, D, nd, N, W, pairs);
+    const size_t need = s3d_attn_bwd_workspace_bytes(H, D, nd, table_len, N, W, pairs);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_bwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
@@ -1130,6 +1346,27 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.dtq = dtable_q; a.dtk = dtable_k; a.dtv = dtable_v;
     a.units = static_cast<int32_t *>(workspace);
+    if (general) {
+        // the form for shapes outside the register-blocked kernels: units | delta | dk accumulator | dv accumulator
+        hipStream_t gs = static_cast<hipStream_t>(stream);
+        a.pairs = 0;
+        if (N == 0 || W == 0) {
+            a.N = 0;
+            hipLaunchKernelGGL((bwd_prepare_kernel<float>), dim3(64), dim3(256), 0, gs, a);
+            S3D_HIP_CHECK(hipGetLastError());
+            return S3D_OK;
+        }
+        char *g_at = static_cast<char *>(workspace) + bwd_units_bytes(W, N, H, 0);
+        a.delta = reinterpret_cast<float *>(g_at);
+        g_at += bwd_delta_bytes(N, H);
+        float *dk_acc = reinterpret_cast<float *>(g_at);
+        float *dv_acc = reinterpret_cast<float *>(g_at + bwd_general_acc_bytes(N, H, D));
+        switch (dtype) {
+        case S3D_DTYPE_F32: return launch_bwd_general<float, float>(a, dk_acc, dv_acc, gs);
+        case S3D_DTYPE_F16: return launch_bwd_general<__half, __half>(a, dk_acc, dv_acc, gs);
+        default: return launch_bwd_general<__half, float>(a, dk_acc, dv_acc, gs);
+        }
+    }
     a.delta = reinterpret_cast<float *>(static_cast<char *>(workspace) + bwd_units_bytes(W, N, H, pairs));
     char *at = static_cast<char *>(workspace) + bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H);
     a.tgrad = reinterpret_cast<float *>(at);

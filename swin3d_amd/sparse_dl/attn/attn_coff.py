@@ -47,10 +47,11 @@ _DTYPE_CODE = {torch.float32: _lib.S3D_DTYPE_F32, torch.float16: _lib.S3D_DTYPE_
 # (window_attention_backward): switch, and the size above which it runs the fused sweeps instead
 BWD_PAIR_STORE = True
 BWD_PAIR_STORE_MAX_BYTES = 32 << 30
-# s3d_attn_bwd keeps a head's table gradients in registers: at most 64 rows per axis on average, head_dim 8 or 16
-# (the forward also takes head_dim 32)
+# s3d_attn_bwd keeps a head's table gradients in registers where they fit: at most 64 rows per axis on average and
+# head_dim 8 or 16.  Beyond that (and at head_dim 32) the library runs its general form, which adds with global
+# atomics as the reference does and is many times slower.
 BWD_MAX_ROWS_PER_AXIS = 64
-BWD_HEAD_DIMS = (8, 16)
+BWD_HEAD_DIMS = (8, 16, 32)
 
 # debugging / ablation switch: run the generic VALU kernel even where the MFMA kernel applies
 FORCE_GENERIC = False
@@ -321,7 +322,7 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
         if t.shape != q.shape or t.dtype != q.dtype:
             raise ValueError(f"{name} must match query: {tuple(t.shape)} {t.dtype}")
     if d not in BWD_HEAD_DIMS:
-        raise NotImplementedError(f"attention backward supports head_dim 8 and 16, got {d}")
+        raise NotImplementedError(f"attention backward supports head_dim 8, 16 and 32, got {d}")
     sizes = _host_table_sizes(table_sizes)
     nd = len(sizes)
     if nd not in (3, 6, 9):
@@ -330,8 +331,7 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     if any(sz <= 0 or sz % (h * d) for sz in sizes) or sum(sizes) != table_len:
         raise ValueError(f"table_sizes {sizes} must be positive multiples of H*D = {h * d} that sum "
                          f"to the table length {table_len}")
-    if sum(sizes) // (h * d) > BWD_MAX_ROWS_PER_AXIS * nd:
-        raise NotImplementedError(f"attention backward supports at most {BWD_MAX_ROWS_PER_AXIS * nd} table rows per head")
+    general = d == 32 or sum(sizes) // (h * d) > BWD_MAX_ROWS_PER_AXIS * nd     # the library's general form
     mixed = q.dtype == torch.float16 and table_q.dtype == torch.float32
     for name, t in (("query_table", table_q), ("key_table", table_k), ("value_table", table_v)):
         _require_cuda(name, t, dev)
@@ -357,7 +357,7 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     if 12 * pairs * h > BWD_PAIR_STORE_MAX_BYTES:
         pairs = 0
     code = _lib.S3D_DTYPE_F32_F16_ROWS if mixed else _DTYPE_CODE[q.dtype]
-    if mixed and pairs == 0:
+    if mixed and pairs == 0 and not general:
         # the fused sweeps take one dtype: fp32 copies of the features, the gradients rounded afterwards
         q, k, v, out, dout = (t.float() for t in (q, k, v, out, dout))
         code = _lib.S3D_DTYPE_F32
@@ -367,7 +367,7 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     tensors = [t.contiguous() for t in (q, k, v, table_q, table_k, table_v)]
     out, dout, out_max, out_sum, n_coords = (t.contiguous() for t in (out, dout, out_max, out_sum, n_coords))
     with torch.cuda.device(dev):
-        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, n, w_sizes.numel(), pairs)
+        ws_bytes = lib.s3d_attn_bwd_workspace_bytes(h, d, nd, table_len, n, w_sizes.numel(), pairs)
         workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream(dev).cuda_stream
         status = lib.s3d_attn_bwd(
@@ -415,15 +415,8 @@ class SelfAttnAIOFunction(Function):
             # the backward's limits, reported where the op is called and not from inside autograd
             if raw_query_feats.shape[2] not in BWD_HEAD_DIMS:
                 raise NotImplementedError(
-                    f"attention backward supports head_dim 8 and 16, got {raw_query_feats.shape[2]}; run the forward "
-                    "under torch.no_grad()")
-            sizes = _host_table_sizes(table_offsets)
-            rows = sum(sizes) // max(raw_query_feats.shape[1] * raw_query_feats.shape[2], 1)
-            if rows > BWD_MAX_ROWS_PER_AXIS * len(sizes):
-                raise NotImplementedError(
-                    f"attention backward supports at most {BWD_MAX_ROWS_PER_AXIS} table rows per axis on average "
-                    f"({BWD_MAX_ROWS_PER_AXIS * len(sizes)} per head for {len(sizes)} axes), got {rows}; "
-                    "run the forward under torch.no_grad() or use smaller tables")
+                    f"attention backward supports head_dim 8, 16 and 32, got {raw_query_feats.shape[2]}; run the "
+                    "forward under torch.no_grad()")
         res = window_attention_forward(*feats, *tables, table_offsets, w_sizes, w2n, n2n, n_coords,
                                        return_stats=needs_grad)
         if not needs_grad:

@@ -77,14 +77,21 @@ def test_more_argument_errors_without_a_device(hip_lib):
     st = hip_lib.s3d_attn_bwd(*([None] * 6), c_sizes, 9, total, *([None] * 14), 10, 6, 8, 1, 0, 1, None, 0, None)
     assert st < 0 and (b"gradient pointer" in hip_lib.s3d_last_error_string()
                        or b"workspace" in hip_lib.s3d_last_error_string())
-    # backward: more table rows per head than its registers cover (window 10 at quant 8)
-    big = crse.crse_table_sizes(10, 8, 6, 8, "XYZ_RGB_NORM")
-    c_big = (ctypes.c_int32 * 9)(*big)
-    st = hip_lib.s3d_attn_bwd(*([None] * 6), c_big, 9, sum(big), *([None] * 14), 10, 6, 8, 1, 0, 1, None, 0, None)
-    assert st < 0 and b"table rows per head" in hip_lib.s3d_last_error_string()
-    assert hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, 1000, 40, 0) >= 4 * (40 + 6) + 4 * 6000
-    assert (hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, 1000, 40, 30000) >=
-            hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, 1000, 40, 0) + 12 * 6 * 30000)
+    # backward: a head_dim that no form covers
+    small = crse.crse_table_sizes(5, 4, 6, 24, "XYZ_RGB_NORM")
+    c_small = (ctypes.c_int32 * 9)(*small)
+    st = hip_lib.s3d_attn_bwd(*([None] * 6), c_small, 9, sum(small), *([None] * 14), 10, 6, 24, 1, 0, 1, None, 0, None)
+    assert st < 0 and b"head_dim 24" in hip_lib.s3d_last_error_string()
+    table_len = sum(crse.crse_table_sizes(5, 4, 6, 8, "XYZ_RGB_NORM"))
+    assert hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, table_len, 1000, 40, 0) >= 4 * (40 + 6) + 4 * 6000
+    assert (hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, table_len, 1000, 40, 30000) >=
+            hip_lib.s3d_attn_bwd_workspace_bytes(6, 8, 9, table_len, 1000, 40, 0) + 12 * 6 * 30000)
+    # the general form (head_dim 32; more table rows per head than the register blocks cover, window 10 at quant 8):
+    # fp32 accumulators of dk and dv, no pair store
+    big = sum(crse.crse_table_sizes(10, 8, 6, 8, "XYZ_RGB_NORM"))
+    for dim, length in ((32, table_len * 4), (8, big)):
+        need = hip_lib.s3d_attn_bwd_workspace_bytes(6, dim, 9, length, 1000, 40, 30000)
+        assert 2 * 4 * 1000 * 6 * dim + 4 * 6000 <= need <= 2 * 4 * 1000 * 6 * dim + 4 * 6000 + (1 << 20)
     st = hip_lib.s3d_knn_interpolate(None, None, 0, 10, None, 10, 8, 0, None, None)
     assert st < 0 and b"K=0" in hip_lib.s3d_last_error_string()
     st = hip_lib.s3d_knn_interpolate(None, None, 3, 10, None, 10, 8, 7, None, None)

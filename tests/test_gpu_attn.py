@@ -388,11 +388,14 @@ def test_head_dim_32_forward(oracle_lib, hip_lib, dtype, heads, ws, cRSE, shift)
         import ctypes
         c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
         assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, 32, 1, 343000, 1000) == 0
+        # the backward of this head_dim is the library's general form (checked against the oracle in
+        # test_gpu_attn_bwd.py::test_general_form): here only that autograd reaches it
         leaves = [x.clone().requires_grad_() for x in feats]
-        with pytest.raises(NotImplementedError):
-            attn_coff.SelfAttnAIOFunction.apply(*leaves, sizes, (None, index[0], None, index[1], index[2], index[3]),
-                                                attn_coff.PosEmb.SEPARATE, attn_coff.TableDims.D0,
-                                                attn_coff.IndexMode.INDIRECT, attn_coff.PrecisionMode.HALF_NONE)
+        out = attn_coff.SelfAttnAIOFunction.apply(*leaves, sizes, (None, index[0], None, index[1], index[2], index[3]),
+                                                  attn_coff.PosEmb.SEPARATE, attn_coff.TableDims.D0,
+                                                  attn_coff.IndexMode.INDIRECT, attn_coff.PrecisionMode.HALF_NONE)
+        out.sum().backward()
+        assert all(x.grad is not None and bool(torch.isfinite(x.grad).all()) for x in leaves)
 
 
 def test_fp32_elementwise_bound_report(oracle_lib, hip_lib, capsys):

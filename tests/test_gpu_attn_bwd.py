@@ -215,7 +215,7 @@ def test_fp16_rows_without_a_pair_count_are_refused_by_the_library(hip_lib):
     ints = torch.zeros(n, dtype=torch.int32, device=dev)
     coords = torch.zeros((n, 3), device=dev)
     lib = _lib.lib()
-    ws_bytes = lib.s3d_attn_bwd_workspace_bytes(heads, dim, 3, n, 1, 0)
+    ws_bytes = lib.s3d_attn_bwd_workspace_bytes(heads, dim, 3, table_len, n, 1, 0)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     c_sizes = (ctypes.c_int32 * 3)(*sizes)
     p = lambda x: x.data_ptr()
@@ -224,6 +224,55 @@ def test_fp16_rows_without_a_pair_count_are_refused_by_the_library(hip_lib):
                               p(table), p(table), p(table), n, heads, dim, 1, 0, _lib.S3D_DTYPE_F32_F16_ROWS, p(ws),
                               ws_bytes, None)
     assert status == -4 and b"pair count" in lib.s3d_last_error_string()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("ws,quant,heads,dim,cRSE", [
+    (5, 4, 3, 32, "XYZ_RGB_NORM"),    # head_dim 32
+    (7, 4, 2, 32, "XYZ"),
+    (7, 8, 2, 8, "XYZ"),              # 112 rows per axis: more than the register blocks of the table-gradient kernels
+    (10, 4, 2, 16, "XYZ"),            # window 10: 80 rows on each of the three position axes
+])
+def test_general_form(oracle_lib, hip_lib, dtype, ws, quant, heads, dim, cRSE):
+    """head_dim 32 and tables of more than 64 rows per axis on average run in the library's general form (global
+    atomic adds, as the reference works); the pair count is ignored there."""
+    from swin3d_amd.sparse_dl.attn import attn_coff
+    case = make_attn_case(oracle_lib, seed=400 + ws + dim, n=800, ws=ws, quant=quant, heads=heads, dim=dim, cRSE=cRSE,
+                          extent=(10, 10, 4))
+    rows = int(sum(case.table_sizes)) // (heads * dim)
+    assert dim == 32 or rows > attn_coff.BWD_MAX_ROWS_PER_AXIS * len(case.table_sizes)
+    if dtype == torch.float16:
+        case.v *= np.float32(0.4)
+        case.tv *= np.float32(0.2)
+    _check(oracle_lib, case, dtype)
+
+
+def test_general_form_on_fp16_rows_with_fp32_tables(oracle_lib, hip_lib):
+    """The general form under PrecisionMode.HALF_FORWARD: fp16 tensors, fp32 tables, against the fp32 call on copies."""
+    import swin3d_amd
+    case = make_attn_case(oracle_lib, seed=433, n=800, ws=5, quant=4, heads=3, dim=32, cRSE="XYZ_RGB_NORM",
+                          extent=(10, 10, 4))
+    case.v *= np.float32(0.4)
+    case.tv *= np.float32(0.2)
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    feats16 = [t(x).half() for x in (case.q, case.k, case.v)]
+    tables = [t(x) for x in (case.tq, case.tk, case.tv)]
+    idx = (t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
+    out, omax, osum = swin3d_amd.window_attention_forward(*feats16, *[x.half() for x in tables], *idx, return_stats=True)
+    dout = torch.from_numpy(np.random.default_rng(434).standard_normal(case.q.shape).astype(np.float32)).to(dev).half()
+    wide = swin3d_amd.window_attention_backward(*[x.float() for x in feats16], *tables, *idx, out.float(), omax, osum,
+                                                dout.float())
+    mixed = swin3d_amd.window_attention_backward(*feats16, *tables, *idx, out, omax, osum, dout)
+    torch.cuda.synchronize()
+    row_scale = max(float(w.abs().max()) for w in wide[:3])
+    for name, g, w in zip(NAMES[:3], mixed, wide):
+        assert g.dtype == torch.float16, name
+        assert bool(((g.float() - w).abs() <= _half_rounding(w, row_scale) + 2e-5 * row_scale).all()), name
+    scale = max(float(w.abs().max()) for w in wide[3:])
+    for name, g, w in zip(NAMES[3:], mixed[3:], wide[3:]):
+        assert g.dtype == torch.float32 and float((g - w).abs().max()) <= 2e-5 * scale, name
 
 
 def test_single_voxel_windows(oracle_lib, hip_lib):

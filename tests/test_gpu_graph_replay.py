@@ -94,7 +94,7 @@ def test_backward_replays_equal_eager_calls(oracle_lib, hip_lib):
     dout = torch.randn_like(out)
     grads = [torch.empty_like(x["q"]) for _ in range(3)] + [torch.empty(table_len, dtype=torch.float32, device="cuda")
                                                            for _ in range(3)]
-    nbytes = hip_lib.s3d_attn_bwd_workspace_bytes(h, d, len(sizes), n, w, pairs)
+    nbytes = hip_lib.s3d_attn_bwd_workspace_bytes(h, d, len(sizes), table_len, n, w, pairs)
     workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     side = torch.cuda.Stream()      # default priority
 
