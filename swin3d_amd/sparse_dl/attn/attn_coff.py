@@ -308,7 +308,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
     swin3d_layers.py:96-103); None = read it from w_sizes once and keep it on that tensor.  With it the library
     runs the pair sweeps, which keep dL and P of every (pair, head) in the workspace (12 bytes each); 0, or a
     store above BWD_PAIR_STORE_MAX_BYTES, selects the fused sweeps, which need no such store and take about a
-    third longer."""
+    third longer.  head_dim 32 and tables of more than BWD_MAX_ROWS_PER_AXIS rows per axis on average run in the
+    library's general form (atomic adds, as the reference works): correct, some fifty times slower per pair."""
     w_sizes_in = w_sizes
     _require_cuda("query", q)
     dev = q.device
