@@ -27,7 +27,7 @@ SETTLE_MS = 80.0         # untimed, continuous launches before every timed regio
 SETTLE = {"ms": SETTLE_MS}
 HEADLINE_PROFILE = os.path.join("profiles", "attn_fwd_headline.txt")
 # the sources of the headline kernel: counter figures taken from a profile are only quoted while these are unchanged
-KERNEL_SOURCES = ["attn_fwd.hip", "attn_fwd_generic.hip", "attn_kernels.h", "sweep_common.h", "s3d_common.h"]
+KERNEL_SOURCES = ["attn_fwd.hip", "attn_sweep.hip", "attn_kernels.h", "sweep_common.h", "s3d_common.h"]
 
 
 def kernel_sources_sha256():
@@ -70,7 +70,6 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="untimed launches after the warm-up steps until the card has been busy this long (0 = none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--flags", type=int, default=0, help="s3d_attn_fwd flags (0 = the library picks, 1 = sweep kernel, 2 = MFMA kernel)")
     ap.add_argument("--no-extras", action="store_true", help="skip the KNN / window-index side figures")
     ap.add_argument("--no-other-shapes", action="store_true",
                     help="skip the window-7 layers of the side figures (a profile then holds the headline layer's kernels only)")
@@ -142,50 +141,52 @@ def main():
     c_sizes = (ctypes.c_int32 * nd)(*sizes)
     out = torch.empty_like(q_d)
     num_w, num_m = index.num_windows, index.num_pairs
-    ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, heads, dim, n, num_w, index.max_window_voxels)
+    ws_bytes = lib.s3d_attn_fwd_workspace_bytes(heads, n, num_w)
     workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev)
 
     # The sweep kernel's work list depends on the window set only; like the index arrays it is built once per set
     # and shared by the blocks that use the set (s3d_attn_plan), so the timed call runs on a prebuilt plan.  The
     # same call with the list built inside it is timed beside it (kernel_ms.with_list_build).
-    planned = args.flags == 0 and not lib.s3d_attn_fwd_uses_mfma(c_sizes, nd, heads, dim, _lib.S3D_DTYPE_F16, n, num_w)
     plan = torch.empty(max(lib.s3d_attn_plan_bytes(heads, n, num_w), 1), dtype=torch.uint8, device=dev)
-    if planned:
-        _lib.check(lib.s3d_attn_plan(c_sizes, nd, table_len, index.w_sizes.data_ptr(), index.w2n.data_ptr(), n, heads, dim,
-                                     num_w, _lib.S3D_DTYPE_F16, plan.data_ptr(), plan.numel(), stream.cuda_stream),
-                   "s3d_attn_plan")
+    _lib.check(lib.s3d_attn_plan(c_sizes, nd, table_len, index.w_sizes.data_ptr(), index.w2n.data_ptr(), n, heads, dim,
+                                 num_w, _lib.S3D_DTYPE_F16, plan.data_ptr(), plan.numel(), stream.cuda_stream),
+               "s3d_attn_plan")
 
-    def step(use_plan=planned):
+    def step(use_plan=True):
         status = lib.s3d_attn_fwd(q_d.data_ptr(), k_d.data_ptr(), v_d.data_ptr(), tq_d.data_ptr(),
                                   tk_d.data_ptr(), tv_d.data_ptr(), c_sizes, nd, table_len,
                                   index.w_sizes.data_ptr(), index.w2n.data_ptr(), index.n2n.data_ptr(),
                                   n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16,
-                                  (args.flags | _lib.S3D_ATTN_PLANNED) if use_plan else args.flags,
+                                  0, _lib.S3D_DTYPE_F16, _lib.S3D_ATTN_PLANNED if use_plan else 0,
                                   plan.data_ptr() if use_plan else workspace.data_ptr(),
                                   plan.numel() if use_plan else ws_bytes, stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")
 
+    def timed_launches(count):
+        """per-launch times (ms) of `count` calls enqueued back to back, from events on the launch stream (torch's
+        current stream), and the wall clock per call"""
+        starts = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        ends = [torch.cuda.Event(enable_timing=True) for _ in range(count)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(count):
+            starts[i].record(stream)
+            step()
+            ends[i].record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return np.array([s.elapsed_time(e) for s, e in zip(starts, ends)]), (t1 - t0) * 1e3 / count
+
     for _ in range(args.warmup):
         step()
-    # ... and further untimed launches until the card has been busy for args.settle_ms (its clocks settle)
+    # the regime of a run that goes straight from the warm-up steps into its timed region (--settle-ms 0): the card
+    # has been busy for a few milliseconds only.  Reported beside the headline figure, never as the headline.
+    unsettled_ms, _ = timed_launches(args.steps)
+    # ... then further untimed launches until the card has been busy for args.settle_ms (its clocks settle)
     settle_launches = _settle(torch, step)
-    torch.cuda.synchronize()
-    # per-launch kernel time from events on the launch stream (torch's current stream)
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        starts[i].record(stream)
-        step()
-        ends[i].record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / args.steps
-    launch_ms = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+    launch_ms, wall_ms = timed_launches(args.steps)
     kernel_ms = float(launch_ms.mean())
 
     bytes_alg = algorithmic_bytes(n, channels, 2, nd, num_w, table_len)
@@ -215,24 +216,28 @@ def main():
         },
         "voxels_per_s": n / (wall_ms * 1e-3),
         "kernel_ms": {"mean": kernel_ms, "median": float(np.median(launch_ms)),
-                      "p10": float(np.percentile(launch_ms, 10)), "p90": float(np.percentile(launch_ms, 90))},
+                      "p10": float(np.percentile(launch_ms, 10)), "p90": float(np.percentile(launch_ms, 90)),
+                      # the same K launches timed right after the warm-up steps, before the settling launches
+                      "unsettled": {"median": float(np.median(unsettled_ms)), "mean": float(unsettled_ms.mean())}},
         # achieved / frac: algorithmic bytes of this run over the launch time measured in this run.  traffic is a
         # counter figure: it is quoted from the committed profile only while the kernel sources are the ones the
         # profile was taken with (from_profile says so), and is null otherwise
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": bytes_alg},
     }
+    result["roofline"]["unsettled_frac"] = bytes_alg / (float(unsettled_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBPS
     figures, current = profile_figures()
-    if args.flags == 0 and figures:
+    if figures:
         result["roofline"]["from_profile"] = {
             "file": HEADLINE_PROFILE, "sources_sha256": figures.get("sources_sha256"),
             "matches_sources_in_tree": current,
             "sweep_kernel_us": float(figures["sweep_kernel_us"]) if "sweep_kernel_us" in figures else None}
         if current:
             result["roofline"]["traffic"] = int(figures["traffic_bytes"]) if "traffic_bytes" in figures else None
+            # the unit that binds the kernel (counter figure, same rule): share of the SIMDs' issue cycles that
+            # carry a VALU instruction
             if "valu_issue_frac" in figures:
-                result["roofline"]["from_profile"]["limiter"] = {"kind": "valu_issue",
-                                                                 "frac": float(figures["valu_issue_frac"])}
+                result["roofline"]["binding"] = {"unit": "valu_issue", "frac": float(figures["valu_issue_frac"])}
 
     # cold figure: a 512 MiB fill between launches evicts q/k/v and the tables from L2 and the
     # Infinity Cache (outside the timed steps above; 10 launches)
@@ -248,7 +253,7 @@ def main():
         cold.append(s_ev.elapsed_time(e_ev))
     del flush
     result["kernel_ms"]["cold_median"] = float(np.median(cold))
-    result["kernel_ms"]["planned"] = bool(planned)
+    result["kernel_ms"]["planned"] = True
     def back_to_back(fn, reps=30, warm=5):
         """median launch time as in the timed region above: all calls enqueued, one wait at the end"""
         for _ in range(warm):
@@ -262,21 +267,21 @@ def main():
         torch.cuda.synchronize()
         return float(np.median([s_ev.elapsed_time(e_ev) for s_ev, e_ev in evs]))
 
-    if planned:
-        result["kernel_ms"]["with_list_build"] = back_to_back(lambda: step(use_plan=False))
-    # the same call on rows that are in window order already (q, k, v, out permuted by n2n; n2n = identity):
-    # what a caller gets who keeps a stage's voxels in the order of its regular windows
-    ident = torch.arange(n, dtype=torch.int32, device=dev)
+    # the call that builds its own work list (two small kernels in front of the sweep): what a caller pays who
+    # does not keep a plan
+    unplanned = back_to_back(lambda: step(use_plan=False))
+    result["kernel_ms"]["with_list_build"] = unplanned
+    result["roofline"]["unplanned_frac"] = bytes_alg / (unplanned * 1e-3) / 1e9 / HBM_PEAK_GBPS
+    # the same call on rows that are in window order already (q, k, v, out permuted by n2n) and without a row map
+    # (n2n = NULL): what a caller gets who keeps a stage's voxels in the order of its regular windows
     qs_d, ks_d, vs_d = q_d[order].contiguous(), k_d[order].contiguous(), v_d[order].contiguous()
 
     def step_ordered():
         status = lib.s3d_attn_fwd(qs_d.data_ptr(), ks_d.data_ptr(), vs_d.data_ptr(), tq_d.data_ptr(), tk_d.data_ptr(),
                                   tv_d.data_ptr(), c_sizes, nd, table_len, index.w_sizes.data_ptr(), index.w2n.data_ptr(),
-                                  ident.data_ptr(), n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
-                                  index.max_window_voxels, 0, _lib.S3D_DTYPE_F16,
-                                  (args.flags | _lib.S3D_ATTN_PLANNED) if planned else args.flags,
-                                  plan.data_ptr() if planned else workspace.data_ptr(),
-                                  plan.numel() if planned else ws_bytes, stream.cuda_stream)
+                                  None, n_crse.data_ptr(), out.data_ptr(), None, None, n, heads, dim, num_w,
+                                  0, _lib.S3D_DTYPE_F16, _lib.S3D_ATTN_PLANNED, plan.data_ptr(), plan.numel(),
+                                  stream.cuda_stream)
         if status != 0:
             _lib.check(status, "s3d_attn_fwd")
 

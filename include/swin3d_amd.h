@@ -5,8 +5,9 @@
  * Plain pointers and sizes only: every pointer named "device" is a HIP device
  * address, `stream` is a hipStream_t passed as void* (NULL = the null stream).
  * All entry points enqueue work on `stream` and return without synchronising
- * unless stated otherwise.  The library keeps no device state; every output and
- * every workspace is allocated by the caller.
+ * unless stated otherwise.  Every output and every workspace is allocated by the
+ * caller; the only device memory the library itself holds is the fixed scratch
+ * array of s3d_attn_fwd_noalloc (8 MiB per GPU, part of the code object).
  *
  * Return value: 0 on success, a negative S3D_ERR_* code for a rejected argument,
  * a positive value = the hipError_t of a failed runtime call.  A human readable
@@ -78,30 +79,23 @@ const char *s3d_last_error_string(void);
  *   table_len      elements per table = sum_n table_sizes[n]
  *   w_sizes, w2n   device int32 [W]: voxels per window, exclusive prefix sum
  *   n2n            device int32 [N]: window-sorted position -> original row, or NULL when the rows of q, k,
- *                  v and out are in window-sorted order already (position = row; sweep kernel)
+ *                  v and out are in window-sorted order already (position = row): the kernels then read and
+ *                  write the rows in place, without the gather of Swin3D/src/attn/attn_utils.cuh:391-409
  *   n_coords       device fp32 [N,nd], window-sorted order, scaled by the quant sizes
  *   out            device [N,H,D] of `dtype`: softmax-normalised attention output
  *   out_max        device fp32 [N,H] or NULL: max logit per (voxel, head)
  *                  (the tensor cal_max_coffs returns)
  *   out_sum        device fp32 [N,H] or NULL: sum_j exp(logit - max)
  *                  (second tensor of self_attn_cuda_forward; raw = out * sum)
- *   max_window_voxels  an upper bound of every w_sizes entry (e.g. counts[2] of s3d_window_index, or
- *                  window^3), or 0 when none is known.  Only the MFMA kernel needs it (it sizes the partial
- *                  results of windows of more than 32 voxels with it); without a bound the sweep kernel,
- *                  which takes windows of any size, serves the call.  With an understated bound the MFMA
- *                  kernel fills the rows of the windows beyond it (out, out_max, out_sum) with NaN.
  *   qkv_row_stride elements between consecutive voxel rows of q, k and v (0 = H*D, dense).  A multiple
  *                  of 8 that is >= H*D: with 3*H*D and q, k, v pointing H*D apart the kernels read the
  *                  [N, 3*H*D] output of the qkv projection (Swin3D/modules/swin3d_layers.py:502-509) in
  *                  place, without the reference's reshape / permute / contiguous copy.
- *   flags          0 (the library picks the kernel), S3D_ATTN_FORCE_GENERIC to run the VALU sweep kernel
- *                  for every case, S3D_ATTN_FORCE_MFMA to run the MFMA kernel wherever it applies, or
- *                  S3D_ATTN_PLANNED (sweep kernel on a work list built by s3d_attn_plan, see below)
- *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(...) bytes.  Sweep kernel:
- *                  work-queue counters, one record per unit of 8 to 64 queries and one per window, about
- *                  2 N + 24 W bytes + 0.3 MB.  MFMA kernel: a transposed copy of the value table, the work
- *                  list and N * ceil(max_window_voxels / 32) * H * (D + 2) floats of partial results when
- *                  max_window_voxels > 32.  The size function returns the larger of the two.
+ *   flags          0, or S3D_ATTN_PLANNED (`workspace` holds a work list built by s3d_attn_plan, see below)
+ *                  and / or S3D_ATTN_SIZES_ON_DEVICE (see table_sizes)
+ *   workspace      device scratch of at least s3d_attn_fwd_workspace_bytes(H, N, W) bytes: the work list of the
+ *                  launch (work-queue counters, one record per unit of 8 to 64 queries and one per window, the
+ *                  list builder's notes), about 2 N + 24 W bytes + 0.3 MB whatever the window sizes
  *   w2n must be ascending (the exclusive prefix sum of w_sizes, as the reference builds it:
  *   Swin3D/modules/swin3d_layers.py:100-103).
  *   D in {8,16,32}, nd in {3,6,9}, H >= 1 (the reference takes head_dim up to 32: self_attn_aio_fwd.cu:486).
@@ -113,28 +107,23 @@ const char *s3d_last_error_string(void);
  * the axis table when the clamped value equals rows_n, this library folds that
  * case onto the last row).
  *
- * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.  The sweep kernel adds the
- * value-table rows of a pair three at a time in fp16 before they enter the fp32 sums (the reference's half path
- * adds all of them and the value in half2, Swin3D/src/attn/self_attn_aio_fwd.cu:147).  Every call gives the
- * same bits for the same inputs (no atomics on data, work list in window order).
+ * fp16: inputs, tables and output are fp16; products accumulate in fp32, exp in fp32.  The value-table rows of a
+ * pair are added three at a time in fp16 before they enter the fp32 sums (the reference's half path adds all of
+ * them and the value in half2, Swin3D/src/attn/self_attn_aio_fwd.cu:147).  Every call gives the same bits for the
+ * same inputs (no atomics on data, work list in window order).
+ *
+ * One kernel family serves every shape: persistent workgroups that keep their heads' table slices in LDS, a lane
+ * per query streaming its window's keys (VALU; packed fp16 dot products for fp16 I/O).
  */
-#define S3D_ATTN_FORCE_GENERIC 1
-#define S3D_ATTN_FORCE_MFMA 2
 #define S3D_ATTN_PLANNED 4   /* `workspace` holds a plan written by s3d_attn_plan: see there */
-#define S3D_ATTN_SIZES_ON_DEVICE 8   /* `table_sizes` is a DEVICE int32 [nd] array (sweep kernel; see s3d_attn_fwd) */
-/* 1 if s3d_attn_fwd with flags 0 runs these shapes on the MFMA kernel (fp16, head_dim 16, every axis
- * table <= 64 rows, and windows of at least 256 voxels on average, N >= 256 W, or 60 with 16 heads or more),
- * 0 if on the VALU sweep kernel.  No counterpart in the reference (it has one kernel). */
-int s3d_attn_fwd_uses_mfma(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype,
-                           int64_t N, int64_t W);
-size_t s3d_attn_fwd_workspace_bytes(const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D,
-                                    int64_t N, int64_t W, int32_t max_window_voxels);
+#define S3D_ATTN_SIZES_ON_DEVICE 8   /* `table_sizes` is a DEVICE int32 [nd] array (see s3d_attn_fwd) */
+size_t s3d_attn_fwd_workspace_bytes(int32_t H, int64_t N, int64_t W);
 int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_q,
                  const void *table_k, const void *table_v, const int32_t *table_sizes, int32_t nd,
                  int64_t table_len, const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n,
                  const float *n_coords, void *out, float *out_max, float *out_sum, int64_t N,
-                 int32_t H, int32_t D, int64_t W, int32_t max_window_voxels, int64_t qkv_row_stride,
-                 int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes, void *stream);
+                 int32_t H, int32_t D, int64_t W, int64_t qkv_row_stride, int32_t dtype, int32_t flags,
+                 void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Work list of the sweep kernel, built once per window set ("plan").
@@ -147,7 +136,7 @@ int s3d_attn_fwd(const void *q, const void *k, const void *v, const void *table_
  * the flag S3D_ATTN_PLANNED, for calls with the same w_sizes, w2n, N, W, H, D, dtype and table_sizes.  Such a call
  * runs the sweep kernel and nothing else.  The plan holds the launch's work counters, which a launch leaves at
  * zero again: a plan serves one call at a time (calls in stream order; not two streams at once).
- *   plan           device buffer of at least s3d_attn_plan_bytes(H, N, W) bytes
+ *   plan           device buffer of at least s3d_attn_plan_bytes(H, N, W) bytes (= s3d_attn_fwd_workspace_bytes)
  */
 size_t s3d_attn_plan_bytes(int32_t H, int64_t N, int64_t W);
 int s3d_attn_plan(const int32_t *table_sizes, int32_t nd, int64_t table_len, const int32_t *w_sizes,
@@ -158,12 +147,14 @@ int s3d_attn_plan(const int32_t *table_sizes, int32_t nd, int64_t table_len, con
  * The same forward without a workspace argument and without any allocation.
  *
  * It has no counterpart in the reference.  It is for callers that cannot allocate device memory around the
- * call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Always the sweep
- * kernel (the MFMA kernel's partial results do not fit a fixed buffer); its work list lives in a device array of
- * 8 MiB that is part of the library's code object, one copy per GPU, held until the process ends.  The call
- * fails with S3D_ERR_WORKSPACE when s3d_attn_fwd_workspace_bytes(table_sizes, nd, H, D, N, W, 0) exceeds
- * 8 MiB (about 2 N + 24 W bytes + 0.3 MB: e.g. one million voxels in up to 200 000 windows fit).  The first
- * call on a device looks up the array's address there (hipGetSymbolAddress); no call allocates or frees.
+ * call: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The work list lives
+ * in a device array of 8 MiB that is part of the library's code object, one copy per GPU, held until the process
+ * ends.  The call fails with S3D_ERR_WORKSPACE when s3d_attn_fwd_workspace_bytes(H, N, W) exceeds 8 MiB (about
+ * 2 N + 24 W bytes + 0.3 MB: e.g. one million voxels in up to 200 000 windows fit).  No call allocates or frees.
+ * The first call on a device looks up the array's address there (hipGetSymbolAddress) and the first call of a
+ * shape (dtype, head_dim, axes, heads per wavefront) raises that kernel's dynamic-LDS limit (hipFuncSetAttribute):
+ * neither belongs into a stream capture, so make ONE eager call per device and shape before capturing; the calls
+ * after it enqueue kernels only.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two host
  * threads) race on it and must be serialised by the caller; calls in stream order on one stream are safe,
  * and nothing is carried over from one call to the next.

@@ -13,8 +13,6 @@ S3D_DTYPE_F32 = 0
 S3D_DTYPE_F16 = 1
 S3D_DTYPE_F32_F16_ROWS = 2     # s3d_attn_bwd only: fp32 tables beside fp16 rows
 KNN_KMAX = 64
-S3D_ATTN_FORCE_GENERIC = 1
-S3D_ATTN_FORCE_MFMA = 2
 S3D_ATTN_PLANNED = 4
 S3D_ATTN_SIZES_ON_DEVICE = 8
 
@@ -28,10 +26,9 @@ _i64 = ctypes.c_int64
 SIGNATURES = {
     "s3d_version": (ctypes.c_int, []),
     "s3d_last_error_string": (ctypes.c_char_p, []),
-    "s3d_attn_fwd_uses_mfma": (ctypes.c_int, [_vp, _i32, _i32, _i32, _i32, _i64, _i64]),
-    "s3d_attn_fwd_workspace_bytes": (ctypes.c_size_t, [_vp, _i32, _i32, _i32, _i64, _i64, _i32]),
+    "s3d_attn_fwd_workspace_bytes": (ctypes.c_size_t, [_i32, _i64, _i64]),
     "s3d_attn_fwd": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +
-                     [_i64, _i32, _i32, _i64, _i32, _i64, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
+                     [_i64, _i32, _i32, _i64, _i64, _i32, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_attn_plan_bytes": (ctypes.c_size_t, [_i32, _i64, _i64]),
     "s3d_attn_plan": (ctypes.c_int, [_vp, _i32, _i64, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp, ctypes.c_size_t, _vp]),
     "s3d_attn_fwd_noalloc": (ctypes.c_int, [_vp] * 7 + [_i32, _i64] + [_vp] * 7 +

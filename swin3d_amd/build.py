@@ -12,7 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libswin3d_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["api_common.hip", "attn_fwd.hip", "attn_fwd_generic.hip", "attn_fwd_mfma.hip", "attn_bwd.hip",
+SOURCES = ["api_common.hip", "attn_fwd.hip", "attn_sweep.hip", "attn_bwd.hip",
            "window_index.hip", "knn.hip", "layernorm.hip"]
 
 # packed-fp32 VALU forms are disabled for every device compilation unit

@@ -11,6 +11,6 @@ char *error_buffer()
 
 }  // namespace s3d
 
-extern "C" __attribute__((visibility("default"))) int s3d_version(void) { return 100; }
+extern "C" __attribute__((visibility("default"))) int s3d_version(void) { return 200; }
 
 extern "C" __attribute__((visibility("default"))) const char *s3d_last_error_string(void) { return s3d::error_buffer(); }

@@ -7,7 +7,7 @@
 //   dq_i  += dL (k_j + Tq(i,j))                    dTq[n][row_n(i,j)] += dL q_i
 //   dk_j  += dL (q_i + Tk(i,j))                    dTk[n][row_n(i,j)] += dL k_j
 // The reference adds every term with a global atomic.  Here every output element has ONE owner, and the call has two
-// forms.  With the window set's pair count it runs the pair sweeps of attn_fwd_generic.hip (dq; dk and dv; on the
+// forms.  With the window set's pair count it runs the pair sweeps of attn_sweep.hip (dq; dk and dv; on the
 // forward's packed work list), which leave dL and P of every (pair, head) in the workspace, and the table-gradient
 // kernels below (attn_bwd_tables_kernel), which read them.  Without it, the fused sweeps (attn_bwd_sweep_kernel),
 // which recompute the logits and need no store:
@@ -1293,7 +1293,7 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_
         return bwd_units_bytes(W, N, H, 0) + bwd_delta_bytes(N, H) + 2 * bwd_general_acc_bytes(N, H, D);
     size_t need = bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
     if (pairs > 0)
-        need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_generic_workspace_bytes(H, W, N), 256);
+        need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_sweep_workspace_bytes(H, W, N), 256);
     return need;
 }
 

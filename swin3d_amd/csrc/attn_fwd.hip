@@ -1,4 +1,4 @@
-// Entry point of the windowed self-attention forward: argument checks and kernel choice.
+// Entry points of the windowed self-attention forward: argument checks, work list, launch.
 #include "attn_kernels.h"
 
 #include <mutex>
@@ -10,7 +10,7 @@ int fill_axes(AttnArgs &a, const int32_t *table_sizes, int nd, int64_t table_len
 {
     const int64_t hd = static_cast<int64_t>(a.H) * a.D;
     int64_t total = 0;
-    int base = 0, pbase = 0;
+    int base = 0;
     for (int n = 0; n < nd; ++n) {
         const int64_t size = table_sizes[n];
         if (size <= 0 || size % hd != 0)
@@ -19,16 +19,13 @@ int fill_axes(AttnArgs &a, const int32_t *table_sizes, int nd, int64_t table_len
         total += size;
         a.rows[n] = static_cast<int32_t>(size / hd);
         a.base[n] = base;
-        a.pbase[n] = pbase;
         base += a.rows[n];
-        pbase += (a.rows[n] + 15) / 16 * 16;
     }
-    for (int n = nd; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = a.pbase[n] = 0;
+    for (int n = nd; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = 0;
     if (total != table_len)
         return fail(S3D_ERR_BAD_SHAPE, "s3d_attn_fwd: sum(table_sizes) = %lld differs from table_len = %lld",
                     (long long)total, (long long)table_len);
     a.total_rows = base;
-    a.padded_rows = pbase + 16;
     return S3D_OK;
 }
 
@@ -51,47 +48,10 @@ int check_shape(int64_t N, int64_t W, int32_t H, int32_t D, int32_t nd, int64_t 
 }  // namespace
 }  // namespace s3d
 
-extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_bytes(
-    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int64_t N, int64_t W,
-    int32_t max_window_voxels)
+extern "C" __attribute__((visibility("default"))) size_t s3d_attn_fwd_workspace_bytes(int32_t H, int64_t N, int64_t W)
 {
-    using namespace s3d;
-    if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1) return 0;
-    int64_t padded = 16;
-    for (int n = 0; n < nd; ++n) {
-        const int64_t rows = table_sizes[n] / (static_cast<int64_t>(H) * D);
-        padded += (rows + 15) / 16 * 16;
-    }
-    if (N < 0 || W < 0) return 0;
-    const size_t generic = attn_generic_workspace_bytes(H, W, N);
-    if (max_window_voxels < 1) return generic;      // no bound: the sweep kernel serves the call
-    // the MFMA kernel's share only for shapes it can run (fp16 is not known here)
-    AttnArgs a{};
-    a.H = H;
-    a.D = D;
-    a.nd = nd;
-    int64_t total = 0;
-    for (int n = 0; n < nd; ++n) total += table_sizes[n];
-    if (fill_axes(a, table_sizes, nd, total) != S3D_OK || !attn_mfma_supported(a, S3D_DTYPE_F16)) return generic;
-    const size_t mfma = attn_mfma_workspace_bytes(H, D, static_cast<int>(padded), W, N, max_window_voxels);
-    return mfma > generic ? mfma : generic;
-}
-
-extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_uses_mfma(
-    const int32_t *table_sizes, int32_t nd, int32_t H, int32_t D, int32_t dtype, int64_t N, int64_t W)
-{
-    using namespace s3d;
-    if (!table_sizes || nd < 1 || nd > kMaxAxes || H < 1 || D < 1 || N < 0 || W < 0) return 0;
-    AttnArgs a{};
-    a.H = H;
-    a.D = D;
-    a.nd = nd;
-    a.N = N;
-    a.W = W;
-    int64_t total = 0;
-    for (int n = 0; n < nd; ++n) total += table_sizes[n];
-    if (fill_axes(a, table_sizes, nd, total) != S3D_OK) return 0;
-    return attn_mfma_supported(a, dtype) && attn_mfma_preferred(a) ? 1 : 0;
+    if (H < 1 || N < 0 || W < 0) return 0;
+    return s3d::attn_sweep_workspace_bytes(H, W, N);
 }
 
 namespace s3d {
@@ -125,9 +85,8 @@ int prepare_attn_args(const char *who, AttnArgs &a, bool *empty, const void *q, 
         if (table_len % hd != 0 || table_len / hd < nd)
             return fail(S3D_ERR_BAD_SHAPE, "%s: table_len = %lld is not a multiple of H*D = %lld with a row per axis", who,
                         (long long)table_len, (long long)hd);
-        for (int n = 0; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = a.pbase[n] = 0;
+        for (int n = 0; n < kMaxAxes; ++n) a.rows[n] = a.base[n] = 0;
         a.total_rows = static_cast<int32_t>(table_len / hd);
-        a.padded_rows = 0;
         a.sizes_dev = table_sizes;
     } else if (int rc = fill_axes(a, table_sizes, nd, table_len)) {
         return rc;
@@ -186,13 +145,14 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
     const void *q, const void *k, const void *v, const void *table_q, const void *table_k,
     const void *table_v, const int32_t *table_sizes, int32_t nd, int64_t table_len,
     const int32_t *w_sizes, const int32_t *w2n, const int32_t *n2n, const float *n_coords, void *out,
-    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W,
-    int32_t max_window_voxels, int64_t qkv_row_stride, int32_t dtype, int32_t flags, void *workspace,
-    size_t workspace_bytes, void *stream)
+    float *out_max, float *out_sum, int64_t N, int32_t H, int32_t D, int64_t W, int64_t qkv_row_stride,
+    int32_t dtype, int32_t flags, void *workspace, size_t workspace_bytes, void *stream)
 {
     using namespace s3d;
     AttnArgs a{};
     bool empty = true;
+    if (flags & ~(S3D_ATTN_PLANNED | S3D_ATTN_SIZES_ON_DEVICE))
+        return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: unknown flag bits in %d", flags);
     const bool sizes_on_device = (flags & S3D_ATTN_SIZES_ON_DEVICE) != 0;
     if (int rc = prepare_attn_args("s3d_attn_fwd", a, &empty, q, k, v, table_q, table_k, table_v, table_sizes, nd,
                                    table_len, w_sizes, w2n, n2n, n_coords, out, out_max, out_sum, N, H, D, W,
@@ -200,33 +160,19 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd(
         return rc;
     if (empty) return S3D_OK;
     a.workspace = workspace;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    // the MFMA kernel needs the window bound (it sizes partial results with it) and the row map
-    const bool want_mfma = !(flags & (S3D_ATTN_FORCE_GENERIC | S3D_ATTN_PLANNED | S3D_ATTN_SIZES_ON_DEVICE)) &&
-                           max_window_voxels >= 1 && n2n &&
-                           attn_mfma_supported(a, dtype) && (attn_mfma_preferred(a) || (flags & S3D_ATTN_FORCE_MFMA));
-    if (want_mfma) {
-        const size_t need = attn_mfma_workspace_bytes(H, D, a.padded_rows, W, N, max_window_voxels);
-        if (!workspace || workspace_bytes < need)
-            return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
-                        workspace ? workspace_bytes : size_t(0), need);
-        a.items = static_cast<char *>(workspace) + attn_mfma_table_bytes(H, D, a.padded_rows);
-        a.partials = reinterpret_cast<float *>(static_cast<char *>(a.items) + attn_mfma_items_bytes(W));
-        a.max_key_tiles = attn_mfma_key_tiles(max_window_voxels);
-        return launch_attn_mfma(a, s);
-    }
-    const size_t need = attn_generic_workspace_bytes(H, W, N);
+    const size_t need = attn_sweep_workspace_bytes(H, W, N);
     if (!workspace || workspace_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
     // with a plan the work list is in the workspace already
-    return launch_attn_generic(a, dtype, s, (flags & S3D_ATTN_PLANNED) ? kAttnSweep : (kAttnBuildList | kAttnSweep));
+    return launch_attn_sweep(a, dtype, static_cast<hipStream_t>(stream),
+                             (flags & S3D_ATTN_PLANNED) ? kAttnSweep : (kAttnBuildList | kAttnSweep));
 }
 
 extern "C" __attribute__((visibility("default"))) size_t s3d_attn_plan_bytes(int32_t H, int64_t N, int64_t W)
 {
     if (H < 1 || N < 0 || W < 0) return 0;
-    return s3d::attn_generic_workspace_bytes(H, W, N);
+    return s3d::attn_sweep_workspace_bytes(H, W, N);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_plan(
@@ -253,13 +199,13 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_plan(
     }
     if (N == 0 || W == 0) return S3D_OK;
     if (!w_sizes || !w2n) return fail(S3D_ERR_NULL_POINTER, "s3d_attn_plan: null device pointer");
-    const size_t need = attn_generic_workspace_bytes(H, W, N);
+    const size_t need = attn_sweep_workspace_bytes(H, W, N);
     if (!plan || plan_bytes < need)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_plan: plan buffer %zu B < required %zu B", plan ? plan_bytes : size_t(0), need);
     a.w_sizes = w_sizes;
     a.w2n = w2n;
     a.workspace = plan;
-    return launch_attn_generic(a, dtype, static_cast<hipStream_t>(stream), kAttnBuildList);
+    return launch_attn_sweep(a, dtype, static_cast<hipStream_t>(stream), kAttnBuildList);
 }
 
 extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_noalloc(
@@ -277,7 +223,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_noalloc(
                                    qkv_row_stride, dtype))
         return rc;
     if (empty) return S3D_OK;
-    const size_t need = attn_generic_workspace_bytes(H, W, N);
+    const size_t need = attn_sweep_workspace_bytes(H, W, N);
     if (need > kScratchBytes)
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_fwd_noalloc: N = %lld voxels in W = %lld windows need %zu B of work "
                     "list, the built-in scratch holds %zu B; use s3d_attn_fwd with a workspace",
@@ -287,5 +233,5 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_fwd_noalloc(
     a.workspace = address;
     // the list kernels write every word of the work list that the sweep kernel reads (the queue counters
     // included), so nothing of an earlier call's contents is used
-    return launch_attn_generic(a, dtype, static_cast<hipStream_t>(stream));
+    return launch_attn_sweep(a, dtype, static_cast<hipStream_t>(stream));
 }

@@ -21,6 +21,9 @@
 #include "attn_kernels.h"
 #include "sweep_common.h"
 
+#include <mutex>
+#include <vector>
+
 namespace s3d {
 namespace {
 
@@ -127,13 +130,13 @@ __host__ __device__ inline UnitPlan plan_units(int total_slots, int waves)
 // lane of a unit runs (almost) the same number of steps, a query's keys never leave its wavefront (the lanes
 // that share a query merge their softmax states by shuffles), and the launch ends on its shortest units.
 //
-// generic_count_kernel: every wavefront takes a run of consecutive windows, 64 at a time.  A window's place in the
+// sweep_count_kernel: every wavefront takes a run of consecutive windows, 64 at a time.  A window's place in the
 // bin of its (class, steps) - its rank there and the queries before it - follows the window numbers: the lanes
 // of each bin present among the 64 are ranked by their lane numbers on top of the bin's running totals, which
 // the wavefront keeps in registers (lane b % 64 holds bin b), and the wavefront leaves its bin totals.  No
 // atomics: the list, and with it the cut of the queries into units and so every bit of the result, is the same
 // on every run.
-__global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
+__global__ __launch_bounds__(kListThreads) void sweep_count_kernel(AttnArgs a)
 {
     constexpr int kWaves = kListThreads / 64;
     const int lane = threadIdx.x & 63;
@@ -204,11 +207,11 @@ __global__ __launch_bounds__(kListThreads) void generic_count_kernel(AttnArgs a)
     sum_bins[static_cast<size_t>(blockIdx.x) * kBins + threadIdx.x] = sum;
 }
 
-// generic_place_kernel (same grid): bins in order, wavefronts in order inside a bin.  Writes one entry (first
+// sweep_place_kernel (same grid): bins in order, wavefronts in order inside a bin.  Writes one entry (first
 // query of its class, voxels, first sorted position, class) per window in sorted order, one record per unit
 // (the entry that holds its first query, lanes per query as a shift, first query, queries), the totals, and
 // the queue counters at zero.
-__global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
+__global__ __launch_bounds__(kListThreads) void sweep_place_kernel(AttnArgs a)
 {
     constexpr int kWaves = kListThreads / 64;
     __shared__ int bin_entry[kWaves][kBins], bin_slot[kWaves][kBins];
@@ -311,6 +314,30 @@ __global__ __launch_bounds__(kListThreads) void generic_place_kernel(AttnArgs a)
         if (threadIdx.x < kQueues) total[(1 + threadIdx.x) * kCounterStride] = 0;
         for (int t = threadIdx.x; t < a.H * kQueues; t += kListThreads) counters[t * kCounterStride] = 0;
     }
+}
+
+// Raises a kernel's dynamic-LDS limit to `bytes`.  The runtime keeps the limit per function and device, so it is
+// set when a (function, device) pair first needs that much and not again: a call under stream capture then issues
+// kernel launches only (one eager call per shape and device has to come before the capture).
+inline int allow_dynamic_lds(const void *kernel, size_t bytes)
+{
+    struct Granted { const void *kernel; int device; size_t bytes; };
+    static std::mutex mutex;
+    static std::vector<Granted> granted;
+    int device = 0;
+    S3D_HIP_CHECK(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(mutex);
+    for (Granted &g : granted) {
+        if (g.kernel == kernel && g.device == device) {
+            if (g.bytes >= bytes) return S3D_OK;
+            S3D_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+            g.bytes = bytes;
+            return S3D_OK;
+        }
+    }
+    S3D_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    granted.push_back({kernel, device, bytes});
+    return S3D_OK;
 }
 
 inline int device_cus()
@@ -997,8 +1024,7 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
         return fail(S3D_ERR_UNSUPPORTED, "s3d_attn_fwd: %d table rows x D=%d need %zu B of LDS (> 160 KiB)",
                     a.total_rows, D, lds);
     auto kernel = attn_fwd_sweep_kernel<T, D, ND, HP, kSorted>;
-    S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return rc;
     // A workgroup serves one head group for its whole life: as many workgroups per CU as registers and LDS allow.
     // They come in whole sets of (XCDs x head groups) - runs of eight consecutive workgroups, one per XCD, serve one
     // head group, so every XCD serves every head group and the rows of a unit reach one L2 - unless whole sets
@@ -1020,8 +1046,8 @@ int launch_sweep_heads(const AttnArgs &a, hipStream_t stream, int what)
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
     const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
     if (what & 1) {
-        hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
-        hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+        hipLaunchKernelGGL(sweep_count_kernel, list_grid, dim3(kListThreads), 0, stream, b);
+        hipLaunchKernelGGL(sweep_place_kernel, list_grid, dim3(kListThreads), 0, stream, b);
         S3D_HIP_CHECK(hipGetLastError());
     }
     if (what & 2) {
@@ -1089,8 +1115,7 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
     constexpr int kThreads = bwd_pair_threads<T, D, HP>();
     int per_cu = 1;
     for (auto kernel : {q_sweep, k_sweep}) {
-        S3D_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), lds)) return rc;
     }
     {
         // workgroups per CU: what the registers of the heavier sweep and the tables in LDS allow
@@ -1112,8 +1137,8 @@ int launch_bwd_pairs_heads(const BwdPairArgs &b0, hipStream_t stream)
     b.f.block_shift = target_shift_for(a.N, a.W, b.f.target_items);
     const int64_t list_want = (a.W + kListThreads - 1) / kListThreads;
     const dim3 list_grid(static_cast<unsigned>(list_want < 1 ? 1 : (list_want > kListGroups ? kListGroups : list_want)));
-    hipLaunchKernelGGL(generic_count_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
-    hipLaunchKernelGGL(generic_place_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
+    hipLaunchKernelGGL(sweep_count_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
+    hipLaunchKernelGGL(sweep_place_kernel, list_grid, dim3(kListThreads), 0, stream, b.f);
     S3D_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(q_sweep, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, stream, b);
     hipLaunchKernelGGL(k_sweep, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, stream, b);
@@ -1162,13 +1187,13 @@ int launch_attn_bwd_pairs(const BwdPairArgs &b, int dtype, hipStream_t stream)
     }
 }
 
-size_t attn_generic_workspace_bytes(int H, int64_t W, int64_t N)
+size_t attn_sweep_workspace_bytes(int H, int64_t W, int64_t N)
 {
     // queue counters, the totals, one record per unit, the sorted window list and the list builder's notes
     return ws_end_offset(H, W, N);
 }
 
-int launch_attn_generic(const AttnArgs &a, int dtype, hipStream_t stream, int what)
+int launch_attn_sweep(const AttnArgs &a, int dtype, hipStream_t stream, int what)
 {
     switch (dtype) {
     case S3D_DTYPE_F32: return dispatch_shape<float>(a, stream, what);

@@ -248,11 +248,14 @@ __device__ __forceinline__ bool window_of(const int4 c, int stride, int window, 
     return !bad;
 }
 
-// partial bounding boxes of the window coordinates (one per workgroup, no atomics) and the cell counters at zero
+// partial bounding boxes of the window coordinates (one per workgroup, no atomics), the cell counters and the
+// call's totals and status word at zero (the later launches only ever OR bits into the status word)
 __global__ __launch_bounds__(kThreads) void grid_bbox_kernel(const int32_t *__restrict__ coords, int64_t N, int stride,
                                                              int window, int shift, int32_t *__restrict__ partials,
-                                                             int32_t *__restrict__ cells, int64_t num_cells)
+                                                             int32_t *__restrict__ cells, int64_t num_cells,
+                                                             int64_t *__restrict__ counts)
 {
+    if (blockIdx.x == 0 && threadIdx.x < 4) counts[threadIdx.x] = 0;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x; i < num_cells;
          i += static_cast<int64_t>(gridDim.x) * kThreads)
         cells[i] = 0;
@@ -289,8 +292,11 @@ __global__ __launch_bounds__(kThreads) void grid_bbox_kernel(const int32_t *__re
     }
 }
 
-// Every workgroup reduces the partial boxes to the lattice (workgroup 0 records it, the status word and zeroed
-// totals); then every voxel draws a slot in its cell - neighbouring lanes of one cell with one atomic.
+// Every workgroup reduces the partial boxes to the lattice (workgroup 0 records it and its bits of the status word);
+// then every voxel draws a slot in its cell - neighbouring lanes of one cell with one atomic.  A cell that runs
+// out of slot numbers (more than 2^kSlotBits voxels in one window: only with masses of equal coordinates) sets the
+// "no grid" bit as well: the status word was zeroed by the launch before this one and every writer ORs into it, so
+// no bit is lost whichever workgroup comes first, and the later launches of the call write nothing once it is set.
 __global__ __launch_bounds__(kThreads) void grid_count_kernel(
     const int32_t *__restrict__ coords, int64_t N, int stride, int window, int shift,
     const int32_t *__restrict__ partials, int64_t cells_cap, GridPlan *__restrict__ plan_out,
@@ -331,8 +337,8 @@ __global__ __launch_bounds__(kThreads) void grid_count_kernel(
             plan.ok = !bad && total <= static_cast<double>(cells_cap);
             if (blockIdx.x == 0) {
                 *plan_out = plan;
-                counts[0] = counts[1] = counts[2] = 0;
-                counts[3] = (bad ? kBadRange : 0) | (plan.ok ? 0 : kNoGrid);
+                const unsigned long long bits = (bad ? kBadRange : 0) | (plan.ok ? 0 : kNoGrid);
+                if (bits) atomicOr(reinterpret_cast<unsigned long long *>(counts + 3), bits);
             }
         }
         __syncthreads();
@@ -371,7 +377,7 @@ __global__ __launch_bounds__(kThreads) void grid_place_kernel(const int2 *__rest
                                                               uint64_t *__restrict__ keys, int32_t *__restrict__ w2n,
                                                               int32_t *__restrict__ w_sizes, int64_t *__restrict__ counts)
 {
-    if (!plan->ok) return;
+    if (!plan->ok || (counts[3] & kNoGrid)) return;
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (i == 0) counts[0] = static_cast<int64_t>(scan[cells_cap] >> 32);   // non-empty cells before the end = windows
     if (i >= N) return;
@@ -396,7 +402,7 @@ __global__ __launch_bounds__(kThreads) void grid_order_kernel(const GridPlan *__
                                                               int32_t *__restrict__ n2n, int32_t *__restrict__ w_w_id,
                                                               int64_t *__restrict__ counts)
 {
-    if (!plan->ok) return;
+    if (!plan->ok || (counts[3] & kNoGrid)) return;
     constexpr int kOrderStage = 512;                       // keys of a window staged in LDS at a time, per wavefront
     constexpr int kTotalGroups = 32;
     __shared__ uint64_t stage_all[kThreads / 64][kOrderStage];
@@ -715,7 +721,7 @@ extern "C" __attribute__((visibility("default"))) int s3d_window_index_grid(
     const int64_t num_cells = L.cells_cap + 1;
     const dim3 grid(static_cast<unsigned>(ceil_div(N, kThreads)));
     hipLaunchKernelGGL(grid_bbox_kernel, dim3(kGridBoxes), dim3(kThreads), 0, s, coords, N, stride, window, shift, partials,
-                       cells, num_cells);
+                       cells, num_cells, counts);
     S3D_HIP_CHECK(hipGetLastError());
     hipLaunchKernelGGL(grid_count_kernel, grid, dim3(kThreads), 0, s, coords, N, stride, window, shift, partials,
                        L.cells_cap, plan, cells, place, counts);

@@ -231,15 +231,40 @@ class StemConv(nn.Module):
         return voxels.with_feats(F.relu(self.conv_layers[1](out.float())))
 
 
+# Inference-time copies of parameters (autocast-dtype weights, scaled projections, flat tables) are kept on their
+# layers and checked against the parameters' addresses and version counters.  An update through `param.data` (EMA
+# helpers, some optimizer and init code) changes values without touching the version counter, so every copy also
+# carries the number of forward passes with autograd enabled that the process had seen when it was made: any
+# training forward in between renews it.  What this does not catch is a `.data` update with no grad-enabled forward
+# between two inference passes; call `drop_inference_copies(model)` after such an update.
+_GRAD_FORWARDS = [0]
+
+
+def _cache_epoch():
+    if torch.is_grad_enabled():
+        _GRAD_FORWARDS[0] += 1
+    return _GRAD_FORWARDS[0]
+
+
+def drop_inference_copies(model):
+    """Forget the inference-time copies of parameters that the layers of `model` keep (see above)."""
+    for m in model.modules():
+        if hasattr(m, "_s3d_cast"):
+            del m._s3d_cast
+        if isinstance(m, WindowAttention):
+            m._cache = None
+
+
 def _linear(layer, x):
     """layer(x) for an nn.Linear.  Inference under autocast keeps the parameters' copies in the autocast dtype on
     the layer (per parameter version) instead of casting them in every forward: autocast's own cache lives only as
     long as its context, and the encoder has about seventy such layers."""
+    epoch = _cache_epoch()
     if torch.is_grad_enabled() or not torch.is_autocast_enabled() or not x.is_cuda:
         return layer(x)
     dtype = torch.get_autocast_dtype("cuda")
     w, b = layer.weight, layer.bias
-    key = (dtype, w.data_ptr(), w._version, None if b is None else (b.data_ptr(), b._version))
+    key = (epoch, dtype, w.data_ptr(), w._version, None if b is None else (b.data_ptr(), b._version))
     kept = getattr(layer, "_s3d_cast", None)
     if kept is None or kept[0] != key:
         kept = (key, w.detach().to(dtype), None if b is None else b.detach().to(dtype))
@@ -346,7 +371,7 @@ class WindowAttention(nn.Module):
         names = ("xyz", "rgb", "norm")[: crse_num_axes(self.cRSE) // 3]
         params = [self.qkv.weight, self.qkv.bias] + [getattr(self, f"{k}_{n}_table") for k in ("query", "key", "value")
                                                      for n in names]
-        key = (dtype,) + tuple((p.data_ptr(), p._version) for p in params if p is not None)
+        key = (_cache_epoch(), dtype) + tuple((p.data_ptr(), p._version) for p in params if p is not None)
         if caching and self._cache is not None and self._cache[0] == key:
             return self._cache[1]
         # q scale folded into the projection (a C x C multiply instead of an N x C one)
@@ -419,10 +444,15 @@ class Stage(nn.Module):
             [SwinBlock(dim, num_heads, window_size, quant_size, cRSE=cRSE, fp16_mode=fp16_mode) for _ in range(depth)])
         self.downsample = GridKNNDownsample(dim, out_channels or dim * 2, stride=down_stride) if downsample else None
 
-    def plan(self, coords, stride, signals, num_batches=None):
+    def plan(self, coords, stride, signals, num_batches=None, rows_in_window_order=False):
         """Everything of the stage that depends on coordinates and signals only: the two window index sets
         (regular and shifted windows) with their scaled signals, and the downsample's geometry.  This is where
-        the host waits for the device (window counts, unique cells); `forward` with a plan does not."""
+        the host waits for the device (window counts, unique cells); `forward` with a plan does not.
+
+        rows_in_window_order: the caller has put the rows into the order of this stage's regular windows (the
+        window sort's n2n applied to coordinates, signals and features alike).  The row map of the regular set is
+        then the identity and is handed to the attention op as None: its kernels read and write the rows in place,
+        without the indirection."""
         local = (signals[:, 1:4].float() - coords[:, 1:].float()) / stride
         extra = signals[:, 4:].float()
         # both window sets (one, for a single block) are enqueued before the host waits for their window counts
@@ -433,6 +463,8 @@ class Stage(nn.Module):
         indices = build_window_indices(coords, stride, self.window_size, shifts)
         cell_index = indices.pop() if pooled else None
         args = [index_arguments(index, local, extra) for index in indices]
+        if rows_in_window_order and args:
+            args[0] = args[0][:5] + (None,) + args[0][6:]      # (.., w2n, n2n, w2m, ..): no row map
         if len(self.blocks) > 0:
             # the quantiser scaling of the signals is the same for every block of the stage: once per index set,
             # fused with the gather into window order
@@ -496,15 +528,18 @@ def geometry_steps(stem_coords, stride, signals, layers, window_ordered=False):
     is then the identity and that of the shifted blocks a near-local permutation, so the attention kernels read
     the rows of a window from neighbouring memory instead of through a scattered gather."""
     coords = stem_coords
+    ordered = False      # the current level's rows are in the order of its regular windows
     if window_ordered:
         order = window_order(coords, stride, layers[0].window_size) if len(layers) else None
         if order is not None:
             coords, signals = coords[order], signals[order]
+            ordered = True
         yield order, coords, signals
     yield conv3x3x3_neighbours(coords, stride)
     num_batches = int(coords[-1, 0]) + 1 if coords.shape[0] else 0    # batch ids are ascending: one read
     for level, layer in enumerate(layers):
-        plan = layer.plan(coords, stride, signals, num_batches)
+        plan = layer.plan(coords, stride, signals, num_batches, rows_in_window_order=ordered)
+        ordered = False
         if plan[1] is not None:
             coarse, coarse_signals, idx = plan[1]
             coarse_stride = stride * layer.downsample.factor
@@ -513,6 +548,7 @@ def geometry_steps(stem_coords, stride, signals, layers, window_ordered=False):
                 if order is not None:
                     coarse, coarse_signals, idx = coarse[order], coarse_signals[order], idx[order]
                     plan = (plan[0], (coarse, coarse_signals, idx))
+                    ordered = True
         yield plan
         if plan[1] is not None:
             coords, signals = plan[1][0], plan[1][1]

@@ -53,9 +53,6 @@ BWD_PAIR_STORE_MAX_BYTES = 32 << 30
 BWD_MAX_ROWS_PER_AXIS = 64
 BWD_HEAD_DIMS = (8, 16, 32)
 
-# debugging / ablation switch: run the generic VALU kernel even where the MFMA kernel applies
-FORCE_GENERIC = False
-
 
 def _require_cuda(name, t, device=None, strided_rows=False):
     if not isinstance(t, torch.Tensor):
@@ -86,7 +83,10 @@ def _row_stride(t):
 
 
 def _as_int32(name, t, device):
-    """Index tensors arrive as int64 from torch ops; the kernels read int32."""
+    """Index tensors arrive as int64 from torch ops (the reference's caller builds every one of them with
+    torch.long, Swin3D/modules/swin3d_layers.py:96-140); the kernels read int32.  The int32 copy of an int64 CUDA
+    tensor is kept on the tensor object, with its version counter and address, so a caller that hands the same
+    index tensors to block after block pays the cast kernels once per window set and not once per call."""
     if not isinstance(t, torch.Tensor):
         t = torch.as_tensor(t)
     if t.dtype not in (torch.int32, torch.int64):
@@ -95,11 +95,21 @@ def _as_int32(name, t, device):
         if t.is_cuda:
             raise RuntimeError(f"{name} is on {t.device}, expected {device}")
         t = t.to(device)
-    return t.to(torch.int32).contiguous()
+    if t.dtype == torch.int32:
+        return t.contiguous()
+    stamp = (t._version, t.data_ptr(), tuple(t.shape), tuple(t.stride()))
+    kept = getattr(t, "_s3d_int32", None)
+    if kept is None or kept[0] != stamp:
+        kept = (stamp, t.to(torch.int32).contiguous())
+        try:
+            t._s3d_int32 = kept
+        except (AttributeError, RuntimeError):     # an object that takes no attributes: cast on every call
+            pass
+    return kept[1]
 
 
 def _host_table_sizes(table_sizes):
-    """The per-axis table sizes as a host list (the backward and the MFMA kernel need them there).  A CUDA
+    """The per-axis table sizes as a host list (the backward needs them there).  A CUDA
     tensor costs one synchronising device-to-host copy; the values are then kept on the tensor object (with
     its version counter), so a module that keeps its table_offsets tensor pays the copy once."""
     if isinstance(table_sizes, torch.Tensor):
@@ -117,7 +127,7 @@ def _host_table_sizes(table_sizes):
 REUSE_PLANS = True
 
 # a CUDA table_sizes tensor whose values the host has not seen yet goes to the sweep kernel as it is, and the
-# host never waits for it (False: always copy it to the host, which also lets the MFMA kernel be chosen)
+# host never waits for it (False: always copy it to the host, which checks the values there)
 DEVICE_TABLE_SIZES = True
 
 
@@ -158,29 +168,20 @@ def _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes, nd, table_l
 
 
 def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_sizes, w2n, n2n,
-                             n_coords, return_stats=False, force_generic=False, max_window_voxels=None,
-                             force_mfma=False):
+                             n_coords, return_stats=False):
     """softmax-normalised window attention, [N,H,D] in the dtype of q.
 
     q, k, v        [N,H,D] fp16 or fp32 CUDA tensors (q already scaled by D**-0.5); dense, or views with
                    a dense (H,D) block and one common row stride (slices of a [N,3*H*D] projection output)
     table_*        flat [sum(table_sizes)] tensors, layout [axis][row][h][c], dtype of q
     table_sizes    int tensor / list [nd], per-axis element counts rows*H*D.  A list or CPU tensor is read on
-                   the host; a CUDA tensor stays on the device and the sweep kernel reads it (no host wait, no
-                   check of the values beyond clipping them to the table; the MFMA kernel is then not chosen)
-                   unless force_mfma or DEVICE_TABLE_SIZES = False ask for the host copy
-    w_sizes, w2n   [W] voxels per window and their exclusive prefix sum
+                   the host; a CUDA tensor stays on the device and the kernel reads it (no host wait, no
+                   check of the values beyond clipping them to the table) unless DEVICE_TABLE_SIZES = False
+    w_sizes, w2n   [W] voxels per window and their exclusive prefix sum (int32, or int64 as torch ops give them)
     n2n            [N] window-sorted position -> row of q/k/v, or None when the rows are in window-sorted
-                   order already (the sweep kernel then reads and writes them without the indirection)
+                   order already (the kernel then reads and writes them without the indirection)
     n_coords       [N,nd] fp32 signals in window-sorted order (already quant-scaled)
     return_stats   also return (max logit [N,H] fp32, sum exp(logit - max) [N,H] fp32)
-    force_generic  run the VALU sweep kernel for every case
-    force_mfma     run the MFMA kernel wherever it applies (fp16, head_dim 8 or 16, axis tables of at most 64
-                   rows); by default it serves head_dim 16 with full windows only
-    max_window_voxels  upper bound of w_sizes; taken from the tensor's `max_window_voxels` attribute
-                   (set by build_window_index) when not given.  Without a bound the sweep kernel serves the
-                   call (it takes windows of any size); the host waits for the device to find one only under
-                   force_mfma
     """
     _require_cuda("query", q, strided_rows=True)
     dev = q.device
@@ -200,7 +201,7 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     row_stride = _row_stride(q)
     if d not in (8, 16, 32):
         raise ValueError(f"head_dim must be 8, 16 or 32, got {d}")
-    if not force_mfma and _sizes_stay_on_device(table_sizes):
+    if _sizes_stay_on_device(table_sizes):
         sizes = None
         sizes_dev = _as_int32("table_sizes", table_sizes.reshape(-1), dev)
         nd = sizes_dev.numel()
@@ -231,8 +232,6 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
         n2n = _as_int32("n2n_indices", n2n, dev)
         if n2n.shape != (n,):
             raise ValueError(f"n2n_indices must be [{n}], got {tuple(n2n.shape)}")
-    elif force_mfma:
-        raise ValueError("the MFMA kernel needs n2n_indices")
     if w_sizes.shape != w2n.shape or w_sizes.dim() != 1:
         raise ValueError("w_sizes and w2n_indices must be 1-D of equal length")
     _require_cuda("n_coords", n_coords, dev)
@@ -242,41 +241,27 @@ def window_attention_forward(q, k, v, table_q, table_k, table_v, table_sizes, w_
     out = torch.empty((n, h, d), dtype=q.dtype, device=dev)
     omax = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
     osum = torch.empty((n, h), dtype=torch.float32, device=dev) if return_stats else None
-    if max_window_voxels is None:
-        max_window_voxels = getattr(w_sizes_in, "max_window_voxels", None)
-    max_window_voxels = max(int(max_window_voxels), 0) if max_window_voxels is not None else 0
-    if force_mfma and max_window_voxels < 1:
-        # the MFMA kernel needs the bound: forcing it without one costs a device read-back
-        max_window_voxels = int(w_sizes.max().item()) if w_sizes.numel() else 1
     lib = _lib.lib()
     code = _DTYPE_CODE[q.dtype]
     num_w = w_sizes.numel()
-    flags = ((_lib.S3D_ATTN_FORCE_GENERIC if (force_generic or FORCE_GENERIC) else 0) |
-             (_lib.S3D_ATTN_FORCE_MFMA if force_mfma else 0) |
-             (_lib.S3D_ATTN_SIZES_ON_DEVICE if sizes is None else 0))
+    flags = _lib.S3D_ATTN_SIZES_ON_DEVICE if sizes is None else 0
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        # the sweep kernel's work list depends on the window set only: it is built once and kept on the
-        # caller's w_sizes tensor, so the blocks that share a window set share it
-        mfma = (sizes is not None and not flags & _lib.S3D_ATTN_FORCE_GENERIC and n2n is not None and
-                max_window_voxels >= 1 and
-                (force_mfma or lib.s3d_attn_fwd_uses_mfma(c_sizes, nd, h, d, code, n, num_w)))
-        plan = None if mfma or not REUSE_PLANS else _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes,
-                                                              nd, table_len, n, h, d, code, stream)
+        # the work list depends on the window set only: it is built once and kept on the caller's w_sizes
+        # tensor, so the blocks that share a window set share it
+        plan = None if not REUSE_PLANS else _plan_for(lib, w_sizes_in, w2n_in, w_sizes, w2n, c_sizes, sizes,
+                                                      nd, table_len, n, h, d, code, stream)
         if plan is not None:
             workspace, ws_bytes, flags = plan, plan.numel(), flags | _lib.S3D_ATTN_PLANNED
-        elif sizes is None:
-            ws_bytes = lib.s3d_attn_plan_bytes(h, n, num_w)   # the sweep kernel's work list
-            workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         else:
-            ws_bytes = lib.s3d_attn_fwd_workspace_bytes(c_sizes, nd, h, d, n, num_w, max_window_voxels)
+            ws_bytes = lib.s3d_attn_fwd_workspace_bytes(h, n, num_w)
             workspace = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
         status = lib.s3d_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), table_q.data_ptr(), table_k.data_ptr(),
             table_v.data_ptr(), c_sizes, nd, table_len, w_sizes.data_ptr(),
             w2n.data_ptr(), n2n.data_ptr() if n2n is not None else None, n_coords.data_ptr(), out.data_ptr(),
             omax.data_ptr() if return_stats else None, osum.data_ptr() if return_stats else None,
-            n, h, d, num_w, max_window_voxels, row_stride, code, flags, workspace.data_ptr(), ws_bytes, stream)
+            n, h, d, num_w, row_stride, code, flags, workspace.data_ptr(), ws_bytes, stream)
     _lib.check(status, "s3d_attn_fwd")
     if return_stats:
         return out, omax, osum
@@ -345,7 +330,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
             raise ValueError(f"{name} must be float32 [{n},{h}]")
     w_sizes = _as_int32("w_sizes", w_sizes, dev)
     w2n = _as_int32("w2n_indices", w2n, dev)
-    n2n = _as_int32("n2n_indices", n2n, dev)
+    # rows in window-sorted order already (the forward took no row map): the backward's kernels read one
+    n2n = torch.arange(n, dtype=torch.int32, device=dev) if n2n is None else _as_int32("n2n_indices", n2n, dev)
     _require_cuda("n_coords", n_coords, dev)
     if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
         raise ValueError(f"n_coords must be float32 [{n},{nd}]")

@@ -87,7 +87,6 @@ def build_window_indices(coords, stride, window_size, shifts):
             raise ValueError("coords outside the supported range (batch 0..4095, window coordinate "
                              "-8192..8191)")
         sizes = w_sizes[:num_w]
-        sizes.max_window_voxels = int(max_w)   # read by the attention op (the MFMA kernel sizes its partial results with it)
         sizes._s3d_pairs = (sizes._version, int(num_m))   # ... and by its backward (the size of the pair store)
         result.append(WindowIndex(n2n, wwid, sizes, w2n[:num_w], int(num_w), int(num_m), int(max_w), int(window)))
     return result

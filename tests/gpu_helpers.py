@@ -6,8 +6,7 @@ import torch
 import swin3d_amd
 
 
-def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", force_generic=False, force_mfma=False,
-                  device_sizes=False):
+def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", device_sizes=False):
     """-> numpy float64 output [N,H,D] of swin3d_amd.window_attention_forward.  device_sizes: the per-axis table
     sizes go in as a CUDA tensor (the sweep kernel reads them, the host never does) instead of a host list."""
     dev = torch.device(device)
@@ -17,8 +16,7 @@ def run_attention(case, dtype=torch.float32, return_stats=False, device="cuda", 
         t(case.q).to(dtype), t(case.k).to(dtype), t(case.v).to(dtype),
         t(case.tq).to(dtype), t(case.tk).to(dtype), t(case.tv).to(dtype),
         t(case.table_sizes) if device_sizes else [int(x) for x in case.table_sizes], t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
-        return_stats=return_stats, force_generic=force_generic, force_mfma=force_mfma,
-        max_window_voxels=int(i["w_sizes"].max()) if len(i["w_sizes"]) else 0)
+        return_stats=return_stats)
     torch.cuda.synchronize()
     if return_stats:
         return tuple(r.double().cpu().numpy() for r in res)

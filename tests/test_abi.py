@@ -15,7 +15,7 @@ def _declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     names = _declared_symbols()
-    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_knn_max_pool", "s3d_attn_fwd_uses_mfma", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_window_signals", "s3d_key_neighbours", "s3d_cell_representatives", "s3d_knn",
+    for must in ("s3d_add_layernorm", "s3d_attn_fwd", "s3d_attn_bwd", "s3d_attn_bwd_workspace_bytes", "s3d_knn_interpolate", "s3d_knn_max_pool", "s3d_attn_plan", "s3d_attn_fwd_noalloc", "s3d_attn_fwd_workspace_bytes", "s3d_window_index", "s3d_window_index_workspace_bytes", "s3d_window_signals", "s3d_key_neighbours", "s3d_cell_representatives", "s3d_knn",
                  "s3d_knn_workspace_bytes", "s3d_last_error_string", "s3d_version"):
         assert must in names
 
@@ -36,14 +36,14 @@ def test_python_constants_equal_the_header():
     text = open(os.path.join(ROOT, "include", "swin3d_amd.h")).read()
     defines = {name: int(value, 0) for name, value in re.findall(r"^#define (S3D_[A-Z0-9_]+) \(?(-?(?:0x)?[0-9a-fA-F]+)\)?\s*(?:/\*.*)?$",
                                                               text, flags=re.M)}
-    for name in ("S3D_DTYPE_F32", "S3D_DTYPE_F16", "S3D_DTYPE_F32_F16_ROWS", "S3D_ATTN_FORCE_GENERIC",
-                 "S3D_ATTN_FORCE_MFMA", "S3D_ATTN_PLANNED", "S3D_ATTN_SIZES_ON_DEVICE"):
+    for name in ("S3D_DTYPE_F32", "S3D_DTYPE_F16", "S3D_DTYPE_F32_F16_ROWS", "S3D_ATTN_PLANNED",
+                 "S3D_ATTN_SIZES_ON_DEVICE"):
         assert defines[name] == getattr(_lib, name), name
     assert defines["S3D_KNN_KMAX"] == _lib.KNN_KMAX
 
 
 def test_version_and_error_string(hip_lib):
-    assert hip_lib.s3d_version() >= 100
+    assert hip_lib.s3d_version() >= 200
     assert isinstance(hip_lib.s3d_last_error_string(), bytes)
 
 
@@ -53,7 +53,7 @@ def test_argument_errors_are_reported_without_a_device(hip_lib):
     status = hip_lib.s3d_knn(0, None, 0, None, 0, None, None, 1, None, None, 0.0, None, 0, None)
     assert status < 0
     assert b"K=0" in hip_lib.s3d_last_error_string()
-    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 125, 0, 1, 0, None, 0, None)
+    status = hip_lib.s3d_attn_fwd(*([None] * 7), 9, 0, *([None] * 7), 10, 6, 8, 1, 0, 1, 0, None, 0, None)
     assert status < 0 and b"table_len" in hip_lib.s3d_last_error_string()
     try:
         _lib.check(status, "s3d_attn_fwd")
@@ -71,8 +71,11 @@ def test_more_argument_errors_without_a_device(hip_lib):
     sizes = crse.crse_table_sizes(5, 4, 6, 8, "XYZ_RGB_NORM")
     c_sizes = (ctypes.c_int32 * 9)(*sizes)
     total = sum(sizes)
-    st = hip_lib.s3d_attn_fwd(*([None] * 6), c_sizes, 9, total, *([None] * 7), 10, 6, 8, 1, 125, 50, 1, 0, None, 0, None)
+    st = hip_lib.s3d_attn_fwd(*([None] * 6), c_sizes, 9, total, *([None] * 7), 10, 6, 8, 1, 50, 1, 0, None, 0, None)
     assert st < 0 and b"qkv_row_stride" in hip_lib.s3d_last_error_string()
+    # flag bits that name no behaviour of the call (1 and 2 selected a kernel in earlier versions of the library)
+    st = hip_lib.s3d_attn_fwd(*([None] * 6), c_sizes, 9, total, *([None] * 7), 10, 6, 8, 1, 0, 1, 2, None, 0, None)
+    assert st < 0 and b"flag" in hip_lib.s3d_last_error_string()
     # backward: workspace missing
     st = hip_lib.s3d_attn_bwd(*([None] * 6), c_sizes, 9, total, *([None] * 14), 10, 6, 8, 1, 0, 1, None, 0, None)
     assert st < 0 and (b"gradient pointer" in hip_lib.s3d_last_error_string()
@@ -104,21 +107,14 @@ def test_more_argument_errors_without_a_device(hip_lib):
     assert hip_lib.s3d_add_layernorm(None, None, 0, None, None, 1e-5, None, None, 1, 0, 64, None) == 0
 
 
-def test_kernel_choice_is_reported(hip_lib):
-    """fp16 Swin3D shapes with head_dim 16 (S and L, stages 2-5) go to the MFMA kernel when the windows hold
-    300 voxels or more on average; sparser scenes, head_dim 8 and fp32 go to the sweep kernel."""
-    import ctypes
-    from swin3d_amd import crse
-    for ws, heads, dim in [(5, 6, 8), (7, 6, 16), (7, 12, 16), (7, 24, 16), (5, 10, 8), (7, 40, 16)]:
-        sizes = crse.crse_table_sizes(ws, 4, heads, dim, "XYZ_RGB_NORM")
-        c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 300000, 1000) == (1 if dim == 16 else 0)
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 299999, 1000) == 0
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, 60000, 1000) == 0
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 0, 320000, 1000) == 0
-    sizes = crse.crse_table_sizes(10, 4, 6, 8, "XYZ")          # 80-row tables: generic kernel
-    c_sizes = (ctypes.c_int32 * 3)(*sizes)
-    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, 3, 6, 8, 1, 320000, 1000) == 0
+def test_work_list_size_depends_on_the_window_set_only(hip_lib):
+    """The forward's workspace is its work list: counters per head, a record per unit of at least 8 queries, 24
+    bytes per window and the list builder's notes; the plan buffer is the same thing."""
+    for heads, n, w in ((6, 199_327, 7_554), (40, 2_713, 40), (10, 595_677, 22_000), (1, 0, 0)):
+        need = hip_lib.s3d_attn_fwd_workspace_bytes(heads, n, w)
+        assert need == hip_lib.s3d_attn_plan_bytes(heads, n, w)
+        assert 2 * n + 24 * w <= need <= 2 * n + 24 * w + 2048 * heads + (1 << 19)
+    assert hip_lib.s3d_attn_fwd_workspace_bytes(0, 10, 1) == 0 and hip_lib.s3d_attn_fwd_workspace_bytes(6, -1, 1) == 0
 
 
 def test_window_signals_rejects_bad_arguments(hip_lib):

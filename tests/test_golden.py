@@ -37,8 +37,7 @@ def test_oracle_knn_matches_fixture(oracle_lib):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("half", [False, True])
-@pytest.mark.parametrize("kernel", ["default", "sweep", "mfma"])
-def test_hip_attention_matches_fixture(hip_lib, half, kernel):
+def test_hip_attention_matches_fixture(hip_lib, half):
     import torch
     import swin3d_amd
     from gpu_helpers import assert_attn_close
@@ -49,7 +48,7 @@ def test_hip_attention_matches_fixture(hip_lib, half, kernel):
     t = lambda a: torch.from_numpy(a).to(dev)
     out = swin3d_amd.window_attention_forward(
         f(g["q"]), f(g["k"]), f(g["v"]), f(g["tq"]), f(g["tk"]), f(g["tv"]), t(g["table_sizes"]),
-        t(g["w_sizes"]), t(g["w2n"]), t(g["n2n"]), t(g["n_coords"]), force_generic=kernel == "sweep", force_mfma=kernel == "mfma")
+        t(g["w_sizes"]), t(g["w2n"]), t(g["n2n"]), t(g["n_coords"]))
     torch.cuda.synchronize()
     assert_attn_close(out.double().cpu().numpy(), g["out"], dtype)
 

@@ -16,13 +16,8 @@ def _check(oracle_lib, case, dtype):
     ref = oracle_lib.attn_fwd(*case.oracle_args())
     got = run_attention(case, dtype)
     assert_attn_close(got, ref, dtype)
-    # per-axis table sizes read by the kernel from device memory: the bits of the sweep kernel with host sizes
-    assert np.array_equal(run_attention(case, dtype, device_sizes=True), run_attention(case, dtype, force_generic=True))
-    if dtype == torch.float16:
-        # fp16: the library picks the sweep or the MFMA kernel by head_dim; both must agree with the oracle
-        assert_attn_close(run_attention(case, dtype, force_generic=True), ref, dtype)
-        if case.D <= 16:
-            assert_attn_close(run_attention(case, dtype, force_mfma=True), ref, dtype)
+    # per-axis table sizes read by the kernel from device memory: the bits of the call with host sizes
+    assert np.array_equal(run_attention(case, dtype, device_sizes=True), got)
     return got, ref
 
 
@@ -90,8 +85,7 @@ def test_large_dense_windows_stay_inside_a_wavefront(oracle_lib, hip_lib, heads)
     """A 56x56x28 grid at 62 % fill, window 7: 256 windows of about 210 voxels.  The sweep kernel gives each query
     of such a window four adjacent lanes that take alternate keys and merge their softmax states by shuffles, so no
     partial result passes through memory: the workspace holds the work list only, whatever the window sizes
-    (quant 5 gives 70-row axis tables, which only the sweep kernel takes, so the size is that kernel's)."""
-    import ctypes
+    (quant 5: 70-row axis tables)."""
     ws, quant, dim = 7, 5, 16
     rng = np.random.default_rng(52)
     g = np.stack(np.meshgrid(np.arange(56), np.arange(56), np.arange(28), indexing="ij"), -1).reshape(-1, 3)
@@ -108,11 +102,7 @@ def test_large_dense_windows_stay_inside_a_wavefront(oracle_lib, hip_lib, heads)
         n, heads * dim, heads, int(sum(case.table_sizes)), seed=52, recipe="sharp")
     w_sizes = case.index["w_sizes"]
     assert w_sizes.shape[0] == 256 and 128 < int(w_sizes.max()) <= 256
-    sizes = [int(x) for x in case.table_sizes]
-    c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
-    assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, dim, 1, n, 256) == 0
-    ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), heads, dim, n, 256, int(w_sizes.max()))
-    assert ws_bytes == hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), heads, dim, n, 256, 0)   # no bound needed
+    ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(heads, n, 256)
     assert ws_bytes < 2 * n + 24 * 256 + (1 << 20)     # a unit record per 8 queries, 24 bytes per window, fixed part
     _sharp16(case)
     _check(oracle_lib, case, torch.float16)
@@ -120,8 +110,8 @@ def test_large_dense_windows_stay_inside_a_wavefront(oracle_lib, hip_lib, heads)
 
 def boundary_size_case(oracle_lib, heads, dim, seed=41):
     """One window per size in 1, 16, 31..33, 63..65, 127..129, 192, 193 voxels (window 7): the sizes around the
-    tile and block lengths at which the kernels split a window (key blocks of 64 in the sweep kernel, tiles of 32
-    queries and keys in the MFMA kernel; the backward changes its lane mapping at 32 voxels)."""
+    block lengths at which the kernels split a window (a lane of the sweep kernel streams 16, 32 or 64 keys, a query
+    of a larger window gets 2, 4 or 8 lanes; the backward changes its lane mapping at 32 voxels)."""
     ws, quant = 7, 4
     sizes = [1, 16, 31, 32, 33, 63, 64, 65, 127, 128, 129, 192, 193]
     rng = np.random.default_rng(seed)
@@ -214,44 +204,10 @@ def test_stats_outputs(oracle_lib, hip_lib):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("kernel", ["sweep", "mfma"])
-def test_understated_window_bound_is_visible(oracle_lib, hip_lib, kernel):
-    """max_window_voxels below the real maximum.  The sweep kernel does not use the bound: every row is complete.
-    The MFMA kernel sizes its partial results with it (rounded up to its key tile of 32 voxels): the rows of
-    windows beyond the bound, and their statistics, read NaN instead of what the buffer held; every other window
-    is complete and nothing is written out of bounds."""
-    import swin3d_amd
-    case = make_attn_case(oracle_lib, seed=38, n=1000, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
-    to_half_and_back(_sharp16(case))
-    w_sizes = case.index["w_sizes"]
-    assert w_sizes.max() > 32 and (w_sizes <= 32).any()
-    ref = oracle_lib.attn_fwd(*case.oracle_args())
-    dev = torch.device("cuda")
-    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-    h = lambda a: t(a).half()
-    i = case.index
-    got, gmax, gsum = swin3d_amd.window_attention_forward(
-        h(case.q), h(case.k), h(case.v), h(case.tq), h(case.tk), h(case.tv), t(case.table_sizes),
-        t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords), max_window_voxels=32, return_stats=True,
-        force_generic=kernel == "sweep", force_mfma=kernel == "mfma")
-    torch.cuda.synchronize()
-    got = got.double().cpu().numpy()
-    small = np.repeat(w_sizes <= 32, w_sizes)           # per sorted position
-    rows_small, rows_large = i["n2n"][small], i["n2n"][~small]
-    from gpu_helpers import assert_attn_close
-    assert_attn_close(got[rows_small], ref[rows_small], torch.float16)
-    if kernel == "sweep":
-        assert_attn_close(got[rows_large], ref[rows_large], torch.float16)
-    else:
-        assert np.isnan(got[rows_large]).all()
-        assert torch.isnan(gmax[t(rows_large).long()]).all() and torch.isnan(gsum[t(rows_large).long()]).all()
-        assert np.isfinite(got[rows_small]).all()
-
-
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 def test_strided_qkv_views_are_read_in_place(oracle_lib, hip_lib, dtype):
     """q, k, v as slices of one [N, 3*H*D] buffer (the layout of the qkv projection output): same result as
-    dense copies, on both kernels, and no copy is made (checked through the data pointers the op sees)."""
+    dense copies, and no copy is made (checked through the data pointers the op sees)."""
     import swin3d_amd
     from gpu_helpers import assert_attn_close
     case = make_attn_case(oracle_lib, seed=39, n=1200, ws=5, quant=4, heads=6, dim=8, extent=(10, 10, 3))
@@ -266,13 +222,16 @@ def test_strided_qkv_views_are_read_in_place(oracle_lib, hip_lib, dtype):
     assert not q.is_contiguous() and q.stride(0) == 3 * h * d
     i = case.index
     f = lambda a: t(a).to(dtype)
-    for force_generic, force_mfma in ((False, False), (True, False), (False, True)):
-        got = swin3d_amd.window_attention_forward(q, k, v, f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
-                                                  t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords),
-                                                  force_generic=force_generic, force_mfma=force_mfma)
-        torch.cuda.synchronize()
-        assert got.is_contiguous() and got.shape == (n, h, d)
-        assert_attn_close(got.double().cpu().numpy(), ref, dtype)
+    got = swin3d_amd.window_attention_forward(q, k, v, f(case.tq), f(case.tk), f(case.tv), t(case.table_sizes),
+                                              t(i["w_sizes"]), t(i["w2n"]), t(i["n2n"]), t(case.n_coords))
+    torch.cuda.synchronize()
+    assert got.is_contiguous() and got.shape == (n, h, d)
+    assert_attn_close(got.double().cpu().numpy(), ref, dtype)
+    # the bits of the call on dense copies: where a row lives does not enter the arithmetic
+    dense = swin3d_amd.window_attention_forward(q.contiguous(), k.contiguous(), v.contiguous(), f(case.tq), f(case.tk),
+                                                f(case.tv), t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]),
+                                                t(i["n2n"]), t(case.n_coords))
+    assert torch.equal(got, dense)
     # a row stride the kernels cannot read (not a multiple of 8 elements) is rejected, as non-contiguous
     # input is by the reference's CHECK_INPUT
     odd = torch.zeros((n, 3 * h * d + 3), dtype=dtype, device=dev)[:, : h * d].view(n, h, d)
@@ -300,7 +259,7 @@ def test_other_window_and_quant_sizes(oracle_lib, hip_lib, dtype, ws, quant, hea
 def test_random_shapes(oracle_lib, hip_lib, seed):
     """Randomly drawn shapes: odd and even head counts (one or two heads per wavefront in the sweep kernel), both
     head_dims, 3 / 6 / 9 axes, sparse to dense windows (all unit kinds, split and unsplit windows), several batch
-    elements, strides and window shifts; fp32 on even seeds, fp16 (both kernels) on odd ones."""
+    elements, strides and window shifts; fp32 on even seeds, fp16 on odd ones."""
     rng = np.random.default_rng(1000 + seed)
     ws = int(rng.choice([3, 5, 7]))
     heads = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 12]))
@@ -340,7 +299,7 @@ def test_table_sizes_on_the_device_need_no_host_read(oracle_lib, hip_lib, dtype)
     feats = [f(x) for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
     index = [t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)]
     host_sizes = [int(x) for x in case.table_sizes]
-    ref = swin3d_amd.window_attention_forward(*feats, host_sizes, *index, force_generic=True)
+    ref = swin3d_amd.window_attention_forward(*feats, host_sizes, *index)
     for sizes_dtype in (torch.int32, torch.int64):
         sizes = torch.tensor(host_sizes, dtype=sizes_dtype).cuda()
         got = swin3d_amd.window_attention_forward(*feats, sizes, *index)
@@ -369,8 +328,8 @@ def test_table_sizes_on_the_device_need_no_host_read(oracle_lib, hip_lib, dtype)
 @pytest.mark.parametrize("heads,ws,cRSE,shift", [(2, 5, "XYZ_RGB_NORM", 0), (3, 7, "XYZ_RGB", 3), (4, 3, "XYZ", 0)])
 def test_head_dim_32_forward(oracle_lib, hip_lib, dtype, heads, ws, cRSE, shift):
     """head_dim 32, the largest the reference takes (Swin3D/src/attn/self_attn_aio_fwd.cu:486): the sweep kernel
-    serves it (one head per wavefront, windows of all unit kinds); the MFMA kernel never takes it, and the backward
-    says where the op is called that it does not."""
+    serves it with one head per wavefront (windows of all unit kinds), and the backward runs in the library's
+    general form."""
     import swin3d_amd
     from swin3d_amd.sparse_dl.attn import attn_coff
     case = make_attn_case(oracle_lib, seed=90 + heads, n=2500, ws=ws, quant=4, heads=heads, dim=32, cRSE=cRSE,
@@ -385,9 +344,6 @@ def test_head_dim_32_forward(oracle_lib, hip_lib, dtype, heads, ws, cRSE, shift)
         feats = [t(x) for x in (case.q, case.k, case.v, case.tq, case.tk, case.tv)]
         index = [t(i["w_sizes"]).int(), t(i["w2n"]).int(), t(i["n2n"]).int(), t(case.n_coords)]
         sizes = [int(x) for x in case.table_sizes]
-        import ctypes
-        c_sizes = (ctypes.c_int32 * len(sizes))(*sizes)
-        assert hip_lib.s3d_attn_fwd_uses_mfma(c_sizes, len(sizes), heads, 32, 1, 343000, 1000) == 0
         # the backward of this head_dim is the library's general form (checked against the oracle in
         # test_gpu_attn_bwd.py::test_general_form): here only that autograd reaches it
         leaves = [x.clone().requires_grad_() for x in feats]
@@ -457,6 +413,48 @@ def test_autograd_function_surface(oracle_lib, hip_lib):
     assert out16.dtype == torch.float16 and out32.dtype == torch.float32
     ref16 = oracle_lib.attn_fwd(*to_half_and_back(case).oracle_args())
     assert_attn_close(out16.double().cpu().numpy(), ref16, torch.float16)
+
+
+def test_int64_index_tensors_are_cast_once(oracle_lib, hip_lib):
+    """The reference's caller hands int64 index tensors (torch.long everywhere in Swin3D/modules/swin3d_layers.py:
+    96-140) and reuses one `indices` list for the blocks of a window set; the kernels read int32.  The int32 copies
+    are made on the first call and kept on the caller's tensors: a second call launches no cast kernel (checked in
+    a profiler trace of the call), and an in-place change of a tensor renews its copy."""
+    import swin3d_amd as s3d
+    from torch.profiler import ProfilerActivity, profile
+    case = make_attn_case(oracle_lib, seed=87, n=900, ws=5, quant=4, heads=6, dim=8, extent=(8, 8, 3), recipe="layer")
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    idx = [None, t(case.index["w_sizes"]).long(), None, t(case.index["w2n"]).long(),
+           t(case.index["n2n"]).long(), t(case.n_coords)]
+    args = [t(case.q), t(case.k), t(case.v), t(case.tq), t(case.tk), t(case.tv), [int(x) for x in case.table_sizes], idx,
+            s3d.PosEmb.SEPARATE, s3d.TableDims.D0, s3d.IndexMode.INDIRECT, s3d.PrecisionMode.HALF_NONE]
+
+    def traced_call():
+        with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as prof:
+            out = s3d.SelfAttnAIOFunction.apply(*args)
+            torch.cuda.synchronize()
+        return out, [e.name for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA]
+
+    first, kernels_first = traced_call()
+    copies = [idx[i]._s3d_int32[1] for i in (1, 3, 4)]
+    assert all(c.dtype == torch.int32 for c in copies)
+    second, kernels_second = traced_call()
+    assert torch.equal(first, second)
+    assert [idx[i]._s3d_int32[1].data_ptr() for i in (1, 3, 4)] == [c.data_ptr() for c in copies]
+    # the second call is the sweep kernel and nothing else: the plan and the int32 copies are on the tensors
+    # (where the profiler records no device activity at all, the addresses above are the check)
+    if kernels_first:
+        assert any("attn_fwd_sweep_kernel" in k for k in kernels_second)
+        assert len(kernels_second) == 1, kernels_second
+        assert len(kernels_first) > len(kernels_second)
+    from gpu_helpers import assert_attn_close
+    assert_attn_close(second.double().cpu().numpy(), oracle_lib.attn_fwd(*case.oracle_args()), torch.float32)
+    # an in-place edit bumps the version counter: a new copy (and a new plan), same result for the same values
+    idx[4].add_(0)
+    third = s3d.SelfAttnAIOFunction.apply(*args)
+    assert idx[4]._s3d_int32[1].data_ptr() != copies[2].data_ptr() or idx[4]._s3d_int32[0][0] != 0
+    assert torch.equal(third, first)
 
 
 def test_headline_size_properties(oracle_lib, hip_lib):
@@ -567,13 +565,13 @@ def test_planned_forward_reuses_one_work_list(oracle_lib, hip_lib):
     def call(flags, workspace, out):
         status = hip_lib.s3d_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
                                       c_sizes, len(sizes), tq.numel(), w_sizes.data_ptr(), w2n.data_ptr(), n2n.data_ptr(),
-                                      n_coords.data_ptr(), out.data_ptr(), None, None, n, h, d, w, 0, 0, _lib.S3D_DTYPE_F16,
+                                      n_coords.data_ptr(), out.data_ptr(), None, None, n, h, d, w, 0, _lib.S3D_DTYPE_F16,
                                       flags, workspace.data_ptr(), workspace.numel(), stream)
         _lib.check(status, "s3d_attn_fwd")
 
-    ws = torch.empty(hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), h, d, n, w, 0), dtype=torch.uint8, device=dev)
+    ws = torch.empty(hip_lib.s3d_attn_fwd_workspace_bytes(h, n, w), dtype=torch.uint8, device=dev)
     ref = torch.empty_like(q)
-    call(_lib.S3D_ATTN_FORCE_GENERIC, ws, ref)
+    call(0, ws, ref)
     plan = torch.empty(hip_lib.s3d_attn_plan_bytes(h, n, w), dtype=torch.uint8, device=dev)
     _lib.check(hip_lib.s3d_attn_plan(c_sizes, len(sizes), tq.numel(), w_sizes.data_ptr(), w2n.data_ptr(), n, h, d, w,
                                      _lib.S3D_DTYPE_F16, plan.data_ptr(), plan.numel(), stream), "s3d_attn_plan")

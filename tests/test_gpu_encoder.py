@@ -25,26 +25,27 @@ def _small_model(fp16_mode):
     return encoder.Swin3DEncoder(**cfg, in_channels=9, cRSE="XYZ_RGB_NORM", fp16_mode=fp16_mode).cuda().eval()
 
 
-def test_encoder_forward_fp16_runs_on_both_kernels(hip_lib):
+def test_encoder_forward_fp16(hip_lib):
+    """fp16 inference; the blocks of a stage share one work list per window set (kept on the index tensors), and a
+    pass in which every attention call builds its own list gives the same bits."""
     vox, signals = _inputs()
     model = _small_model(fp16_mode=2)
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
         outs = model(vox, signals)
-        attn_coff.FORCE_GENERIC = True
+        attn_coff.REUSE_PLANS = False
         try:
-            outs_generic = model(vox, signals)
+            outs_own_lists = model(vox, signals)
         finally:
-            attn_coff.FORCE_GENERIC = False
+            attn_coff.REUSE_PLANS = True
     torch.cuda.synchronize()
     assert [o.feats.shape[1] for o in outs] == [48, 96, 192]
     assert [o.stride for o in outs] == [1, 2, 4]
     assert outs[0].coords.shape[0] == vox.coords.shape[0]
     assert outs[1].coords.shape[0] < outs[0].coords.shape[0] and outs[2].coords.shape[0] < outs[1].coords.shape[0]
-    for a, b in zip(outs, outs_generic):
+    for a, b in zip(outs, outs_own_lists):
         assert torch.isfinite(a.feats).all()
         assert torch.equal(a.coords, b.coords)
-        # two different kernels, fp16 attention inside: agreement to fp16 resolution of O(1) features
-        assert (a.feats - b.feats).abs().max().item() < 2e-2 * max(1.0, b.feats.abs().max().item())
+        assert torch.equal(a.feats, b.feats)
     # batches stay contiguous and ascending at every level, coordinates sit on the level's lattice
     for o in outs:
         bcol = o.coords[:, 0]
@@ -74,6 +75,13 @@ def test_window_ordered_levels_equal_input_ordered_levels(hip_lib):
         assert torch.equal(index.n2n.long(), torch.arange(a.coords.shape[0], device="cuda")), level
         assert not torch.equal(build_window_index(b.coords, b.stride, ordered.layers[level].window_size, 0).n2n.long(),
                                torch.arange(b.coords.shape[0], device="cuda"))
+    # the regular blocks of such levels get no row map at all (the kernels then read the rows in place); the
+    # shifted blocks keep theirs
+    _, _, _, _, plans = encoder.plan_stages_window_ordered(vox, signals, ordered.layers)
+    for level, (args, _) in enumerate(plans):
+        assert args[0][5] is None and args[1][5] is not None, level
+    _, plans = encoder.plan_stages(vox.coords, vox.stride, signals, plain.layers)
+    assert all(a[5] is not None for args, _ in plans for a in args)
     unet_o, unet_p = _small_unet(fp16_mode=2), _small_unet(fp16_mode=2)
     unet_o.eval(), unet_p.eval()
     unet_o.window_ordered, unet_p.window_ordered = True, False
@@ -81,6 +89,26 @@ def test_window_ordered_levels_equal_input_ordered_levels(hip_lib):
         lo, lp = unet_o(vox, signals), unet_p(vox, signals)
     assert lo.shape == lp.shape
     assert float((lo - lp).abs().max()) < 2e-3 * max(1.0, float(lp.abs().max()))
+
+
+def test_window_ordered_levels_train_like_input_ordered_levels(hip_lib):
+    """fp32 forward and backward (the attention backward gets no row map for the regular blocks either): logits and
+    parameter gradients of the window-ordered network equal those of the input-ordered one to fp32 rounding."""
+    vox, signals = _inputs(target=4000, batches=2)
+    nets = _small_unet(fp16_mode=0), _small_unet(fp16_mode=0)       # same seed: same weights
+    nets[0].window_ordered, nets[1].window_ordered = True, False
+    labels = (vox.coords[:, 3] // 8 % 13).long()
+    logits = []
+    for net in nets:
+        out = net(vox, signals)
+        torch.nn.functional.cross_entropy(out, labels).backward()
+        logits.append(out.detach())
+    assert float((logits[0] - logits[1]).abs().max()) < 1e-4 * max(1.0, float(logits[1].abs().max()))
+    for name in ("layers.0.blocks.0.attn.query_xyz_table", "layers.0.blocks.0.attn.value_norm_table",
+                 "layers.1.blocks.0.attn.qkv.weight", "layers.2.blocks.0.attn.key_rgb_table", "stem_layer.conv_layers.0.kernel"):
+        ga, gb = (dict(net.named_parameters())[name].grad for net in nets)
+        assert ga is not None and float(gb.abs().max()) > 0, name
+        assert float((ga - gb).abs().max()) < 1e-3 * float(gb.abs().max()), name
 
 
 def test_knn_downsample_matches_oracle_neighbours(oracle_lib, hip_lib):
@@ -240,3 +268,29 @@ def test_cell_representatives_on_the_gpu_match_the_host_statement(hip_lib):
     ref_coarse, ref_pick = encoder.pool_and_pick(coords, 2, 2, signals)
     got_coarse, got_pick = encoder.pool_and_pick(coords.cuda(), 2, 2, signals.cuda())
     assert torch.equal(got_coarse.cpu(), ref_coarse) and torch.equal(got_pick.cpu(), ref_pick)
+
+
+def test_inference_copies_of_parameters_follow_training_updates(hip_lib):
+    """The autocast-dtype copies that the layers keep for inference are renewed after any forward with autograd
+    enabled, also when the update went through `param.data` (which leaves the version counter alone), and on
+    request (drop_inference_copies)."""
+    torch.manual_seed(3)
+    layer = torch.nn.Linear(16, 8).cuda()
+    x = torch.randn(5, 16, device="cuda")
+
+    def infer():
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+            return encoder._linear(layer, x).float()
+
+    first = infer()
+    assert torch.equal(infer(), first) and hasattr(layer, "_s3d_cast")
+    layer.weight.data.mul_(2.0)                 # version counter unchanged
+    layer.bias.data.zero_()
+    encoder._linear(layer, x).sum().backward()  # a training forward in between
+    second = infer()
+    expect = torch.nn.functional.linear(x.half(), layer.weight.half(), layer.bias.half()).float()
+    assert torch.equal(second, expect) and not torch.equal(second, first)
+    layer.weight.data.mul_(0.5)                 # no training forward: the copy is stale until it is dropped
+    encoder.drop_inference_copies(layer)
+    third = infer()
+    assert torch.equal(third, torch.nn.functional.linear(x.half(), layer.weight.half(), layer.bias.half()).float())

@@ -91,8 +91,8 @@ def _knn_scene():
 @pytest.mark.parametrize("direction", ["down", "up"])
 def test_headline_sizes(oracle_lib, hip_lib, direction):
     """Config 4: 200k sources / 50k cell-centre queries, K=16, and the reverse with K=3.
-    Whole output: ordering and self-consistency properties; a random 2000-query sample is
-    compared bit for bit with the brute-force oracle."""
+    Whole output: every row is compared bit for bit with the brute-force oracle (10^10 candidate distances, about a
+    second on the host threads), on top of the ordering and self-consistency properties."""
     fine, centres = _knn_scene()
     src, qry, k = (fine, centres, 16) if direction == "down" else (centres, fine, 3)
     one = lambda n: np.array([n], np.int32)
@@ -105,10 +105,9 @@ def test_headline_sizes(oracle_lib, hip_lib, direction):
     recomputed = ((d[..., 0] * d[..., 0]).astype(np.float32) + (d[..., 1] * d[..., 1]).astype(np.float32)).astype(np.float32)
     recomputed = (recomputed + (d[..., 2] * d[..., 2]).astype(np.float32)).astype(np.float32)
     np.testing.assert_array_equal(d2, recomputed)
-    pick = np.sort(np.random.default_rng(0).choice(qry.shape[0], 2000, replace=False))
-    ridx, rd2 = oracle_lib.knn(k, src, qry[pick], one(src.shape[0]), one(2000))
-    np.testing.assert_array_equal(idx[pick], ridx)
-    np.testing.assert_array_equal(d2[pick], rd2)
+    ridx, rd2 = oracle_lib.knn(k, src, qry, one(src.shape[0]), one(qry.shape[0]))
+    np.testing.assert_array_equal(idx, ridx)
+    np.testing.assert_array_equal(d2, rd2)
 
 
 @pytest.mark.parametrize("half", [False, True])

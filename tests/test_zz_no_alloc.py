@@ -43,17 +43,24 @@ def _call_both(hip_lib, case, x, dtype):
                 x["n2n"].data_ptr(), x["n_coords"].data_ptr(), out.data_ptr(), omax.data_ptr(), osum.data_ptr(),
                 n, h, d, w]
         if which == "workspace":
-            ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, len(sizes), h, d, n, w, 0)
+            ws_bytes = hip_lib.s3d_attn_fwd_workspace_bytes(h, n, w)
             workspace = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
-            status = hip_lib.s3d_attn_fwd(*head, 0, 0, code, _lib.S3D_ATTN_FORCE_GENERIC, workspace.data_ptr(),
-                                          ws_bytes, stream)
+            status = hip_lib.s3d_attn_fwd(*head, 0, code, 0, workspace.data_ptr(), ws_bytes, stream)
             _lib.check(status, "s3d_attn_fwd")
         else:
+            # one call first: the code object, the scratch array's address and the kernel's LDS limit are set up
+            # by the first call on a device (and of a shape); the measured call comes after it
+            _lib.check(hip_lib.s3d_attn_fwd_noalloc(*head, 0, code, stream), "s3d_attn_fwd_noalloc")
             torch.cuda.synchronize()
-            before = torch.cuda.memory_allocated()
+            out.fill_(float("nan")), omax.fill_(float("nan")), osum.fill_(float("nan"))
+            torch.cuda.synchronize()
+            before = torch.cuda.memory_allocated()          # torch's caching allocator
+            free_before = torch.cuda.mem_get_info()[0]      # the device's free bytes (hipMemGetInfo): sees any hipMalloc
             status = hip_lib.s3d_attn_fwd_noalloc(*head, 0, code, stream)
             _lib.check(status, "s3d_attn_fwd_noalloc")
+            torch.cuda.synchronize()
             assert torch.cuda.memory_allocated() == before
+            assert torch.cuda.mem_get_info()[0] == free_before
         torch.cuda.synchronize()
         outs.append((out, omax, osum))
     return outs
@@ -79,7 +86,7 @@ def test_noalloc_forward_rejects_inputs_beyond_its_scratch(hip_lib):
     n = w = 1 << 30
     sizes = [40 * 48] * 3
     c_sizes = (ctypes.c_int32 * 3)(*sizes)
-    assert hip_lib.s3d_attn_fwd_workspace_bytes(c_sizes, 3, 6, 8, n, w, 0) > (1 << 34)
+    assert hip_lib.s3d_attn_fwd_workspace_bytes(6, n, w) > (1 << 34)
     one = torch.zeros(16, dtype=torch.float16, device="cuda")
     p = one.data_ptr()
     status = hip_lib.s3d_attn_fwd_noalloc(p, p, p, p, p, p, c_sizes, 3, sum(sizes), p, p, p, p, p, None, None,
