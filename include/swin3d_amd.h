@@ -175,7 +175,8 @@ int s3d_attn_fwd_noalloc(const void *q, const void *k, const void *v, const void
  * Swin3D/sparse_dl/attn/attn_coff.py:219-224) for pos_mode SEPARATE and indice_mode INDIRECT,
  * without the O(M) pair arrays.  Arithmetic is fp32 for both dtypes.
  *
- *   q .. n_coords  as for s3d_attn_fwd (the forward's inputs)
+ *   q .. n_coords  as for s3d_attn_fwd (the forward's inputs; with n2n NULL - rows in window order - the call
+ *                  writes the identity map into its workspace and reads that)
  *   out, out_max, out_sum   the forward's outputs for the same inputs (out of `dtype`, statistics fp32):
  *                  the tensors the reference saves for backward (attn_coff.py:186-187)
  *   dout           device [N,H,D] of `dtype`: gradient of the loss w.r.t. `out`

@@ -1278,6 +1278,14 @@ size_t bwd_tgrad_bytes(int H, int D, int nd)
 size_t bwd_pos_base_bytes(int64_t N) { return align_up(sizeof(int64_t) * static_cast<size_t>(N > 0 ? N : 1), 256); }
 size_t bwd_pd_bytes(int H, int64_t pairs) { return align_up(sizeof(float2) * static_cast<size_t>(H) * pairs, 256); }
 size_t bwd_dlt_bytes(int H, int64_t pairs) { return align_up(sizeof(float) * static_cast<size_t>(H) * pairs, 256); }
+// the last part of every form's workspace: the identity row map that stands in for a null n2n
+size_t bwd_row_map_bytes(int64_t N) { return align_up(sizeof(int32_t) * static_cast<size_t>(N > 0 ? N : 1), 256); }
+
+__global__ void bwd_identity_rows_kernel(int32_t *map, int64_t n)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) map[i] = static_cast<int32_t>(i);
+}
 
 }  // namespace
 }  // namespace s3d
@@ -1290,8 +1298,10 @@ extern "C" __attribute__((visibility("default"))) size_t s3d_attn_bwd_workspace_
     using namespace s3d;
     if (H < 1 || D < 1 || nd < 1 || nd > kMaxAxes || table_len < 1 || N < 0 || W < 0 || pairs < 0) return 0;
     if (bwd_general_form(H, D, nd, table_len))
-        return bwd_units_bytes(W, N, H, 0) + bwd_delta_bytes(N, H) + 2 * bwd_general_acc_bytes(N, H, D);
-    size_t need = bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) + bwd_pos_base_bytes(N);
+        return bwd_units_bytes(W, N, H, 0) + bwd_delta_bytes(N, H) + 2 * bwd_general_acc_bytes(N, H, D) +
+               bwd_row_map_bytes(N);
+    size_t need = bwd_units_bytes(W, N, H, pairs) + bwd_delta_bytes(N, H) + bwd_tgrad_bytes(H, D, nd) +
+                  bwd_pos_base_bytes(N) + bwd_row_map_bytes(N);
     if (pairs > 0)
         need += bwd_pd_bytes(H, pairs) + bwd_dlt_bytes(H, pairs) + align_up(attn_sweep_workspace_bytes(H, W, N), 256);
     return need;
@@ -1336,9 +1346,17 @@ extern "C" __attribute__((visibility("default"))) int s3d_attn_bwd(
         return fail(S3D_ERR_WORKSPACE, "s3d_attn_bwd: workspace %zu B < required %zu B",
                     workspace ? workspace_bytes : size_t(0), need);
     if (N > 0 && W > 0 &&
-        (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n2n || !n_coords || !out ||
+        (!q || !k || !v || !table_q || !table_k || !table_v || !w_sizes || !w2n || !n_coords || !out ||
          !out_max || !out_sum || !dout || !dq || !dk || !dv))
         return fail(S3D_ERR_NULL_POINTER, "s3d_attn_bwd: null device pointer");
+    if (!n2n && N > 0 && W > 0) {
+        // rows in window order: the kernels read the identity map from the end of the workspace
+        int32_t *map = reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + need - bwd_row_map_bytes(N));
+        hipLaunchKernelGGL(bwd_identity_rows_kernel, dim3(static_cast<unsigned>((N + 255) / 256)), dim3(256), 0,
+                           static_cast<hipStream_t>(stream), map, N);
+        S3D_HIP_CHECK(hipGetLastError());
+        n2n = map;
+    }
     a.q = q; a.k = k; a.v = v;
     a.table_q = table_q; a.table_k = table_k; a.table_v = table_v;
     a.dout = dout; a.out = out; a.out_max = out_max; a.out_sum = out_sum;

@@ -330,8 +330,9 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
             raise ValueError(f"{name} must be float32 [{n},{h}]")
     w_sizes = _as_int32("w_sizes", w_sizes, dev)
     w2n = _as_int32("w2n_indices", w2n, dev)
-    # rows in window-sorted order already (the forward took no row map): the backward's kernels read one
-    n2n = torch.arange(n, dtype=torch.int32, device=dev) if n2n is None else _as_int32("n2n_indices", n2n, dev)
+    # None: rows in window-sorted order already (the forward took no row map); the library then reads the identity
+    # map that it writes into its workspace
+    n2n = None if n2n is None else _as_int32("n2n_indices", n2n, dev)
     _require_cuda("n_coords", n_coords, dev)
     if n_coords.dtype != torch.float32 or n_coords.shape != (n, nd):
         raise ValueError(f"n_coords must be float32 [{n},{nd}]")
@@ -359,8 +360,8 @@ def window_attention_backward(q, k, v, table_q, table_k, table_v, table_sizes, w
         stream = torch.cuda.current_stream(dev).cuda_stream
         status = lib.s3d_attn_bwd(
             *(t.data_ptr() for t in tensors), c_sizes, nd, table_len, w_sizes.data_ptr(), w2n.data_ptr(),
-            n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(), out_max.data_ptr(), out_sum.data_ptr(),
-            dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dtq.data_ptr(), dtk.data_ptr(),
+            None if n2n is None else n2n.data_ptr(), n_coords.data_ptr(), out.data_ptr(), out_max.data_ptr(),
+            out_sum.data_ptr(), dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dtq.data_ptr(), dtk.data_ptr(),
             dtv.data_ptr(), n, h, d, w_sizes.numel(), pairs, code, workspace.data_ptr(), ws_bytes,
             stream)
     _lib.check(status, "s3d_attn_bwd")

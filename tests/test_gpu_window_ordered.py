@@ -133,3 +133,55 @@ def test_rows_in_window_order_need_no_row_map(oracle_lib, hip_lib, dtype, heads,
         assert np.abs(omax.double().cpu().numpy() - rmax).max() <= stat_tol * max(1.0, np.abs(rmax).max()), how
         assert np.abs(osum.double().cpu().numpy() / rsum - 1.0).max() <= 5 * stat_tol, how
         assert torch.equal(out, mapped[0]) and torch.equal(omax, mapped[1]) and torch.equal(osum, mapped[2]), how
+
+
+BWD_SHAPES = [(torch.float16, 6, 8, 5, "XYZ_RGB_NORM", None), (torch.float32, 4, 8, 5, "XYZ_RGB", None),
+              (torch.float16, 4, 16, 7, "XYZ_RGB_NORM", None), (torch.float32, 3, 16, 7, "XYZ", 0),
+              (torch.float16, 6, 8, 5, "XYZ_RGB_NORM", 0), (torch.float32, 2, 32, 5, "XYZ", None)]
+
+
+@pytest.mark.parametrize("dtype,heads,dim,ws,cRSE,pairs", BWD_SHAPES)
+def test_backward_on_rows_in_window_order(oracle_lib, hip_lib, dtype, heads, dim, ws, cRSE, pairs):
+    """s3d_attn_bwd with a NULL row map (the library reads the identity map that it writes into its workspace): all
+    six gradients against the float64 oracle, dq / dk / dv bit for bit those of the call with the row map on rows in
+    voxel order.  pairs None: the pair sweeps and their store; 0: the fused sweeps; head_dim 32: the general form."""
+    import swin3d_amd
+    case = _case(oracle_lib, 900 + heads * dim + ws, heads, dim, ws, cRSE, dtype == torch.float16)
+    rng = np.random.default_rng(5)
+    dout = rng.standard_normal(case.q.shape).astype(np.float32)
+    if dtype == torch.float16:
+        dout = dout.astype(np.float16).astype(np.float32)
+    ref = [np.asarray(r, np.float64) for r in oracle_lib.attn_bwd(*case.oracle_args(), dout)]
+    dev = torch.device("cuda")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    i = case.index
+    n2n = t(i["n2n"]).long()
+    tabs = [t(a).to(dtype) for a in (case.tq, case.tk, case.tv)]
+    tail = (t(case.table_sizes), t(i["w_sizes"]), t(i["w2n"]))
+    n_coords = t(case.n_coords)
+    rows = [t(a).to(dtype) for a in (case.q, case.k, case.v)]
+    d_out = t(dout).to(dtype)
+
+    def grads(feats, row_map, dout_rows):
+        args = (*feats, *tabs, *tail, row_map, n_coords)
+        out, omax, osum = swin3d_amd.window_attention_forward(*args, return_stats=True)
+        return swin3d_amd.window_attention_backward(*args, out, omax, osum, dout_rows, pairs=pairs)
+
+    mapped = grads(rows, n2n.int(), d_out)
+    ordered = grads([r[n2n].contiguous() for r in rows], None, d_out[n2n].contiguous())
+    torch.cuda.synchronize()
+    rel = 2e-5 if dtype == torch.float32 else 3e-3
+    scale_rows = max(np.abs(r).max() for r in ref[:3])
+    scale_tabs = max(np.abs(r).max() for r in ref[3:])
+    for which, (g_sorted, g_mapped, r) in enumerate(zip(ordered, mapped, ref)):
+        if which < 3:
+            g = torch.empty_like(g_sorted)
+            g[n2n] = g_sorted                                        # back to voxel order
+            if dim != 32:        # the general form adds dk, dv with atomics: not the same bits from call to call
+                assert torch.equal(g, g_mapped), which
+            scale = scale_rows
+        else:
+            g, scale = g_sorted, scale_tabs
+        got = g.double().cpu().numpy().reshape(r.shape)
+        assert np.isfinite(got).all(), which
+        assert np.abs(got - r).max() <= rel * scale, (which, np.abs(got - r).max(), scale)
