@@ -410,8 +410,11 @@ def other_shapes(torch, swin3d_amd, synth, crse, scene, dev):
         o, mx, sm = swin3d_amd.window_attention_forward(*a, return_stats=True)
         dout = torch.randn_like(o)
         bwd = _time_gpu(torch, lambda: swin3d_amd.window_attention_backward(*a, o, mx, sm, dout), reps=3, warm=1)
+        nbytes = algorithmic_bytes(n, heads * dim, 2, len(sizes), int(w_sizes.numel()), int(sum(sizes)))
         out[f"H{heads}_D{dim}_window7"] = {"fwd_ms": fwd, "bwd_ms": bwd,
-                                          "fwd_ps_per_pair_head": fwd * 1e9 / (pairs * heads)}
+                                          "fwd_ps_per_pair_head": fwd * 1e9 / (pairs * heads),
+                                          "fwd_algorithmic_bytes": nbytes,
+                                          "fwd_hbm_frac": nbytes / (fwd * 1e-3) / 1e9 / HBM_PEAK_GBPS}
     return out
 
 
